@@ -1,0 +1,343 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2|C3|C1|C4|C5] [--no-cpu] [--no-extra]
+
+A step is one attention call through the C ABI on synthetic, seeded inputs that are resident in
+HBM before the timed region.  The default workload is C2 (Llama-3-8B-shaped decode, batch 16, 4096
+f16 KV tokens per sequence): `value` is its KV-streaming rate in GB/s (algorithmic bytes per call /
+time per call, combine pass included).  The same JSON line also carries the C3 prefill figure
+(TFLOP/s, MFMA roofline) under "prefill", the HBM/MFMA roofline of the dominant kernel measured
+with HIP events on the launch stream, and the CPU checker timed on the host cores ("cpu_baseline").
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "attn prefill TFLOP/s + decode KV GB/s, % of roofline, 1xMI355X"
+PEAK_HBM_GBS = 8000.0
+PEAK_MFMA_F16_TFLOPS = 2500.0
+PEAK_MFMA_F32_TFLOPS = 157.3
+SEED = 0xF10E0000
+
+
+def configs():
+    # name -> description of the synthetic workload (BASELINE.json `configs`, in order)
+    return {
+        "C1": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True),
+        "C2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
+        "C3": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=8192, Skv=8192, D=128, dtype="f16", std=1.0, causal=True),
+        # reference-faithful sliding-window continuation: K/V are the last 4096 cached positions and the
+        # mask is get_mask(512, 16384, Some(4096)) = 3584 visible columns + a causal 512x512 block
+        "C4": dict(kind="prefill", B=4, H=32, Hkv=8, Sq=512, Skv=4096, D=128, dtype="f16", std=1.0, causal=True,
+                   q_pos_offset=3584, window=4096),
+        "C5": dict(kind="decode", B=32, H=32, Hkv=32, Sq=1, Skv=32768, D=96, dtype="f16", std=1.0, causal=False,
+                   ragged=(128, 32768)),
+    }
+
+
+def visible_pairs(c, lens=None):
+    """Number of (query, key) pairs per (batch, head) that the mask leaves visible, summed over batch."""
+    if lens is not None:
+        return int(np.sum(lens)) * c["Sq"]
+    if not c["causal"]:
+        return c["B"] * c["Sq"] * c["Skv"]
+    off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
+    w = c.get("window", 0)
+    i = np.arange(c["Sq"], dtype=np.int64) + off
+    hi = np.minimum(i + 1, c["Skv"])
+    lo = np.maximum(i - w + 1, 0) if w else np.zeros_like(i)
+    return c["B"] * int(np.sum(np.maximum(hi - lo, 0)))
+
+
+def algorithmic(c, lens=None):
+    """FLOPs = 4 D x visible pairs x heads; bytes = |Q| + |K| + |V| + |O| with K/V once per KV head."""
+    eb = 4 if c["dtype"] == "f32" else 2
+    pairs = visible_pairs(c, lens)
+    flops = 4 * c["D"] * pairs * c["H"]
+    kv_rows = int(np.sum(lens)) if lens is not None else c["B"] * c["Skv"]
+    byts = eb * (2 * c["B"] * c["H"] * c["Sq"] * c["D"] + 2 * kv_rows * c["Hkv"] * c["D"])
+    return flops, byts
+
+
+class Event:
+    def __init__(self, fa, dev):
+        self.fa, self.h = fa, ctypes.c_void_p()
+        fa.check(fa.lib().fhip_event_create(dev.handle, ctypes.byref(self.h)))
+
+    def record(self, dev):
+        self.fa.check(self.fa.lib().fhip_event_record(self.h, dev.stream))
+
+    def sync(self):
+        self.fa.check(self.fa.lib().fhip_event_synchronize(self.h))
+
+    def ms_since(self, start):
+        ms = ctypes.c_float()
+        self.fa.check(self.fa.lib().fhip_event_elapsed_ms(start.h, self.h, ctypes.byref(ms)))
+        return ms.value
+
+
+def _big_normal(synth, seed, tid, shape, std, npdt, max_batches=2):
+    """Normals for shape [B, ...]: the first `max_batches` batch entries are generated, the rest
+    repeat them with alternating sign (timing needs distinct memory, not distinct statistics)."""
+    B = shape[0]
+    if B <= max_batches:
+        return synth.normal(seed, tid, shape, std, npdt)
+    base = synth.normal(seed, tid, (max_batches,) + tuple(shape[1:]), std, npdt)
+    out = np.empty(shape, npdt)
+    for b in range(B):
+        out[b] = base[b % max_batches] if (b // max_batches) % 2 == 0 else -base[b % max_batches]
+    return out
+
+
+def make_inputs(fa, synth, dev, c, cfg_id, n_sets):
+    """n_sets rotating (Q, K, V) sets so a decode step never finds its KV in the 256 MB Infinity
+    Cache.  Set 0 is the seeded workload (and the one spot-checked); sets 1.. are rolled, sign-flipped
+    copies of it, which cost no generator time."""
+    dt = {"f32": fa.F32, "f16": fa.F16}[c["dtype"]]
+    npdt = np.float32 if dt == fa.F32 else np.float16
+    seed = SEED + cfg_id
+    big = c["B"] * c["Hkv"] * c["Skv"] * c["D"] > (1 << 28)
+    gen = (lambda tid, shp: _big_normal(synth, seed, tid, shp, c["std"], npdt)) if big else \
+          (lambda tid, shp: synth.normal(seed, tid, shp, c["std"], npdt))
+    q = gen(0, (c["B"], c["H"], c["Sq"], c["D"]))
+    k = gen(1, (c["B"], c["Hkv"], c["Skv"], c["D"]))
+    v = gen(2, (c["B"], c["Hkv"], c["Skv"], c["D"]))
+    sets = []
+    for s in range(n_sets):
+        if s == 0:
+            arrs = (q, k, v)
+        else:
+            sg = npdt(-1.0 if s % 2 else 1.0)
+            arrs = (q * sg, np.roll(k, s, axis=2) * sg, np.roll(v, s, axis=2))
+        sets.append(tuple(fa.Tensor.from_numpy(dev, a, dt) for a in arrs))
+    return dt, sets, (q, k, v)
+
+
+def prepare(fa, dev, c, sets, lens_t):
+    """Argument blocks (one per input set) with output and workspace bound once, outside the timed region."""
+    L = fa.lib()
+    blocks = []
+    for (q, k, v) in sets:
+        analytic = None
+        if c["causal"]:
+            analytic = (True, c.get("q_pos_offset", c["Skv"] - c["Sq"]), c.get("window", 0))
+        args = q._attn_args(k, v, c["D"] ** -0.5, None, analytic, lens_t, None, fa.KERNEL_AUTO, None)
+        need = ctypes.c_size_t()
+        fa.check(L.fhip_flash_attention_workspace_bytes(ctypes.byref(args), dev.compute_units, ctypes.byref(need)))
+        if need.value:
+            ws = fa.Buffer(dev, need.value)
+            args.workspace, args.workspace_bytes = ws.ptr, need.value
+            args._keep.append(ws)
+        blocks.append(args)
+    kid = ctypes.c_int32()
+    fa.check(L.fhip_flash_attention_select(ctypes.byref(blocks[0]), dev.compute_units, ctypes.byref(kid)))
+    return blocks, fa.KERNEL_NAMES[kid.value]
+
+
+def time_config(fa, dev, c, blocks, steps, warmup):
+    """Wall-clock over exactly `steps` calls (sync on both sides), then a second instrumented pass
+    of `steps` calls with HIP events around the main kernel of every call."""
+    L = fa.lib()
+    n = len(blocks)
+    for i in range(warmup):
+        fa.check(L.fhip_flash_attention(dev.stream, ctypes.byref(blocks[i % n])))
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fa.check(L.fhip_flash_attention(dev.stream, ctypes.byref(blocks[i % n])))
+    dev.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    starts = [Event(fa, dev) for _ in range(steps)]
+    mids = [Event(fa, dev) for _ in range(steps)]
+    ends = [Event(fa, dev) for _ in range(steps)]
+    for i in range(steps):
+        a = blocks[i % n]
+        a.main_kernel_done = mids[i].h
+        starts[i].record(dev)
+        fa.check(L.fhip_flash_attention(dev.stream, ctypes.byref(a)))
+        ends[i].record(dev)
+        a.main_kernel_done = None
+    dev.synchronize()
+    main_ms = np.array([mids[i].ms_since(starts[i]) for i in range(steps)])
+    call_ms = np.array([ends[i].ms_since(starts[i]) for i in range(steps)])
+    for e in starts + mids + ends:
+        L.fhip_event_destroy(e.h)
+    return wall_ms, float(main_ms.mean()), float(np.median(main_ms)), float(call_ms.mean())
+
+
+def parity_spot_check(fa, oracle, c, out_t, host, lens):
+    """A few output rows of the timed workload against the CPU checker (cheap: rows are independent)."""
+    q, k, v = host
+    f32 = lambda a: np.asarray(a, np.float32)  # noqa: E731  (slices are widened, never the whole cache)
+    out = np.asarray(out_t.to_numpy(), np.float32)
+    if c["kind"] == "decode":
+        bs = [0, c["B"] - 1]
+        worst = 0.0
+        for b in bs:
+            n = int(lens[b]) if lens is not None else c["Skv"]
+            ref = oracle.flash_attention(f32(q[b:b + 1]), f32(k[b:b + 1, :, :n]), f32(v[b:b + 1, :, :n]),
+                                         c["D"] ** -0.5)
+            worst = max(worst, float(np.abs(out[b:b + 1] - ref).max()))
+        return worst
+    q, k, v = f32(q), f32(k), f32(v)
+    rows = np.unique(np.linspace(0, c["Sq"] - 1, 16).astype(np.int32))
+    off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
+    mask = None
+    if c["causal"]:
+        i = rows[:, None].astype(np.int64) + off
+        j = np.arange(c["Skv"])[None, :]
+        masked = j > i
+        if c.get("window", 0):
+            masked |= (j + c["window"]) <= i
+        mask = np.where(masked, -np.inf, 0.0).astype(np.float32)
+    # the checker takes a [Sq, Skv] mask: evaluate the selected rows as their own Sq
+    ref = oracle.flash_attention(q[:, :, rows], k, v, c["D"] ** -0.5, mask, "qk" if mask is not None else None)
+    return float(np.abs(out[:, :, rows] - ref).max())
+
+
+def cpu_baseline(oracle, c, host, lens, flops, byts):
+    """The CPU checker (a C port of fusor's CPU composite) on the host cores, bounded to ~10-30 s."""
+    q, k, v = host
+    f32 = lambda a: np.asarray(a, np.float32)  # noqa: E731
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    scale = c["D"] ** -0.5
+    if c["kind"] == "decode":
+        if lens is not None:
+            # ragged: one un-padded call per sequence on a subset of sequences (upcast outside the clock,
+            # as kalosm-llama keeps its cache in f32)
+            pick = list(range(min(4, c["B"])))
+            dt = 0.0
+            for b in pick:
+                n = int(lens[b])
+                qb, kb, vb = f32(q[b:b + 1]), f32(k[b:b + 1, :, :n]), f32(v[b:b + 1, :, :n])
+                t0 = time.perf_counter()
+                oracle.flash_attention(qb, kb, vb, scale)
+                dt += time.perf_counter() - t0
+            frac = float(np.sum(lens[pick])) / float(np.sum(lens))
+            sample = f"sequences {pick} of the batch, un-padded, f16 upcast to f32, 1 pass"
+            return dict(value=byts * frac / dt / 1e9, unit="GB/s", cores=threads, kind="port", sample=sample)
+        reps = 3
+        q, k, v = f32(q), f32(k), f32(v)
+        oracle.flash_attention(q, k, v, scale)
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            oracle.flash_attention(q, k, v, scale)
+        dt = (time.perf_counter() - t0) / reps
+        return dict(value=byts / dt / 1e9, unit="GB/s", cores=threads, kind="port",
+                    sample=f"the full step (all {c['B']} sequences), f16 upcast to f32 first, mean of {reps} passes")
+    # prefill: a subset of query rows of every head (rows are independent in the reference algorithm)
+    q, k, v = f32(q), f32(k), f32(v)
+    target_flops = 4e11
+    stride = max(1, int(np.ceil(flops / target_flops)))
+    rows = np.arange(stride - 1, c["Sq"], stride, dtype=np.int32)
+    off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
+    i = rows[:, None].astype(np.int64) + off
+    j = np.arange(c["Skv"])[None, :]
+    masked = j > i if c["causal"] else np.zeros((len(rows), c["Skv"]), bool)
+    if c.get("window", 0):
+        masked |= (j + c["window"]) <= i
+    mask = np.where(masked, -np.inf, 0.0).astype(np.float32)
+    t0 = time.perf_counter()
+    oracle.flash_attention(q[:, :, rows], k, v, scale, mask, "qk")
+    dt = time.perf_counter() - t0
+    # the CPU path has no tile skipping: it computes every (row, key) pair and masks afterwards, but
+    # it is credited, like the GPU, with the visible pairs only
+    sample_flops = 4 * c["D"] * c["H"] * c["B"] * int((~masked).sum())
+    return dict(value=sample_flops / dt / 1e12, unit="TFLOP/s", cores=threads, kind="port",
+                sample=f"every {stride}th query row of every head ({len(rows)} of {c['Sq']} rows), dense "
+                       f"[rows, Skv] scores then mask, as the reference does")
+
+
+def run_config(name, steps, warmup, with_cpu=True):
+    import floneum_amd as fa
+    from floneum_amd import synth
+    import oracle
+
+    c = configs()[name]
+    cfg_id = int(name[1])
+    dev = fa.Device.default()
+    lens = lens_t = None
+    if "ragged" in c:
+        lens = synth.integers(SEED + cfg_id, 7, c["B"], *c["ragged"]).astype(np.int32)
+        lens_t = fa.IntTensor(dev, lens)
+    flops, byts = algorithmic(c, lens)
+    # decode streams the KV cache from HBM: rotate enough distinct sets to exceed the 256 MB MALL
+    kv_bytes = byts
+    n_sets = 1 if c["kind"] == "prefill" else max(2, min(8, int(np.ceil(1.2e9 / max(kv_bytes, 1)))))
+    if name == "C5":
+        n_sets = 1  # 6.5 GB per step already dwarfs the cache; one padded set is 13 GB of HBM
+    dt, sets, host = make_inputs(fa, synth, dev, c, cfg_id, n_sets)
+    blocks, kernel = prepare(fa, dev, c, sets, lens_t)
+    wall_ms, main_ms_mean, main_ms_med, call_ms = time_config(fa, dev, c, blocks, steps, warmup)
+    err = parity_spot_check(fa, oracle, c, blocks[0]._out_tensor, host, lens)
+
+    if c["kind"] == "decode":
+        value, unit = byts / (wall_ms * 1e-3) / 1e9, "GB/s"
+        roof = dict(bound="hbm", achieved=byts / (main_ms_mean * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
+    else:
+        peak = PEAK_MFMA_F32_TFLOPS if c["dtype"] == "f32" else PEAK_MFMA_F16_TFLOPS
+        value, unit = flops / (wall_ms * 1e-3) / 1e12, "TFLOP/s"
+        roof = dict(bound="mfma", achieved=flops / (main_ms_mean * 1e-3) / 1e12, peak=peak, unit="TFLOP/s")
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = kernel
+    roof["kernel_ms_mean"] = main_ms_mean
+    roof["kernel_ms_median"] = main_ms_med
+    roof["call_ms_events"] = call_ms
+    res = dict(value=value, unit=unit, ms_per_step=wall_ms, roofline=roof,
+               config=dict(workload=name, kind=c["kind"], batch=c["B"], q_heads=c["H"], kv_heads=c["Hkv"],
+                           q_len=c["Sq"], kv_len=c["Skv"], head_dim=c["D"], causal=c["causal"],
+                           q_pos_offset=c.get("q_pos_offset"), window=c.get("window"),
+                           ragged_lens=c.get("ragged"), kv_sets_rotated=n_sets,
+                           algorithmic_flops=flops, algorithmic_bytes=byts),
+               dtype=c["dtype"], frac_of_roofline=value / roof["peak"], spot_check_max_abs_err=err)
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline(oracle, c, host, lens, flops, byts)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="C2", choices=sorted(configs()))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary (prefill C3) figure")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this build runs on exactly one GPU (no sharding, no collectives); --gpus {a.gpus} is "
+              "not supported", file=sys.stderr)
+        sys.exit(2)
+
+    main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
+    line = {"metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (seeded SplitMix64 normals)",
+            "config": main_res["config"], "roofline": main_res["roofline"],
+            "frac_of_roofline": main_res["frac_of_roofline"],
+            "spot_check_max_abs_err": main_res["spot_check_max_abs_err"]}
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = main_res["cpu_baseline"]
+    if not a.no_extra and a.config == "C2":
+        # the other half of the metric: C3 prefill on the matrix cores
+        pre = run_config("C3", max(5, a.steps // 5), max(2, a.warmup // 5), with_cpu=not a.no_cpu)
+        line["prefill"] = {k: pre[k] for k in ("value", "unit", "ms_per_step", "roofline", "config", "dtype",
+                                               "frac_of_roofline", "spot_check_max_abs_err") if k in pre}
+        if "cpu_baseline" in pre:
+            line["prefill"]["cpu_baseline"] = pre["cpu_baseline"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,909 @@
+// C-ABI layer: handles, argument validation, kernel selection and dispatch, host mask builders,
+// device KV cache.  Everything here is host code; kernels live in the attn_*.hip files.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+#include "common.h"
+
+struct fhip_device {
+    int ordinal;
+    hipDeviceProp_t prop;
+};
+struct fhip_stream {
+    fhip_device *dev;
+    hipStream_t s;
+};
+struct fhip_event {
+    fhip_device *dev;
+    hipEvent_t e;
+};
+
+namespace fhip {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+    return FHIP_ERR_HIP;
+}
+
+static int elem_bytes(fhip_dtype d) { return d == FHIP_F32 ? 4 : 2; }
+
+static bool dtype_ok(int d) { return d == FHIP_F32 || d == FHIP_F16 || d == FHIP_BF16; }
+
+// ---- validation (host only) -------------------------------------------------------------------
+
+static int validate(const fhip_attn_args *a) {
+    if (!a) {
+        set_error("args is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!dtype_ok(a->dtype) || !dtype_ok(a->out_dtype)) {
+        set_error("unknown dtype %d / out_dtype %d", (int)a->dtype, (int)a->out_dtype);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (a->out_dtype != a->dtype && !(a->out_dtype == FHIP_F32 && a->dtype != FHIP_F32)) {
+        set_error("out_dtype must equal dtype, or be f32 for 16-bit inputs");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const uint32_t *qs = a->q.shape, *ks = a->k.shape, *vs = a->v.shape, *os = a->out.shape;
+    for (int i = 0; i < 4; i++) {
+        if (qs[i] == 0 || ks[i] == 0 || vs[i] == 0) {
+            set_error("empty tensors are not supported (q %u,%u,%u,%u k %u,%u,%u,%u)", qs[0], qs[1], qs[2],
+                      qs[3], ks[0], ks[1], ks[2], ks[3]);
+            return FHIP_ERR_INVALID_ARG;
+        }
+        if (qs[i] > 0x7fffffffu || ks[i] > 0x7fffffffu) {
+            set_error("dimension larger than 2^31-1");
+            return FHIP_ERR_INVALID_ARG;
+        }
+    }
+    const uint32_t B = qs[0], H = qs[1], Sq = qs[2], D = qs[3];
+    const uint32_t Hkv = ks[1], Skv = ks[2];
+    // reference: assert!(num_heads.is_multiple_of(num_kv_heads), ...) flash_attention.rs:94-99
+    if (H % Hkv != 0) {
+        set_error("Number of Q heads (%u) must be divisible by number of K/V heads (%u)", H, Hkv);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (ks[0] != B || ks[3] != D) {
+        set_error("K shape [%u, %u, %u, %u] does not match Q shape [%u, %u, %u, %u] in batch/head_dim", ks[0],
+                  ks[1], ks[2], ks[3], B, H, Sq, D);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (int i = 0; i < 4; i++)
+        if (vs[i] != ks[i]) {
+            set_error("V shape [%u, %u, %u, %u] does not match K shape [%u, %u, %u, %u]", vs[0], vs[1], vs[2],
+                      vs[3], ks[0], ks[1], ks[2], ks[3]);
+            return FHIP_ERR_INVALID_ARG;
+        }
+    for (int i = 0; i < 4; i++)
+        if (os[i] != qs[i]) {
+            set_error("output shape [%u, %u, %u, %u] does not match Q shape [%u, %u, %u, %u]", os[0], os[1],
+                      os[2], os[3], B, H, Sq, D);
+            return FHIP_ERR_INVALID_ARG;
+        }
+    if (!a->q.ptr || !a->k.ptr || !a->v.ptr || !a->out.ptr) {
+        set_error("q, k, v and out need device pointers");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (int i = 0; i < 4; i++)
+        if (os[i] > 1 && a->out.stride[i] == 0) {
+            set_error("output stride %d is 0 (overlapping writes)", i);
+            return FHIP_ERR_INVALID_ARG;
+        }
+    if (!std::isfinite(a->scale)) {
+        set_error("scale must be finite");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    switch (a->mask_kind) {
+        case FHIP_MASK_NONE:
+            if (a->mask.ptr) {
+                set_error("mask pointer given with FHIP_MASK_NONE");
+                return FHIP_ERR_INVALID_ARG;
+            }
+            break;
+        case FHIP_MASK_QK:
+            // reference: assert_eq!(m_shape, [q_seq_len, kv_seq_len], ...) flash_attention.rs:153-160
+            if (a->mask.shape[0] != Sq || a->mask.shape[1] != Skv) {
+                set_error("QKMask shape [%u, %u] does not match expected [%u, %u]", a->mask.shape[0],
+                          a->mask.shape[1], Sq, Skv);
+                return FHIP_ERR_INVALID_ARG;
+            }
+            break;
+        case FHIP_MASK_BATCH_KEY:
+            // reference: flash_attention.rs:165-172
+            if (a->mask.shape[0] != B || a->mask.shape[1] != Skv) {
+                set_error("BatchKeyMask shape [%u, %u] does not match expected [%u, %u]", a->mask.shape[0],
+                          a->mask.shape[1], B, Skv);
+                return FHIP_ERR_INVALID_ARG;
+            }
+            break;
+        default:
+            set_error("unknown mask_kind %d", (int)a->mask_kind);
+            return FHIP_ERR_INVALID_ARG;
+    }
+    if (a->mask_kind != FHIP_MASK_NONE && !a->mask.ptr) {
+        set_error("mask_kind set but mask pointer is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (a->analytic.enabled) {
+        if (a->mask_kind != FHIP_MASK_NONE) {
+            set_error("analytic mask and mask tensor are mutually exclusive");
+            return FHIP_ERR_INVALID_ARG;
+        }
+        if (a->analytic.window < 0 || a->analytic.q_pos_offset < 0) {
+            set_error("analytic mask: window and q_pos_offset must be >= 0");
+            return FHIP_ERR_INVALID_ARG;
+        }
+    }
+    if (D > 512) {
+        set_error("head_dim %u > 512 has no kernel", D);
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    return FHIP_OK;
+}
+
+static bool aligned16(const void *p, uint64_t off_elems, int eb) {
+    return (((uintptr_t)p + off_elems * (uint64_t)eb) & 15u) == 0;
+}
+
+static bool rows_vectorizable(const fhip_tensor4 &t, int eb) {
+    const int per16 = 16 / eb;
+    if (t.shape[3] > 1 && t.stride[3] != 1) return false;
+    if (!aligned16(t.ptr, t.offset, eb)) return false;
+    for (int i = 0; i < 3; i++)
+        if (t.shape[i] > 1 && (t.stride[i] % per16) != 0) return false;
+    return true;
+}
+
+static bool decode_eligible(const fhip_attn_args *a) {
+    if (a->dtype == FHIP_F32) return false;
+    const uint32_t D = a->q.shape[3];
+    if (a->q.shape[2] != 1) return false;
+    if (D % 8 != 0 || D < 8 || D > 128) return false;
+    if (!rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
+    if (a->k.stride[2] < 0 || a->v.stride[2] < 0) return false;
+    return true;
+}
+
+static bool prefill_mfma_eligible(const fhip_attn_args *a) {
+    if (a->dtype == FHIP_F32) return false;
+    const uint32_t D = a->q.shape[3];
+    if (!(D == 64 || D == 96 || D == 128)) return false;
+    if (!(a->scale > 0.0f)) return false;
+    if (a->mask_kind != FHIP_MASK_NONE) return false;  // dense additive masks take the generic kernel
+    if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
+    return true;
+}
+
+static bool prefill_f32_eligible(const fhip_attn_args *a) {
+    if (a->dtype != FHIP_F32) return false;
+    const uint32_t D = a->q.shape[3];
+    if (!(D == 32 || D == 64 || D == 96 || D == 128)) return false;
+    if (!(a->scale > 0.0f)) return false;
+    if (a->mask_kind != FHIP_MASK_NONE) return false;
+    if (!rows_vectorizable(a->q, 4) || !rows_vectorizable(a->k, 4) || !rows_vectorizable(a->v, 4)) return false;
+    return true;
+}
+
+static int select_kernel(const fhip_attn_args *a, int32_t *id) {
+    const int f = a->force_kernel;
+    if (f != FHIP_KERNEL_AUTO) {
+        bool ok = false;
+        switch (f) {
+            case FHIP_KERNEL_GENERIC: ok = true; break;
+            case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a); break;
+            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a); break;
+            case FHIP_KERNEL_DECODE_SPLITKV: ok = decode_eligible(a); break;
+            default: set_error("unknown force_kernel %d", f); return FHIP_ERR_INVALID_ARG;
+        }
+        if (!ok) {
+            set_error("force_kernel %d cannot run these arguments (dtype/head_dim/stride/mask constraints)", f);
+            return FHIP_ERR_UNSUPPORTED;
+        }
+        *id = f;
+        return FHIP_OK;
+    }
+    if (decode_eligible(a))
+        *id = FHIP_KERNEL_DECODE_SPLITKV;
+    else if (prefill_mfma_eligible(a))
+        *id = FHIP_KERNEL_PREFILL_MFMA;
+    else if (prefill_f32_eligible(a))
+        *id = FHIP_KERNEL_PREFILL_F32;
+    else
+        *id = FHIP_KERNEL_GENERIC;
+    return FHIP_OK;
+}
+
+static void fill_params(const fhip_attn_args *a, AttnParams *p) {
+    const int eb = elem_bytes(a->dtype);
+    const int ob = elem_bytes(a->out_dtype);
+    memset(p, 0, sizeof(*p));
+    p->q = (const char *)a->q.ptr + a->q.offset * eb;
+    p->k = (const char *)a->k.ptr + a->k.offset * eb;
+    p->v = (const char *)a->v.ptr + a->v.offset * eb;
+    p->out = (char *)a->out.ptr + a->out.offset * ob;
+    for (int i = 0; i < 4; i++) {
+        p->qs[i] = a->q.stride[i];
+        p->ks[i] = a->k.stride[i];
+        p->vs[i] = a->v.stride[i];
+        p->os[i] = a->out.stride[i];
+    }
+    p->B = (int)a->q.shape[0];
+    p->H = (int)a->q.shape[1];
+    p->Sq = (int)a->q.shape[2];
+    p->D = (int)a->q.shape[3];
+    p->Hkv = (int)a->k.shape[1];
+    p->Skv = (int)a->k.shape[2];
+    p->G = p->H / p->Hkv;
+    p->mask_kind = a->mask_kind;
+    if (a->mask_kind != FHIP_MASK_NONE) {
+        p->mask = (const char *)a->mask.ptr + a->mask.offset * eb;
+        p->ms0 = a->mask.stride[0];
+        p->ms1 = a->mask.stride[1];
+    }
+    p->analytic = a->analytic.enabled ? 1 : 0;
+    p->causal = a->analytic.enabled ? (a->analytic.causal ? 1 : 0) : 0;
+    p->q_pos_offset = a->analytic.q_pos_offset;
+    p->window = a->analytic.enabled ? a->analytic.window : 0;
+    p->kv_lens = a->kv_lens;
+    p->scale = a->scale;
+    p->out_f32 = (a->out_dtype == FHIP_F32 && a->dtype != FHIP_F32) ? 1 : 0;
+    p->workspace = a->workspace;
+}
+
+}  // namespace fhip
+
+using namespace fhip;
+
+extern "C" {
+
+const char *fhip_last_error(void) { return g_err; }
+
+const char *fhip_version(void) { return "fusor-hip 0.1 (gfx950)"; }
+
+int fhip_device_count(int32_t *count) {
+    if (!count) {
+        set_error("count is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        return hip_fail(e, "hipGetDeviceCount");
+    }
+    *count = n;
+    return FHIP_OK;
+}
+
+int fhip_device_create(int32_t ordinal, fhip_device **out) {
+    if (!out) {
+        set_error("out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *out = nullptr;
+    int n = 0;
+    FHIP_HIP_CHECK(hipGetDeviceCount(&n));
+    if (ordinal < 0 || ordinal >= n) {
+        set_error("device ordinal %d out of range (%d devices)", ordinal, n);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    fhip_device *d = new (std::nothrow) fhip_device();
+    if (!d) {
+        set_error("out of host memory");
+        return FHIP_ERR_HIP;
+    }
+    d->ordinal = ordinal;
+    hipError_t e = hipGetDeviceProperties(&d->prop, ordinal);
+    if (e != hipSuccess) {
+        delete d;
+        return hip_fail(e, "hipGetDeviceProperties");
+    }
+    if (strncmp(d->prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library carries gfx950 code only", ordinal, d->prop.gcnArchName);
+        delete d;
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    *out = d;
+    return FHIP_OK;
+}
+
+int fhip_device_destroy(fhip_device *dev) {
+    delete dev;
+    return FHIP_OK;
+}
+
+int fhip_device_get_info(fhip_device *dev, fhip_device_info *info) {
+    if (!dev || !info) {
+        set_error("dev/info is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    memset(info, 0, sizeof(*info));
+    snprintf(info->name, sizeof(info->name), "%s", dev->prop.name);
+    snprintf(info->arch, sizeof(info->arch), "%s", dev->prop.gcnArchName);
+    info->compute_units = dev->prop.multiProcessorCount;
+    info->wavefront_size = dev->prop.warpSize;
+    info->clock_khz = dev->prop.clockRate;
+    info->memory_clock_khz = dev->prop.memoryClockRate;
+    info->memory_bus_bits = dev->prop.memoryBusWidth;
+    info->total_memory = dev->prop.totalGlobalMem;
+    info->lds_per_cu = dev->prop.maxSharedMemoryPerMultiProcessor;
+    info->l2_bytes = (uint64_t)dev->prop.l2CacheSize;
+    return FHIP_OK;
+}
+
+int fhip_stream_create(fhip_device *dev, fhip_stream **out) {
+    if (!dev || !out) {
+        set_error("dev/out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *out = nullptr;
+    FHIP_HIP_CHECK(hipSetDevice(dev->ordinal));
+    hipStream_t s;
+    FHIP_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    fhip_stream *st = new (std::nothrow) fhip_stream();
+    if (!st) {
+        (void)hipStreamDestroy(s);
+        set_error("out of host memory");
+        return FHIP_ERR_HIP;
+    }
+    st->dev = dev;
+    st->s = s;
+    *out = st;
+    return FHIP_OK;
+}
+
+int fhip_stream_destroy(fhip_stream *s) {
+    if (!s) return FHIP_OK;
+    hipError_t e = hipStreamDestroy(s->s);
+    delete s;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamDestroy");
+    return FHIP_OK;
+}
+
+int fhip_stream_synchronize(fhip_stream *s) {
+    if (!s) {
+        set_error("stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipStreamSynchronize(s->s));
+    return FHIP_OK;
+}
+
+int fhip_malloc(fhip_device *dev, size_t bytes, void **out) {
+    if (!dev || !out) {
+        set_error("dev/out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *out = nullptr;
+    FHIP_HIP_CHECK(hipSetDevice(dev->ordinal));
+    FHIP_HIP_CHECK(hipMalloc(out, bytes ? bytes : 1));
+    return FHIP_OK;
+}
+
+int fhip_free(fhip_device *dev, void *ptr) {
+    if (!dev) {
+        set_error("dev is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!ptr) return FHIP_OK;
+    FHIP_HIP_CHECK(hipSetDevice(dev->ordinal));
+    FHIP_HIP_CHECK(hipFree(ptr));
+    return FHIP_OK;
+}
+
+int fhip_memcpy_h2d(fhip_stream *s, void *dst, const void *src, size_t bytes) {
+    if (!s || (bytes && (!dst || !src))) {
+        set_error("memcpy_h2d: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!bytes) return FHIP_OK;
+    // pageable host memory: the copy is staged by the runtime, the host buffer is reusable on return
+    FHIP_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s->s));
+    FHIP_HIP_CHECK(hipStreamSynchronize(s->s));
+    return FHIP_OK;
+}
+
+int fhip_memcpy_d2h(fhip_stream *s, void *dst, const void *src, size_t bytes) {
+    if (!s || (bytes && (!dst || !src))) {
+        set_error("memcpy_d2h: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!bytes) return FHIP_OK;
+    FHIP_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s->s));
+    FHIP_HIP_CHECK(hipStreamSynchronize(s->s));
+    return FHIP_OK;
+}
+
+int fhip_memcpy_d2d(fhip_stream *s, void *dst, const void *src, size_t bytes) {
+    if (!s || (bytes && (!dst || !src))) {
+        set_error("memcpy_d2d: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!bytes) return FHIP_OK;
+    FHIP_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s->s));
+    return FHIP_OK;
+}
+
+int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes) {
+    if (!s || (bytes && !dst)) {
+        set_error("memset: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!bytes) return FHIP_OK;
+    FHIP_HIP_CHECK(hipMemsetAsync(dst, value, bytes, s->s));
+    return FHIP_OK;
+}
+
+int fhip_event_create(fhip_device *dev, fhip_event **out) {
+    if (!dev || !out) {
+        set_error("dev/out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *out = nullptr;
+    FHIP_HIP_CHECK(hipSetDevice(dev->ordinal));
+    hipEvent_t e;
+    FHIP_HIP_CHECK(hipEventCreate(&e));
+    fhip_event *ev = new (std::nothrow) fhip_event();
+    if (!ev) {
+        (void)hipEventDestroy(e);
+        set_error("out of host memory");
+        return FHIP_ERR_HIP;
+    }
+    ev->dev = dev;
+    ev->e = e;
+    *out = ev;
+    return FHIP_OK;
+}
+
+int fhip_event_destroy(fhip_event *e) {
+    if (!e) return FHIP_OK;
+    hipError_t r = hipEventDestroy(e->e);
+    delete e;
+    if (r != hipSuccess) return hip_fail(r, "hipEventDestroy");
+    return FHIP_OK;
+}
+
+int fhip_event_record(fhip_event *e, fhip_stream *s) {
+    if (!e || !s) {
+        set_error("event/stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipEventRecord(e->e, s->s));
+    return FHIP_OK;
+}
+
+int fhip_event_synchronize(fhip_event *e) {
+    if (!e) {
+        set_error("event is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipEventSynchronize(e->e));
+    return FHIP_OK;
+}
+
+int fhip_event_elapsed_ms(fhip_event *start, fhip_event *stop, float *ms) {
+    if (!start || !stop || !ms) {
+        set_error("event_elapsed_ms: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipEventElapsedTime(ms, start->e, stop->e));
+    return FHIP_OK;
+}
+
+// ---- attention ----------------------------------------------------------------------------------
+
+int fhip_flash_attention_validate(const fhip_attn_args *args) { return validate(args); }
+
+int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id) {
+    (void)compute_units;
+    if (!kernel_id) {
+        set_error("kernel_id is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    int rc = validate(args);
+    if (rc) return rc;
+    return select_kernel(args, kernel_id);
+}
+
+int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t compute_units, size_t *bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *bytes = 0;
+    int rc = validate(args);
+    if (rc) return rc;
+    int32_t id;
+    rc = select_kernel(args, &id);
+    if (rc) return rc;
+    if (id == FHIP_KERNEL_DECODE_SPLITKV) {
+        int chunk, nsplit;
+        const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
+        const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2];
+        decode_plan(B, Hkv, H / Hkv, Skv, D, compute_units > 0 ? compute_units : 256, &chunk, &nsplit);
+        *bytes = decode_workspace_bytes(B, H, D, nsplit);
+    }
+    return FHIP_OK;
+}
+
+int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
+    if (!s) {
+        set_error("stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    int rc = validate(args);
+    if (rc) return rc;
+    int32_t id;
+    rc = select_kernel(args, &id);
+    if (rc) return rc;
+    AttnParams p;
+    fill_params(args, &p);
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    switch (id) {
+        case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
+        case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
+        case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, s->s); break;
+        case FHIP_KERNEL_DECODE_SPLITKV: {
+            decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, &p.chunk, &p.nsplit);
+            const size_t need = decode_workspace_bytes(p.B, p.H, p.D, p.nsplit);
+            if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
+                set_error("decode needs a workspace of %zu bytes, got %zu", need,
+                          args->workspace ? args->workspace_bytes : (size_t)0);
+                return FHIP_ERR_WORKSPACE;
+            }
+            return launch_decode(p, args->dtype, s->s);  // records main_done itself, before the combine
+        }
+        default: set_error("internal: no kernel for id %d", id); return FHIP_ERR_UNSUPPORTED;
+    }
+    if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+    return rc;
+}
+
+// ---- masks (host, bit-exact) --------------------------------------------------------------------
+
+static inline void put_mask(void *out, fhip_dtype dt, uint64_t idx, bool masked) {
+    switch (dt) {
+        case FHIP_F32: ((uint32_t *)out)[idx] = masked ? 0xFF800000u : 0u; break;
+        case FHIP_F16: ((uint16_t *)out)[idx] = masked ? 0xFC00u : 0u; break;
+        case FHIP_BF16: ((uint16_t *)out)[idx] = masked ? 0xFF80u : 0u; break;
+    }
+}
+
+int fhip_mask_causal(fhip_dtype dtype, uint32_t n, void *out) {
+    if (!dtype_ok(dtype) || (n && !out)) {
+        set_error("mask_causal: bad dtype or NULL out");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (uint64_t i = 0; i < n; i++)
+        for (uint64_t j = 0; j < n; j++) put_mask(out, dtype, i * n + j, j > i);
+    return FHIP_OK;
+}
+
+int fhip_mask_sliding_window(fhip_dtype dtype, uint32_t n, uint64_t window, void *out) {
+    if (!dtype_ok(dtype) || (n && !out)) {
+        set_error("mask_sliding_window: bad dtype or NULL out");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (uint64_t i = 0; i < n; i++)
+        for (uint64_t j = 0; j < n; j++) put_mask(out, dtype, i * n + j, i < j || j + window <= i);
+    return FHIP_OK;
+}
+
+static uint64_t mask_offset(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window, uint64_t window) {
+    if (!has_window) return seqlen_offset;
+    const uint64_t room = window > seq_len ? window - seq_len : 0;  // saturating_sub
+    return seqlen_offset < room ? seqlen_offset : room;
+}
+
+int fhip_mask_get_mask_shape(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window, uint64_t window,
+                             uint32_t *rows, uint64_t *cols) {
+    if (!rows || !cols) {
+        set_error("rows/cols is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *rows = seq_len;
+    *cols = mask_offset(seq_len, seqlen_offset, has_window, window) + seq_len;
+    return FHIP_OK;
+}
+
+int fhip_mask_get_mask(fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
+                       uint64_t window, void *out) {
+    if (!dtype_ok(dtype) || (seq_len && !out)) {
+        set_error("mask_get_mask: bad dtype or NULL out");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const uint64_t off = mask_offset(seq_len, seqlen_offset, has_window, window);
+    const uint64_t cols = off + seq_len;
+    for (uint64_t i = 0; i < seq_len; i++) {
+        for (uint64_t j = 0; j < off; j++) put_mask(out, dtype, i * cols + j, false);
+        for (uint64_t j = 0; j < seq_len; j++) {
+            const bool masked = has_window ? (i < j || j + window <= i) : (j > i);
+            put_mask(out, dtype, i * cols + off + j, masked);
+        }
+    }
+    return FHIP_OK;
+}
+
+int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window, uint64_t window,
+                           fhip_analytic_mask *out) {
+    if (!out) {
+        set_error("out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (has_window && window == 0) {
+        // a window of 0 masks every key of every row; there is no analytic form with window>0
+        set_error("sliding window of 0 masks everything; build the dense mask instead");
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    out->enabled = 1;
+    out->causal = 1;
+    out->q_pos_offset = (int64_t)mask_offset(seq_len, seqlen_offset, has_window, window);
+    out->window = has_window ? (int64_t)window : 0;
+    return FHIP_OK;
+}
+
+}  // extern "C"
+
+// ---- growable KV cache on the device ---------------------------------------------------------------
+
+struct fhip_tensor_cache_side {
+    void *buf = nullptr;    // [B, Hkv, allocated, D] contiguous
+    void *spare = nullptr;  // second buffer of max_sequence_len rows, used once the cache is full
+};
+
+struct fhip_kv_cache {
+    fhip_device *dev;
+    fhip_dtype dtype;
+    uint64_t max_len;
+    uint32_t B, Hkv, D;  // fixed by the first append
+    uint64_t current, allocated;
+    fhip_tensor_cache_side side[2];  // 0 = keys, 1 = values
+};
+
+static void kv_contig_strides(const fhip_kv_cache *c, uint64_t alloc, int64_t st[4]) {
+    st[3] = 1;
+    st[2] = c->D;
+    st[1] = (int64_t)alloc * c->D;
+    st[0] = (int64_t)c->Hkv * st[1];
+}
+
+static void kv_view(const fhip_kv_cache *c, void *buf, uint64_t alloc, uint64_t len, fhip_tensor4 *t) {
+    t->ptr = buf;
+    t->offset = 0;
+    t->shape[0] = c->B;
+    t->shape[1] = c->Hkv;
+    t->shape[2] = (uint32_t)len;
+    t->shape[3] = c->D;
+    kv_contig_strides(c, alloc, t->stride);
+}
+
+static uint64_t next_pow2(uint64_t x) {
+    uint64_t p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+extern "C" {
+
+int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequence_len, fhip_kv_cache **out) {
+    if (!dev || !out || !fhip::dtype_ok(dtype)) {
+        set_error("kv_cache_create: NULL argument or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (max_sequence_len == 0 || max_sequence_len > 0x7fffffffull) {
+        set_error("kv_cache_create: max_sequence_len must be in 1..2^31-1");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    fhip_kv_cache *c = new (std::nothrow) fhip_kv_cache();
+    if (!c) {
+        set_error("out of host memory");
+        return FHIP_ERR_HIP;
+    }
+    c->dev = dev;
+    c->dtype = dtype;
+    c->max_len = max_sequence_len;
+    c->B = c->Hkv = c->D = 0;
+    c->current = c->allocated = 0;
+    *out = c;
+    return FHIP_OK;
+}
+
+static int kv_release(fhip_kv_cache *c) {
+    int rc = FHIP_OK;
+    if (hipSetDevice(c->dev->ordinal) != hipSuccess) rc = FHIP_ERR_HIP;
+    for (int s = 0; s < 2; s++) {
+        if (c->side[s].buf && hipFree(c->side[s].buf) != hipSuccess) rc = FHIP_ERR_HIP;
+        if (c->side[s].spare && hipFree(c->side[s].spare) != hipSuccess) rc = FHIP_ERR_HIP;
+        c->side[s].buf = c->side[s].spare = nullptr;
+    }
+    c->current = c->allocated = 0;
+    c->B = c->Hkv = c->D = 0;
+    if (rc) set_error("kv_cache: hipFree failed");
+    return rc;
+}
+
+int fhip_kv_cache_destroy(fhip_kv_cache *c) {
+    if (!c) return FHIP_OK;
+    int rc = kv_release(c);
+    delete c;
+    return rc;
+}
+
+// TensorCache::reset (tensor_cache.rs:39-43): drops the data, keeps the limits.
+int fhip_kv_cache_reset(fhip_kv_cache *c) {
+    if (!c) {
+        set_error("cache is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    return kv_release(c);
+}
+
+int fhip_kv_cache_current_seq_len(const fhip_kv_cache *c, uint64_t *len) {
+    if (!c || !len) {
+        set_error("cache/len is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *len = c->current;
+    return FHIP_OK;
+}
+
+int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len) {
+    if (!c || !len) {
+        set_error("cache/len is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *len = c->allocated;
+    return FHIP_OK;
+}
+
+int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
+                         fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    if (!c || !s || !k_new || !v_new || !k_all || !v_all) {
+        set_error("kv_cache_append: NULL argument");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (!k_new->ptr || !v_new->ptr) {
+        set_error("kv_cache_append: new keys/values need device pointers");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (int i = 0; i < 4; i++) {
+        if (k_new->shape[i] != v_new->shape[i]) {
+            set_error("kv_cache_append: key shape [%u, %u, %u, %u] != value shape [%u, %u, %u, %u]", k_new->shape[0],
+                      k_new->shape[1], k_new->shape[2], k_new->shape[3], v_new->shape[0], v_new->shape[1],
+                      v_new->shape[2], v_new->shape[3]);
+            return FHIP_ERR_INVALID_ARG;
+        }
+        if (k_new->shape[i] == 0) {
+            set_error("kv_cache_append: empty tensor");
+            return FHIP_ERR_INVALID_ARG;
+        }
+    }
+    const bool first = c->side[0].buf == nullptr;
+    if (!first && (k_new->shape[0] != c->B || k_new->shape[1] != c->Hkv || k_new->shape[3] != c->D)) {
+        set_error("kv_cache_append: [%u, %u, _, %u] does not match the cached [%u, %u, _, %u]", k_new->shape[0],
+                  k_new->shape[1], k_new->shape[3], c->B, c->Hkv, c->D);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(c->dev->ordinal));
+    const int eb = fhip::elem_bytes(c->dtype);
+    const uint64_t n = k_new->shape[2];
+    const uint64_t required = c->current + n;
+    if (first) {
+        c->B = k_new->shape[0];
+        c->Hkv = k_new->shape[1];
+        c->D = k_new->shape[3];
+    }
+    const size_t row_elems = (size_t)c->B * c->Hkv * c->D;
+    const fhip_tensor4 *news[2] = {k_new, v_new};
+    fhip_tensor4 *alls[2] = {k_all, v_all};
+
+    if (required > c->max_len) {
+        // keep the last max_len positions of old[new_start..] ++ new (tensor_cache.rs:55-78)
+        const uint64_t mx = c->max_len;
+        const uint64_t new_start = required - mx;
+        const uint64_t keep_old = c->current > new_start ? c->current - new_start : 0;  // rows kept from the cache
+        const uint64_t take_new = mx - keep_old;                                          // last rows of the new block
+        for (int sd = 0; sd < 2; sd++) {
+            fhip_tensor_cache_side &S = c->side[sd];
+            if (!S.spare) FHIP_HIP_CHECK(hipMalloc(&S.spare, row_elems * mx * eb));
+            int64_t dst_st[4];
+            kv_contig_strides(c, mx, dst_st);
+            if (keep_old) {
+                int64_t src_st[4];
+                kv_contig_strides(c, c->allocated, src_st);
+                const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
+                int rc = launch_copy_rows((const char *)S.buf + new_start * c->D * eb, src_st, S.spare, dst_st, shp,
+                                          eb, s->s);
+                if (rc) return rc;
+            }
+            const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)take_new, c->D};
+            const char *src = (const char *)news[sd]->ptr +
+                              (news[sd]->offset + (n - take_new) * news[sd]->stride[2]) * (uint64_t)eb;
+            int rc = launch_copy_rows(src, news[sd]->stride, (char *)S.spare + keep_old * c->D * eb, dst_st, shp, eb,
+                                      s->s);
+            if (rc) return rc;
+            if (S.buf && c->allocated != mx) {
+                // the growing buffer is retired; hipFree waits for the copies above
+                FHIP_HIP_CHECK(hipFree(S.buf));
+                S.buf = nullptr;
+            }
+            void *t = S.buf;
+            S.buf = S.spare;
+            S.spare = t;
+            kv_view(c, S.buf, mx, mx, alls[sd]);
+        }
+        c->current = mx;
+        c->allocated = mx;
+        return FHIP_OK;
+    }
+
+    if (first) {
+        // first append stores the tensor as it is (tensor_cache.rs:111-116)
+        for (int sd = 0; sd < 2; sd++) {
+            fhip_tensor_cache_side &S = c->side[sd];
+            FHIP_HIP_CHECK(hipMalloc(&S.buf, row_elems * n * eb));
+            int64_t dst_st[4];
+            kv_contig_strides(c, n, dst_st);
+            const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)n, c->D};
+            const char *src = (const char *)news[sd]->ptr + news[sd]->offset * (uint64_t)eb;
+            int rc = launch_copy_rows(src, news[sd]->stride, S.buf, dst_st, shp, eb, s->s);
+            if (rc) return rc;
+            kv_view(c, S.buf, n, n, alls[sd]);
+        }
+        c->current = n;
+        c->allocated = n;
+        return FHIP_OK;
+    }
+
+    uint64_t alloc = c->allocated;
+    if (required > c->allocated) alloc = next_pow2(required);  // tensor_cache.rs:80-96
+    for (int sd = 0; sd < 2; sd++) {
+        fhip_tensor_cache_side &S = c->side[sd];
+        int64_t dst_st[4];
+        kv_contig_strides(c, alloc, dst_st);
+        if (alloc != c->allocated) {
+            void *nb = nullptr;
+            FHIP_HIP_CHECK(hipMalloc(&nb, row_elems * alloc * eb));
+            int64_t src_st[4];
+            kv_contig_strides(c, c->allocated, src_st);
+            const uint32_t shp_old[4] = {c->B, c->Hkv, (uint32_t)c->current, c->D};
+            int rc = launch_copy_rows(S.buf, src_st, nb, dst_st, shp_old, eb, s->s);
+            if (rc) return rc;
+            if (alloc > required) {  // the reference concatenates zeros behind the data
+                const uint32_t shp_z[4] = {c->B, c->Hkv, (uint32_t)(alloc - required), c->D};
+                rc = launch_fill_zero_rows((char *)nb + required * c->D * eb, dst_st, shp_z, eb, s->s);
+                if (rc) return rc;
+            }
+            FHIP_HIP_CHECK(hipFree(S.buf));  // waits for the copy
+            S.buf = nb;
+            if (S.spare) {
+                FHIP_HIP_CHECK(hipFree(S.spare));
+                S.spare = nullptr;
+            }
+        }
+        const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)n, c->D};
+        const char *src = (const char *)news[sd]->ptr + news[sd]->offset * (uint64_t)eb;
+        int rc = launch_copy_rows(src, news[sd]->stride, (char *)S.buf + c->current * c->D * eb, dst_st, shp, eb, s->s);
+        if (rc) return rc;
+        kv_view(c, S.buf, alloc, required, alls[sd]);
+    }
+    c->current = required;
+    c->allocated = alloc;
+    return FHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,58 @@
+// Internal declarations shared by the C-ABI layer and the kernel launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fusor_hip.h"
+
+namespace fhip {
+
+// What every attention kernel receives: base pointers with the view offset already applied,
+// element strides, and the mask description reduced to what the device needs.
+struct AttnParams {
+    const void *q, *k, *v;
+    void *out;
+    const void *mask;       // nullptr when there is no additive mask tensor
+    const int32_t *kv_lens; // nullptr or [B]
+    int64_t qs[4], ks[4], vs[4], os[4];
+    int64_t ms0, ms1;       // mask strides: row (query for QK, batch for BATCH_KEY), key
+    int32_t B, H, Hkv, G, Sq, Skv, D;
+    int32_t mask_kind;      // fhip_mask_kind of `mask`
+    int32_t analytic, causal;
+    int64_t q_pos_offset, window;
+    float scale;
+    int32_t out_f32;        // 1: out is f32 although the inputs are 16-bit
+    // split-KV decode only
+    void *workspace;
+    int32_t chunk;          // keys per split
+    int32_t nsplit;         // splits per (batch, kv head) over Skv
+    hipEvent_t main_done;   // host-side only: recorded after the main kernel when not null
+};
+
+// thread-local error text
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define FHIP_HIP_CHECK(expr)                                  \
+    do {                                                      \
+        hipError_t e__ = (expr);                              \
+        if (e__ != hipSuccess) return fhip::hip_fail(e__, #expr); \
+    } while (0)
+
+// launchers (each returns a status code, all asynchronous on `stream`)
+int launch_generic(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
+int launch_decode(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
+int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
+int launch_prefill_f32(const AttnParams &p, hipStream_t stream);
+
+// decode planning (host): keys per split and number of splits
+void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, int *chunk, int *nsplit);
+size_t decode_workspace_bytes(int B, int H, int D, int nsplit);
+
+// KV cache copies
+int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
+                     const uint32_t shape[4], int elem_bytes, hipStream_t stream);
+int launch_fill_zero_rows(void *dst, const int64_t dstride[4], const uint32_t shape[4], int elem_bytes,
+                          hipStream_t stream);
+
+}  // namespace fhip

@@ -1,0 +1,232 @@
+/*
+ * fusor_hip.h -- C ABI of the MI355X (gfx950) attention backend for fusor-ml.
+ *
+ * This is the boundary a fusor HIP backend crate binds with `unsafe extern "C"`; it replaces the
+ * GPU arm of `fusor::Tensor<4,D>::flash_attention` (reference:
+ * fusor-ml/fusor/src/composite/flash_attention.rs:52-73), i.e. the WGSL custom op
+ * `fusor_core::Tensor::flash_attention` / `FlashAttentionOperation`
+ * (fusor-ml/core/src/composite/flash_attention.rs:28-99, 442-557).
+ *
+ * Conventions
+ *   - Plain pointers and sizes only.  Every function returns an `int` status (0 = FHIP_OK); the
+ *     text of the last failure on the calling thread is available from fhip_last_error().
+ *     Nothing throws or aborts across this boundary: the reference's `assert!` panics on shape
+ *     errors (flash_attention.rs:94-99,153-172) become FHIP_ERR_INVALID_ARG with the same message.
+ *   - Tensors are described the way fusor's kernels receive them: a device buffer plus
+ *     {offset, shape, strides} in ELEMENT units (fusor-ml/types/src/layout.rs:88-129,
+ *     fusor-ml/core/src/mir/inputs/tensor.rs:33-119).  Arbitrary strided views are accepted
+ *     (narrowed KV-cache views, transposed Q/V, broadcast strides of 0 on inputs).
+ *   - The library never allocates or frees caller tensors.  The output buffer and the workspace
+ *     are supplied by the caller.  Launches are asynchronous on the given stream.
+ *   - Re-entrant: no global mutable state besides per-device handles and the thread-local error
+ *     string.  One stream is used from one thread at a time.
+ */
+#ifndef FUSOR_HIP_H
+#define FUSOR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status ---------------------------------------------------------------------------------- */
+enum {
+    FHIP_OK = 0,
+    FHIP_ERR_INVALID_ARG = 1, /* what the reference panics on: shapes, divisibility, null pointers  */
+    FHIP_ERR_UNSUPPORTED = 2, /* valid request with no kernel (e.g. head_dim > 512)                */
+    FHIP_ERR_HIP = 3,         /* a HIP runtime call failed (reference: fusor::Error::Gpu,
+                                 fusor-ml/fusor/src/lib.rs:391-403)                                */
+    FHIP_ERR_WORKSPACE = 4    /* workspace missing or smaller than *_workspace_bytes reports       */
+};
+
+/* Message of the last non-zero status returned on this thread ("" if none).  Never NULL. */
+const char *fhip_last_error(void);
+
+typedef struct fhip_device fhip_device;
+typedef struct fhip_stream fhip_stream;
+typedef struct fhip_event fhip_event;
+
+/* ---- element types (reference: DataTypeEnum, fusor-ml/core/src/tensor.rs:110-134) ------------ */
+typedef enum { FHIP_F32 = 0, FHIP_F16 = 1, FHIP_BF16 = 2 } fhip_dtype;
+
+/* ---- mask layout (reference: enum MaskKind, fusor flash_attention.rs:11-19) ------------------ */
+typedef enum {
+    FHIP_MASK_NONE = 0,
+    FHIP_MASK_QK = 1,       /* [q_seq_len, kv_seq_len], shared by every (batch, head)            */
+    FHIP_MASK_BATCH_KEY = 2 /* [batch, kv_seq_len], broadcast over heads and queries             */
+} fhip_mask_kind;
+
+/* Rank-4 strided view [batch, heads, seq, head_dim].  Element (b,h,s,d) lives at
+ * ptr[offset + b*stride[0] + h*stride[1] + s*stride[2] + d*stride[3]]  (element units). */
+typedef struct {
+    void *ptr;
+    uint64_t offset;
+    uint32_t shape[4];
+    int64_t stride[4];
+} fhip_tensor4;
+
+/* Rank-2 strided view (the mask). */
+typedef struct {
+    void *ptr;
+    uint64_t offset;
+    uint32_t shape[2];
+    int64_t stride[2];
+} fhip_tensor2;
+
+/* Optional analytic description of the mask.  It NEVER replaces semantics: when `enabled`, the
+ * caller promises that the additive mask it would otherwise pass is exactly
+ *     mask[i][j] = -inf  if  j > i + q_pos_offset                      (causal part)
+ *                  -inf  if  window > 0 and j + window <= i + q_pos_offset   (sliding part)
+ *                  0     otherwise
+ * which is what MaskCache::get_mask builds (fusor-ml/fusor/src/cache/mask_cache.rs:36-116) with
+ * q_pos_offset = the left padding it computes.  The kernels then skip fully masked key tiles
+ * and never read a mask tensor.  `mask.ptr` must be NULL when this is enabled. */
+typedef struct {
+    int32_t enabled;
+    int32_t causal;       /* 0: no causal part (only the window, if any)                          */
+    int64_t q_pos_offset; /* key index the first query row may still see: kv_seq_len - q_seq_len
+                             for a chunk appended to a cache                                      */
+    int64_t window;       /* 0 = none                                                             */
+} fhip_analytic_mask;
+
+/* Arguments of one attention call.  Zero-initialise, then fill. */
+typedef struct {
+    fhip_tensor4 q;   /* [B, H,   Sq,  D] */
+    fhip_tensor4 k;   /* [B, Hkv, Skv, D] */
+    fhip_tensor4 v;   /* [B, Hkv, Skv, D] */
+    fhip_tensor4 out; /* [B, H,   Sq,  D]  fresh buffer of Q's shape (reference: core :505-507)  */
+    fhip_dtype dtype;     /* element type of q, k, v and the mask                                  */
+    fhip_dtype out_dtype; /* the reference returns Q's dtype; FHIP_F32 is also accepted for f16/bf16
+                             inputs (accumulators are f32 either way, core :186-203,323-327)       */
+    float scale;
+    fhip_mask_kind mask_kind;
+    fhip_tensor2 mask;
+    fhip_analytic_mask analytic;
+    /* Optional device array of B int32: keys j >= kv_lens[b] are masked for batch b.  Equivalent
+     * to a 0 / -inf BatchKeyMask; it exists so a ragged batch needs no [B,Skv] mask tensor. */
+    const int32_t *kv_lens;
+    void *workspace; /* device scratch, >= fhip_flash_attention_workspace_bytes(); may be NULL
+                        when that reports 0                                                         */
+    size_t workspace_bytes;
+    int32_t force_kernel; /* 0 = choose; otherwise a fhip_kernel_id (testing / benchmarking)       */
+    /* Optional profiling hook: when non-NULL the event is recorded on the stream right after the
+     * main kernel of the call (before the split-KV combine pass, if there is one), so a benchmark
+     * can time that kernel alone with HIP events. */
+    fhip_event *main_kernel_done;
+} fhip_attn_args;
+
+typedef enum {
+    FHIP_KERNEL_AUTO = 0,
+    FHIP_KERNEL_GENERIC = 1,     /* any dtype, any strides, any mask; one wavefront per query row   */
+    FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim in {64,96,128}, LDS-tiled MFMA               */
+    FHIP_KERNEL_PREFILL_F32 = 3, /* f32, head_dim multiple of 32 up to 128, f32 MFMA                */
+    FHIP_KERNEL_DECODE_SPLITKV = 4 /* f16/bf16, Sq == 1, split-KV streaming + LSE combine           */
+} fhip_kernel_id;
+
+
+typedef struct {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t clock_khz;
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    uint64_t total_memory;
+    uint64_t lds_per_cu;
+    uint64_t l2_bytes;
+} fhip_device_info;
+
+/* ---- device / stream / memory: the minimal backend a fusor HIP crate owns ---------------------
+ * Replaces what fusor_core::Device does for WGPU (fusor-ml/core/src/device.rs:89-354): pick an
+ * adapter, create buffers, upload (`Tensor::new`, core/src/tensor.rs) and read back
+ * (`as_slice`, core/src/tensor.rs:797-896). */
+int fhip_device_count(int32_t *count);
+int fhip_device_create(int32_t ordinal, fhip_device **out);
+int fhip_device_destroy(fhip_device *dev);
+int fhip_device_get_info(fhip_device *dev, fhip_device_info *info);
+
+int fhip_stream_create(fhip_device *dev, fhip_stream **out);
+int fhip_stream_destroy(fhip_stream *s);
+int fhip_stream_synchronize(fhip_stream *s);
+
+int fhip_malloc(fhip_device *dev, size_t bytes, void **out);
+int fhip_free(fhip_device *dev, void *ptr);
+int fhip_memcpy_h2d(fhip_stream *s, void *dst, const void *src, size_t bytes);
+int fhip_memcpy_d2h(fhip_stream *s, void *dst, const void *src, size_t bytes); /* synchronises */
+int fhip_memcpy_d2d(fhip_stream *s, void *dst, const void *src, size_t bytes);
+int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes);
+
+/* HIP events on a library stream (timing in benchmarks; the reference has no GPU timers). */
+int fhip_event_create(fhip_device *dev, fhip_event **out);
+int fhip_event_destroy(fhip_event *e);
+int fhip_event_record(fhip_event *e, fhip_stream *s);
+int fhip_event_synchronize(fhip_event *e);
+int fhip_event_elapsed_ms(fhip_event *start, fhip_event *stop, float *ms);
+
+/* ---- attention ------------------------------------------------------------------------------ */
+
+/* Host-only check of everything the reference asserts plus pointer/stride sanity.  Touches no
+ * GPU.  Same status and message fhip_flash_attention would return. */
+int fhip_flash_attention_validate(const fhip_attn_args *args);
+
+/* Which kernel fhip_flash_attention will run for these arguments (host-only). */
+int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id);
+
+/* Bytes of device workspace the call needs (0 for the single-pass kernels).  `compute_units`
+ * is fhip_device_info.compute_units (split count depends on it). */
+int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t compute_units, size_t *bytes);
+
+/* out = softmax(q k^T * scale + mask) v with GQA head mapping kv_head = head / (H / Hkv).
+ * Replaces fusor_core::Tensor::flash_attention (core/src/composite/flash_attention.rs:28-52) and,
+ * for FHIP_MASK_BATCH_KEY, the composite fallback fusor takes on GPU (fusor
+ * flash_attention.rs:61-72).  Asynchronous on `s`. */
+int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
+
+/* ---- masks: host builders, bit-exact with the reference ---------------------------------------
+ * `out` is host memory of the given dtype (f32: 0x00000000 / 0xFF800000; f16: 0x0000 / 0xFC00;
+ * bf16: 0x0000 / 0xFF80), row-major contiguous. */
+
+/* AttentionMask::causal (fusor-ml/fusor/src/cache/attention_mask.rs:26-46): [n, n]. */
+int fhip_mask_causal(fhip_dtype dtype, uint32_t seq_len, void *out);
+/* MaskCache::create_sliding_window_mask (fusor-ml/fusor/src/cache/mask_cache.rs:88-116): [n, n]. */
+int fhip_mask_sliding_window(fhip_dtype dtype, uint32_t seq_len, uint64_t window, void *out);
+/* MaskCache::get_mask (mask_cache.rs:36-86): shape [seq_len, offset' + seq_len] where
+ * offset' = has_window ? min(seqlen_offset, window.saturating_sub(seq_len)) : seqlen_offset. */
+int fhip_mask_get_mask_shape(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
+                             uint64_t window, uint32_t *rows, uint64_t *cols);
+int fhip_mask_get_mask(fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset,
+                       int32_t has_window, uint64_t window, void *out);
+/* The analytic descriptor equal to get_mask(seq_len, seqlen_offset, window) (no tensor built). */
+int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
+                           uint64_t window, fhip_analytic_mask *out);
+
+/* ---- growable KV cache on the device -----------------------------------------------------------
+ * Replaces fusor::cache::KvCache / TensorCache for rank-4 [B, Hkv, seq, D] tensors concatenated
+ * along dim 2 (fusor-ml/fusor/src/cache/kv_cache.rs:13-68, tensor_cache.rs:9-124; kalosm-llama
+ * uses concat dim 2, models/kalosm-llama/src/raw/cache.rs:7).  Same observable behaviour:
+ * first append stores the tensor, later appends grow the allocation to the next power of two and
+ * write the new rows in place, the returned view is the valid prefix (stride[1] = allocated *
+ * D), and once max_sequence_len would be exceeded only the last max_sequence_len positions are
+ * kept.  Unlike the reference, growth copies once and in-place appends copy only the new rows. */
+typedef struct fhip_kv_cache fhip_kv_cache;
+int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequence_len, fhip_kv_cache **out);
+int fhip_kv_cache_destroy(fhip_kv_cache *c);
+int fhip_kv_cache_reset(fhip_kv_cache *c);
+int fhip_kv_cache_current_seq_len(const fhip_kv_cache *c, uint64_t *len);
+int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len);
+/* k_new, v_new: [B, Hkv, n, D] strided device views of the cache dtype.  On return k_all/v_all
+ * describe the cached keys/values including the new rows (views into cache-owned memory, valid
+ * until the next append/reset/destroy). */
+int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new,
+                         const fhip_tensor4 *v_new, fhip_tensor4 *k_all, fhip_tensor4 *v_all);
+
+/* Library version string, e.g. "fusor-hip 0.1 (gfx950)". */
+const char *fhip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUSOR_HIP_H */

@@ -1,0 +1,284 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU checker.
+
+Structure follows the reference's own tests: the unit cases of
+fusor-ml/fusor/src/composite/flash_attention.rs:207-359 and the fuzz tests of
+fusor-ml/core/src/composite/flash_attention.rs:559-1060 (same shape ranges, seeded here), then the
+benchmark configurations at reduced and full size.
+"""
+import numpy as np
+import pytest
+
+import floneum_amd as fa
+import oracle
+from floneum_amd import synth
+from conftest import TOL_16, TOL_F32, assert_parity
+
+pytestmark = pytest.mark.gpu
+
+NEG_INF = float("-inf")
+
+
+def run(device, q, k, v, scale, mask=None, kind=None, dtype=fa.F32, **kw):
+    tq = fa.Tensor.from_numpy(device, q, dtype)
+    tk = fa.Tensor.from_numpy(device, k, dtype)
+    tv = fa.Tensor.from_numpy(device, v, dtype)
+    m = None
+    if mask is not None:
+        m = (fa.Tensor.from_numpy(device, mask, dtype), kind)
+    return tq.flash_attention(tk, tv, scale, m, **kw).to_numpy()
+
+
+def rounded(a, dtype):
+    """The values the device sees after the host rounds to the element type, as float32."""
+    if dtype == fa.F32:
+        return np.asarray(a, np.float32)
+    if dtype == fa.F16:
+        return np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
+    return fa.bf16_bits_to_f32(fa.f32_to_bf16_bits(a))
+
+
+KIND = {fa.MaskKind.QKMask: "qk", fa.MaskKind.BatchKeyMask: "batch_key"}
+
+
+def check(device, q, k, v, scale, mask=None, kind=None, dtype=fa.F32, what="", tol=None, **kw):
+    out = run(device, q, k, v, scale, mask, kind, dtype, **kw)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale,
+                                 None if mask is None else rounded(mask, dtype), KIND.get(kind))
+    tol = tol or (TOL_F32 if dtype == fa.F32 else TOL_16)
+    return assert_parity(out, ref, tol, what)
+
+
+# ---- the reference's unit cases ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("kernel", [fa.KERNEL_AUTO, fa.KERNEL_GENERIC])
+def test_flash_attention_2x2(device, kernel):
+    # fusor flash_attention.rs:207-239
+    q = np.array([1, 0, 0, 1], np.float32).reshape(1, 1, 2, 2)
+    k = q.copy()
+    v = np.array([1, 2, 3, 4], np.float32).reshape(1, 1, 2, 2)
+    out = run(device, q, k, v, 1 / np.sqrt(2), force_kernel=kernel)
+    assert out.shape == (1, 1, 2, 2) and np.isfinite(out).all()
+    check(device, q, k, v, 1 / np.sqrt(2), force_kernel=kernel)
+
+
+def test_flash_attention_causal_row0_is_v0(device):
+    # fusor flash_attention.rs:241-276, core flash_attention.rs:605-673
+    q = np.array([1, 0, 0, 1], np.float32).reshape(1, 1, 2, 2)
+    v = np.array([1, 2, 3, 4], np.float32).reshape(1, 1, 2, 2)
+    mask = np.array([[0, NEG_INF], [0, 0]], np.float32)
+    out = run(device, q, q, v, 1 / np.sqrt(2), mask, fa.MaskKind.QKMask)
+    assert abs(out[0, 0, 0, 0] - 1.0) < 0.01 and abs(out[0, 0, 0, 1] - 2.0) < 0.01
+    check(device, q, q, v, 1 / np.sqrt(2), mask, fa.MaskKind.QKMask)
+
+
+def test_flash_attention_gqa_ramp(device):
+    # fusor flash_attention.rs:278-313
+    q = (np.arange(16, dtype=np.float32) * 0.1).reshape(1, 4, 2, 2)
+    k = (np.arange(8, dtype=np.float32) * 0.1 + 1.0).reshape(1, 2, 2, 2)
+    v = (np.arange(8, dtype=np.float32) * 0.1 + 2.0).reshape(1, 2, 2, 2)
+    out = run(device, q, k, v, 1 / np.sqrt(2))
+    assert out.shape == (1, 4, 2, 2) and np.isfinite(out).all()
+    check(device, q, k, v, 1 / np.sqrt(2))
+
+
+def test_flash_attention_batch_key_mask(device):
+    # fusor flash_attention.rs:315-358
+    q = (np.arange(12, dtype=np.float32) * 0.1).reshape(2, 1, 3, 2)
+    k = (np.arange(12, dtype=np.float32) * 0.1 + 1.0).reshape(2, 1, 3, 2)
+    v = (np.arange(12, dtype=np.float32) * 0.1 + 2.0).reshape(2, 1, 3, 2)
+    mask = np.array([[0, 0, 0], [0, 0, NEG_INF]], np.float32)
+    out = run(device, q, k, v, 1 / np.sqrt(2), mask, fa.MaskKind.BatchKeyMask)
+    assert out.shape == (2, 1, 3, 2) and np.isfinite(out).all()
+    check(device, q, k, v, 1 / np.sqrt(2), mask, fa.MaskKind.BatchKeyMask)
+
+
+def test_head_divisibility_panics(device):
+    # fusor flash_attention.rs:94-99
+    q = np.zeros((1, 3, 2, 2), np.float32)
+    k = np.zeros((1, 2, 2, 2), np.float32)
+    with pytest.raises(AssertionError, match=r"Number of Q heads \(3\) must be divisible by number of K/V heads \(2\)"):
+        run(device, q, k, k, 1.0)
+
+
+def test_mask_shape_panics(device):
+    # fusor flash_attention.rs:153-172
+    q = np.zeros((2, 1, 3, 2), np.float32)
+    with pytest.raises(AssertionError, match=r"QKMask shape \[2, 3\] does not match expected \[3, 3\]"):
+        run(device, q, q, q, 1.0, np.zeros((2, 3), np.float32), fa.MaskKind.QKMask)
+    with pytest.raises(AssertionError, match=r"BatchKeyMask shape \[3, 3\] does not match expected \[2, 3\]"):
+        run(device, q, q, q, 1.0, np.zeros((3, 3), np.float32), fa.MaskKind.BatchKeyMask)
+
+
+# ---- the reference's fuzz tests, seeded ---------------------------------------------------------------
+
+def _uniform(rng, shape):
+    return (rng.random(shape, dtype=np.float32) * 2.0 - 1.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_masked_fuzz(device, dtype):
+    # core flash_attention.rs:675-805: B 1..2, H 1..16, S 1..128, D 1..64; -inf above the diagonal,
+    # random finite bias U(-0.25, 0.25) on and below it
+    rng = np.random.default_rng(0xF10E)
+    for it in range(40):
+        B, H, S, D = rng.integers(1, 3), rng.integers(1, 17), rng.integers(1, 129), rng.integers(1, 65)
+        q, k, v = (_uniform(rng, (B, H, S, D)) for _ in range(3))
+        bias = rng.random((S, S), dtype=np.float32) * 0.5 - 0.25
+        mask = np.where(np.arange(S)[None, :] > np.arange(S)[:, None], NEG_INF, bias).astype(np.float32)
+        check(device, q, k, v, 1 / np.sqrt(np.float32(D)), mask, fa.MaskKind.QKMask, dtype,
+              what=f"it{it} B{B} H{H} S{S} D{D}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_kv_cache_fuzz(device, dtype):
+    # core flash_attention.rs:807-921: Sq 1..4, Skv = Sq + 0..31, zero mask [Sq, Skv]
+    rng = np.random.default_rng(0xF10F)
+    for it in range(40):
+        B, H, D = rng.integers(1, 3), rng.integers(1, 9), rng.integers(1, 65)
+        Sq = rng.integers(1, 5)
+        Skv = Sq + rng.integers(0, 32)
+        q = _uniform(rng, (B, H, Sq, D))
+        k, v = _uniform(rng, (B, H, Skv, D)), _uniform(rng, (B, H, Skv, D))
+        mask = np.zeros((Sq, Skv), np.float32)
+        check(device, q, k, v, 1 / np.sqrt(np.float32(D)), mask, fa.MaskKind.QKMask, dtype,
+              what=f"it{it} B{B} H{H} Sq{Sq} Skv{Skv} D{D}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16, fa.BF16])
+def test_gqa_fuzz(device, dtype):
+    # core flash_attention.rs:923-1060: Hkv 1..4, G 1..4; reference there = K/V expanded by kv_h = h / G
+    rng = np.random.default_rng(0xF110)
+    tol = dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else None
+    for it in range(30):
+        B, Hkv, G = rng.integers(1, 3), rng.integers(1, 5), rng.integers(1, 5)
+        S, D = rng.integers(1, 65), rng.integers(1, 65)
+        q = _uniform(rng, (B, Hkv * G, S, D))
+        k, v = _uniform(rng, (B, Hkv, S, D)), _uniform(rng, (B, Hkv, S, D))
+        check(device, q, k, v, 1 / np.sqrt(np.float32(D)), None, None, dtype, tol=tol,
+              what=f"it{it} B{B} Hkv{Hkv} G{G} S{S} D{D}")
+        # bit-exact head mapping: expanding K/V on the host and calling with H == Hkv gives identical bits
+        if it < 6:
+            out_g = run(device, q, k, v, 0.25, dtype=dtype)
+            out_e = run(device, q, np.repeat(k, G, axis=1), np.repeat(v, G, axis=1), 0.25, dtype=dtype)
+            assert np.array_equal(out_g, out_e), "GQA head mapping differs from expand-then-MHA"
+
+
+# ---- tiled kernels against the checker on shapes that select them ---------------------------------------
+
+def _normal_qkv(seed, B, H, Hkv, Sq, Skv, D, scale=1.0):
+    q = synth.normal(seed, 0, (B, H, Sq, D), scale)
+    k = synth.normal(seed, 1, (B, Hkv, Skv, D), scale)
+    v = synth.normal(seed, 2, (B, Hkv, Skv, D), scale)
+    return q, k, v
+
+
+def _analytic_mask(Sq, Skv, causal, off, window):
+    i = np.arange(Sq)[:, None] + off
+    j = np.arange(Skv)[None, :]
+    masked = np.zeros((Sq, Skv), bool)
+    if causal:
+        masked |= j > i
+    if window:
+        masked |= (j + window) <= i
+    return np.where(masked, NEG_INF, 0.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.F16, 64), (fa.F16, 96), (fa.BF16, 128), (fa.F32, 64),
+                                      (fa.F32, 128), (fa.F32, 32), (fa.F32, 96)])
+@pytest.mark.parametrize("case", ["full", "causal", "causal_offset", "window", "ragged_tail"])
+def test_prefill_tiled(device, dtype, D, case):
+    want = fa.KERNEL_PREFILL_F32 if dtype == fa.F32 else fa.KERNEL_PREFILL_MFMA
+    B, H, Hkv = 2, 4, 2
+    Sq, Skv, analytic = {"full": (200, 333, None), "causal": (257, 257, (True, 0, 0)),
+                         "causal_offset": (130, 400, (True, 270, 0)), "window": (300, 300, (True, 0, 100)),
+                         "ragged_tail": (65, 127, None)}[case]
+    q, k, v = _normal_qkv(11, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == want
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    mask = None if analytic is None else _analytic_mask(Sq, Skv, *analytic)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                 "qk" if mask is not None else None)
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+    assert_parity(out, ref, tol, f"{case} D{D}")
+    # the generic kernel with the dense mask tensor must agree too
+    if mask is not None:
+        tm = fa.Tensor.from_numpy(device, mask, dtype)
+        out_g = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask), force_kernel=fa.KERNEL_GENERIC).to_numpy()
+        assert_parity(out_g, ref, tol, f"generic {case} D{D}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
+                                     (4, 32, 5000), (1, 128, 1), (16, 128, 260)])
+def test_decode_splitkv(device, dtype, G, D, Skv):
+    B, Hkv = 3, 2
+    q, k, v = _normal_qkv(12, B, Hkv * G, Hkv, 1, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5)
+    tol = dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16
+    assert_parity(out, ref, tol, f"decode G{G} D{D} Skv{Skv}")
+
+
+def test_decode_ragged_kv_lens(device):
+    # per-sequence lengths == un-padded calls == -inf BatchKeyMask padding
+    B, H, Hkv, D, Smax = 5, 4, 4, 96, 3000
+    lens = np.array([3000, 1, 129, 1024, 2047], np.int32)
+    q, k, v = _normal_qkv(13, B, H, Hkv, 1, Smax, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))
+    out = tq.flash_attention(tk, tv, D ** -0.5, kv_lens=fa.IntTensor(device, lens)).to_numpy()
+    bk = np.where(np.arange(Smax)[None, :] < lens[:, None], 0.0, NEG_INF).astype(np.float32)
+    out_m = tq.flash_attention(tk, tv, D ** -0.5, (fa.Tensor.from_numpy(device, bk, fa.F16), fa.MaskKind.BatchKeyMask)).to_numpy()
+    for b in range(B):
+        n = int(lens[b])
+        ref = oracle.flash_attention(rounded(q[b:b + 1], fa.F16), rounded(k[b:b + 1, :, :n], fa.F16),
+                                     rounded(v[b:b + 1, :, :n], fa.F16), D ** -0.5)
+        assert_parity(out[b:b + 1], ref, TOL_16, f"kv_lens b{b} len{n}")
+        assert_parity(out_m[b:b + 1], ref, TOL_16, f"batch-key mask b{b} len{n}")
+
+
+def test_strided_views(device):
+    # K/V as narrowed views of a larger cache allocation, V as the transposed view of [B,S,Hkv,D],
+    # Q transposed from [B,S,H,D] (kalosm-llama attention_layer.rs:257-270; tensor_cache.rs:107-110)
+    B, H, Hkv, S, D, alloc = 2, 8, 2, 150, 64, 256
+    q, k, v = _normal_qkv(14, B, H, Hkv, S, S, D)
+    for dtype in (fa.F32, fa.F16):
+        kbuf = np.zeros((B, Hkv, alloc, D), np.float32)
+        kbuf[:, :, :S] = k
+        tk = fa.Tensor.from_numpy(device, kbuf, dtype).narrow(2, 0, S)
+        tv = fa.Tensor.from_numpy(device, np.ascontiguousarray(v.transpose(0, 2, 1, 3)), dtype).transpose(1, 2)
+        tq = fa.Tensor.from_numpy(device, np.ascontiguousarray(q.transpose(0, 2, 1, 3)), dtype).transpose(1, 2)
+        assert tk.strides[1] == alloc * D and tv.strides == (S * Hkv * D, D, Hkv * D, 1)
+        out = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, 0, 0)).to_numpy()
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                     oracle.get_mask(S, 0), "qk")
+        assert_parity(out, ref, TOL_F32 if dtype == fa.F32 else TOL_16, "strided views")
+        # fully general strides (innermost stride != 1) fall back to the generic kernel
+        tq2 = fa.Tensor.from_numpy(device, np.ascontiguousarray(q.transpose(0, 1, 3, 2)), dtype).transpose(2, 3)
+        assert tq2.selected_kernel(tk, tv, 1.0) == fa.KERNEL_GENERIC
+        out2 = tq2.flash_attention(tk, tv, D ** -0.5, analytic=(True, 0, 0)).to_numpy()
+        assert_parity(out2, ref, TOL_F32 if dtype == fa.F32 else TOL_16, "generic strided")
+
+
+def test_f32_output_for_f16_inputs(device):
+    q, k, v = _normal_qkv(15, 1, 4, 2, 300, 300, 128)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))
+    out = tq.flash_attention(tk, tv, 128 ** -0.5, analytic=(True, 0, 0), out_dtype=fa.F32).to_numpy()
+    assert out.dtype == np.float32
+    ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), 128 ** -0.5,
+                                 oracle.get_mask(300, 0), "qk")
+    assert_parity(out, ref, TOL_16, "f32 out")
+
+
+def test_fully_masked_row_is_nan(device):
+    # the reference gives NaN for a row with no visible key ((-inf) - (-inf), fusor :184-196)
+    q, k, v = _normal_qkv(16, 1, 1, 1, 4, 4, 8)
+    mask = np.zeros((4, 4), np.float32)
+    mask[2, :] = NEG_INF
+    out = run(device, q, k, v, 1.0, mask, fa.MaskKind.QKMask)
+    ref = oracle.flash_attention(q, k, v, 1.0, mask, "qk")
+    assert np.isnan(out[0, 0, 2]).all() and np.isnan(ref[0, 0, 2]).all()
+    keep = [0, 1, 3]
+    assert_parity(out[:, :, keep], ref[:, :, keep], TOL_F32, "unmasked rows")
