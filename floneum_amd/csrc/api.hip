@@ -260,7 +260,6 @@ static void fill_params(const fhip_attn_args *a, AttnParams *p) {
     p->kv_lens = a->kv_lens;
     p->scale = a->scale;
     p->out_f32 = (a->out_dtype == FHIP_F32 && a->dtype != FHIP_F32) ? 1 : 0;
-    p->workspace = a->workspace;
 }
 
 }  // namespace fhip
@@ -534,7 +533,7 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
         const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2];
         decode_plan(B, Hkv, H / Hkv, Skv, D, compute_units > 0 ? compute_units : 256, &chunk, &nsplit);
-        *bytes = decode_workspace_bytes(B, H, D, nsplit);
+        *bytes = decode_workspace_bytes(B, H, Hkv, D, nsplit);
     }
     return FHIP_OK;
 }
@@ -559,11 +558,18 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
             decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, &p.chunk, &p.nsplit);
-            const size_t need = decode_workspace_bytes(p.B, p.H, p.D, p.nsplit);
+            const size_t need = decode_workspace_bytes(p.B, p.H, p.Hkv, p.D, p.nsplit);
             if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
                 set_error("decode needs a workspace of %zu bytes, got %zu", need,
                           args->workspace ? args->workspace_bytes : (size_t)0);
                 return FHIP_ERR_WORKSPACE;
+            }
+            if (need > 0) {
+                if (((uintptr_t)args->workspace & 15) != 0) {
+                    set_error("workspace must be 16-byte aligned");
+                    return FHIP_ERR_WORKSPACE;
+                }
+                p.partials = (float *)args->workspace;
             }
             return launch_decode(p, args->dtype, s->s);  // records main_done itself, before the combine
         }

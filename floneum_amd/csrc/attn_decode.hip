@@ -1,13 +1,19 @@
 // Split-KV decode attention for a 16-bit KV cache (query length 1).
 //
-// Pass 1 (decode_splitkv_kernel): grid = (split, batch * kv_head * head_block).  A workgroup of
-// four wavefronts streams one chunk of keys/values of one KV head exactly once for all the query
-// heads that share it (GQA group), with 128-bit loads laid out so that one wavefront load
-// instruction covers 64/LPK whole key rows back to back (LPK lanes x 8 elements per row).
-// Every group of LPK lanes keeps its own online-softmax state (m, l, acc) in the log2 domain, so
-// the streaming loop needs no cross-lane traffic beyond the LPK-lane dot-product reduction.
-// At the end the states are merged (lanes -> wavefront -> workgroup) and written as one partial
-// (acc[D], m, l) per (batch, head, split).
+// Pass 1: grid = (split, batch * kv_head * head_block).  A workgroup of four wavefronts streams one
+// chunk of keys/values of one KV head exactly once for all the query heads that share it (GQA
+// group).  Two variants:
+//   decode_mfma_kernel (head_dim 32/64/96/128): every wavefront load instruction reads 1 KB of
+//     consecutive key (or value) rows with non-temporal 128-bit loads; the rows are parked in a
+//     wavefront-private LDS tile and fed to the matrix cores: S^T[key][head] = K . Q^T with
+//     v_mfma_f32_16x16x32 (the GQA heads, padded to 16, are the N dimension) and
+//     O^T[dim][head] += V^T . P^T with V^T read by the transposing LDS load.  The softmax state of
+//     head j lives in the lanes with lane % 16 == j, so scores, probabilities and the output
+//     accumulator never change lanes.
+//   decode_vec_kernel (any head_dim multiple of 8 up to 128): LPK lanes x 8 elements per row, dot
+//     products on v_dot2, DPP reductions; every group of LPK lanes keeps its own softmax state.
+// Both keep (m, l, acc) in the log2 domain, merge lanes -> wavefront -> workgroup at the end and
+// write one partial (acc[D], m, l) per (batch, head, split).
 // Pass 2 (decode_combine_kernel): log-sum-exp merge of the partials of each (batch, head).
 // With a single split pass 1 writes the final output and pass 2 is not launched.
 //
@@ -31,14 +37,24 @@ static int env_int(const char *name, int dflt) {
     return v > 0 ? v : dflt;
 }
 
-static int decode_gt(int G) { return G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8; }
+static int decode_gt(int G, int D);
+
+static bool decode_use_mfma(int D) {
+    return (D == 32 || D == 64 || D == 96 || D == 128) && env_int("FHIP_DECODE_VARIANT", 1) == 1;
+}
+
+// query heads handled by one workgroup
+static int decode_gt(int G, int D) {
+    if (decode_use_mfma(D)) return 16;
+    return G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
+}
 
 void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, int *chunk, int *nsplit) {
-    (void)D;
-    const int gt = decode_gt(G);
+    const int gt = decode_gt(G, D);
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
-    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", 4);
+    // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more
+    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", decode_use_mfma(D) ? 2 : 4);
     const int max_chunk = env_int("FHIP_DECODE_MAX_CHUNK", 1024);
     const int min_chunk = env_int("FHIP_DECODE_MIN_CHUNK", 256);
     const long target = (long)compute_units * wgs_per_cu;
@@ -49,12 +65,14 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, int *
     if (ns < ns_min) ns = ns_min;
     if (ns < 1) ns = 1;
     long c = (Skv + ns - 1) / ns;
-    c = (c + 63) / 64 * 64;
+    c = (c + 127) / 128 * 128;  // a workgroup step covers 128 keys
     *chunk = (int)c;
     *nsplit = (int)((Skv + c - 1) / c);
 }
 
-size_t decode_workspace_bytes(int B, int H, int D, int nsplit) {
+// Workspace: the partials, B * H * nsplit * (D + 2) floats.
+size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit) {
+    (void)Hkv;
     if (nsplit <= 1) return 0;
     return (size_t)B * H * nsplit * (size_t)(D + 2) * sizeof(float);
 }
@@ -107,7 +125,7 @@ __device__ __forceinline__ float lpk_sum(float x) {
 // ---- pass 1 -------------------------------------------------------------------------------------
 
 template <typename T, int LPK, int GT>
-__global__ __launch_bounds__(64 * DEC_WAVES) void decode_splitkv_kernel(AttnParams p) {
+__global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p) {
     constexpr int KPI = 64 / LPK;   // key rows covered by one wavefront load
     constexpr int U = DEC_UNROLL;
     constexpr int DMAX = LPK * 8;
@@ -287,7 +305,280 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_splitkv_kernel(AttnPara
             if (p.out_f32) ((float *)p.out)[oi] = o;
             else ((T *)p.out)[oi] = from_float<T>(o);
         } else {
-            float *ws = (float *)p.workspace + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
+            float *ws = (float *)p.partials + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
+            ws[d] = A;
+            if (d == 0) {
+                ws[D] = M;
+                ws[D + 1] = L;
+            }
+        }
+    }
+}
+
+// ---- pass 1, matrix-core variant ----------------------------------------------------------------------
+
+#define DLDS_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
+
+typedef uint32_t uint2v_t __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct DecMma;
+template <>
+struct DecMma<half_t> {
+    typedef half8_t vec8;
+    static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float x, float y) {
+        half2_t h = {(half_t)x, (half_t)y};
+        return __builtin_bit_cast(uint32_t, h);
+    }
+};
+template <>
+struct DecMma<bf16_t> {
+    typedef bf16x8_t vec8;
+    static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float x, float y) {
+        return (uint32_t)from_float<bf16_t>(x).bits | ((uint32_t)from_float<bf16_t>(y).bits << 16);
+    }
+};
+
+// max / sum over the four lanes l, l^16, l^32, l^48 (same head, the four key groups)
+__device__ __forceinline__ float quad_rows_max(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+constexpr int DM_KEYS = 32;  // keys per wavefront step
+constexpr int DM_HEADS = 16; // query heads per workgroup (MFMA N dimension)
+
+template <typename T, int D>
+__global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnParams p) {
+    typedef typename DecMma<T>::vec8 vec8;
+    constexpr int KP = D * 2 + 16;          // K tile row pitch (bytes): rows 4 banks apart
+    constexpr int VP = D * 2 + 32;          // V tile row pitch (bytes): rows 8 banks apart
+    constexpr int K_BYTES = DM_KEYS * KP;
+    constexpr int V_BYTES = DM_KEYS * VP;
+    constexpr int WAVE_BYTES = K_BYTES + V_BYTES;
+    constexpr int CPR = D / 8;              // 16-byte chunks per row
+    constexpr int NLD = DM_KEYS * CPR / 64; // 16-byte loads per lane per tile
+    constexpr int KB = D / 32;              // contraction blocks of QK^T
+    constexpr int NB = D / 16;              // 16-dim blocks of the output
+    constexpr int MERGE_BYTES = DEC_WAVES * DM_HEADS * (D + 2) * 4;
+    constexpr int LDS_BYTES = DEC_WAVES * WAVE_BYTES > MERGE_BYTES ? DEC_WAVES * WAVE_BYTES : MERGE_BYTES;
+    __shared__ __attribute__((aligned(16))) char smem[LDS_BYTES];
+
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 15;  // head column of this lane
+    const int q4 = lane >> 4; // key group
+    auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
+
+    const int split = blockIdx.x;
+    const int HB = (p.G + DM_HEADS - 1) / DM_HEADS;
+    const int hb = blockIdx.y % HB;
+    const int bg = blockIdx.y / HB;
+    const int g = bg % p.Hkv;
+    const int b = bg / p.Hkv;
+    const int h0 = g * p.G + hb * DM_HEADS;
+    const int nh = min(DM_HEADS, p.G - hb * DM_HEADS);
+
+    int kv_hi = p.Skv;
+    if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
+    if (p.kv_lens && split * p.chunk >= kv_hi && split > 0) return;  // the combine pass skips it too
+    int lo = split * p.chunk;
+    int hi = min(lo + p.chunk, kv_hi);
+    if (p.analytic) {
+        if (p.causal) hi = (int)min((int64_t)hi, p.q_pos_offset + 1);
+        if (p.window > 0) lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
+    }
+
+    const uint16_t *kbase = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
+    const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
+    const T *mrow = nullptr;
+    if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask;
+    if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const T *)p.mask + b * p.ms0;
+    const float scale2 = p.scale * LOG2E;
+
+    float4_t o[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) o[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.0f;
+
+    // one wavefront step = 32 consecutive keys; the four wavefronts interleave their steps
+    const int lo_al = lo - (lo % DM_KEYS);
+    const int step = DEC_WAVES * DM_KEYS;
+    uint4_t kst[NLD], vst[NLD];
+    auto load_tile = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = lane + 64 * u;
+            const int row = cid / CPR, col = cid % CPR;
+            const int key = base + row;
+            kst[u] = uint4_t{0, 0, 0, 0};
+            vst[u] = uint4_t{0, 0, 0, 0};
+            if (key >= lo && key < hi) {
+                kst[u] = __builtin_nontemporal_load((const uint4_t *)(kbase + (int64_t)key * p.ks[2] + col * 8));
+                vst[u] = __builtin_nontemporal_load((const uint4_t *)(vbase + (int64_t)key * p.vs[2] + col * 8));
+            }
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = lane + 64 * u;
+            const int row = cid / CPR, col = cid % CPR;
+            *DLDS_PTR(uint4_t, row * KP + col * 16) = kst[u];
+            *DLDS_PTR(uint4_t, K_BYTES + row * VP + col * 16) = vst[u];
+        }
+    };
+
+    int base = lo_al + wave * DM_KEYS;
+    if (base < hi) load_tile(base);  // issued first so the Q fetch below overlaps it
+
+    // Q^T operand: head j, dims 32 kb + 8 q4 .. +8 (zero for the padding heads)
+    vec8 qreg[KB];
+    {
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + (int64_t)(h0 + min(j, nh - 1)) * p.qs[1];
+        const bool qvec = p.qs[3] == 1 && (((uintptr_t)qp) & 15) == 0;
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            uint4_t raw = {0, 0, 0, 0};
+            if (j < nh) {
+                if (qvec) {
+                    raw = *(const uint4_t *)(qp + 32 * kb + 8 * q4);
+                } else {
+                    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t x = qp[(int64_t)(32 * kb + 8 * q4 + e) * p.qs[3]];
+                        w[e >> 1] |= x << ((e & 1) * 16);
+                    }
+                    raw = uint4_t{w[0], w[1], w[2], w[3]};
+                }
+            }
+            qreg[kb] = __builtin_bit_cast(vec8, raw);
+        }
+    }
+
+    for (; base < hi; base += step) {
+        wave_lds_sync();  // the previous step's LDS reads precede these writes
+        store_tile();
+        wave_lds_sync();
+        if (base + step < hi) load_tile(base + step);  // in flight during the math below
+
+        // ---- S^T[key][head] = K . Q^T : two 16-key tiles --------------------------------------------
+        float4_t s[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) {
+                const uint4_t raw = *DLDS_PTR(uint4_t, (16 * t + j) * KP + (32 * kb + 8 * q4) * 2);
+                s[t] = DecMma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], s[t]);
+            }
+        }
+        // element (t, r) is key base + 16 t + 4 q4 + r for head j
+        float sv[8];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int key = base + 16 * t + 4 * q4 + r;
+                const bool visible = key >= lo && key < hi;
+                float x = s[t][r] * scale2;
+                if (mrow && visible) x += to_float(mrow[(int64_t)key * p.ms1]) * LOG2E;
+                sv[4 * t + r] = visible ? x : -INFINITY;
+            }
+        float mx = sv[0];
+#pragma unroll
+        for (int e = 1; e < 8; e++) mx = fmaxf(mx, sv[e]);
+        mx = quad_rows_max(mx);
+        const float m_new = fmaxf(m, mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
+        m = m_new;
+        float pe[8], psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            pe[e] = __builtin_amdgcn_exp2f(sv[e] - m_safe);
+            psum += pe[e];
+        }
+        l = l * corr + psum;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[nb][r] *= corr;
+        // P^T operand: contraction slot (q4, e) is key 4 q4 + e (e < 4) or 16 + 4 q4 + e - 4
+        const uint4_t praw = {DecMma<T>::pack2(pe[0], pe[1]), DecMma<T>::pack2(pe[2], pe[3]),
+                              DecMma<T>::pack2(pe[4], pe[5]), DecMma<T>::pack2(pe[6], pe[7])};
+        const vec8 pop = __builtin_bit_cast(vec8, praw);
+
+        // ---- O^T[dim][head] += V^T . P^T ----------------------------------------------------------------
+        // the transposing load hands lane i of a 16-lane block V[row0 + 0..3][dim0 + i]; the lane
+        // supplies the address of row0 + i / 4, dims dim0 + 4 (i % 4)
+        const int trow = 4 * q4 + (j >> 2);
+        const int tcol = 4 * (j & 3) * 2;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                DLDS_PTR(short4_t, K_BYTES + trow * VP + nb * 32 + tcol));
+            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                DLDS_PTR(short4_t, K_BYTES + (16 + trow) * VP + nb * 32 + tcol));
+            const uint2v_t u0 = __builtin_bit_cast(uint2v_t, a0), u1 = __builtin_bit_cast(uint2v_t, a1);
+            const uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
+            o[nb] = DecMma<T>::mfma(__builtin_bit_cast(vec8, araw), pop, o[nb]);
+        }
+    }
+
+    // ---- merge: key groups -> wavefront -> workgroup ------------------------------------------------
+    l = quad_rows_sum(l);
+    __syncthreads();  // every wavefront is done with its K/V tile; the LDS is reused for the merge
+    float *macc = (float *)smem;  // [wave][head][D + 2]
+    if (j < nh) {
+        float *dst = macc + ((wave * DM_HEADS + j) * (D + 2));
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) dst[16 * nb + 4 * q4 + r] = o[nb][r];
+        if (q4 == 0) {
+            dst[D] = m;
+            dst[D + 1] = l;
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nh * D; idx += 64 * DEC_WAVES) {
+        const int hh = idx / D, d = idx % D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
+        const float Ms = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) {
+            const float *src = macc + (w * DM_HEADS + hh) * (D + 2);
+            const float wgt = __builtin_amdgcn_exp2f(src[D] - Ms);
+            L += wgt * src[D + 1];
+            A += wgt * src[d];
+        }
+        const int h = h0 + hh;
+        if (p.nsplit == 1) {
+            const float val = A / L;  // no visible key: 0/0 = NaN like the reference
+            const int64_t oi = b * p.os[0] + h * p.os[1] + d * p.os[3];
+            if (p.out_f32) ((float *)p.out)[oi] = val;
+            else ((T *)p.out)[oi] = from_float<T>(val);
+        } else {
+            float *ws = (float *)p.partials + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
             ws[d] = A;
             if (d == 0) {
                 ws[D] = M;
@@ -298,6 +589,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_splitkv_kernel(AttnPara
 }
 
 // ---- pass 2 -------------------------------------------------------------------------------------
+// One 64-lane wavefront per (batch, head); up to 8 partials are fetched in one round of loads.
 
 template <typename T>
 __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
@@ -309,46 +601,85 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
         const int len = min(p.Skv, max(p.kv_lens[b], 0));
         ns = max(1, min(ns, (len + p.chunk - 1) / p.chunk));  // split 0 is always written
     }
-    const float *ws = (const float *)p.workspace + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < ns; s++) M = fmaxf(M, ws[(int64_t)s * (D + 2) + D]);
-    const float Ms = (M == -INFINITY) ? 0.0f : M;
-    float L = 0.0f;
-    for (int s = 0; s < ns; s++) L += exp2f(ws[(int64_t)s * (D + 2) + D] - Ms) * ws[(int64_t)s * (D + 2) + D + 1];
-    for (int d = threadIdx.x; d < D; d += 64) {
-        float A = 0.0f;
-        for (int s = 0; s < ns; s++) A += exp2f(ws[(int64_t)s * (D + 2) + D] - Ms) * ws[(int64_t)s * (D + 2) + d];
-        const float o = A / L;
-        const int64_t oi = b * p.os[0] + h * p.os[1] + d * p.os[3];
-        if (p.out_f32) ((float *)p.out)[oi] = o;
-        else ((T *)p.out)[oi] = from_float<T>(o);
+    const float *ws = (const float *)p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
+    const int d0 = threadIdx.x, d1 = threadIdx.x + 64;
+    float M = -INFINITY, L = 0.0f, A0 = 0.0f, A1 = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+        float ms[8], ls[8], a0[8], a1[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const bool ok = s0 + u < ns;
+            const float *src = ws + (int64_t)(ok ? s0 + u : s0) * (D + 2);
+            ms[u] = ok ? src[D] : -INFINITY;
+            ls[u] = ok ? src[D + 1] : 0.0f;
+            a0[u] = (ok && d0 < D) ? src[d0] : 0.0f;
+            a1[u] = (ok && d1 < D) ? src[d1] : 0.0f;
+        }
+        float Mn = M;
+#pragma unroll
+        for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
+        const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+        const float c = __builtin_amdgcn_exp2f(M - Ms);
+        L *= c;
+        A0 *= c;
+        A1 *= c;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
+            L += w * ls[u];
+            A0 += w * a0[u];
+            A1 += w * a1[u];
+        }
+        M = Mn;
+    }
+    const int64_t ob = b * p.os[0] + h * p.os[1];
+    if (d0 < D) {
+        const float val = A0 / L;
+        if (p.out_f32) ((float *)p.out)[ob + d0 * p.os[3]] = val;
+        else ((T *)p.out)[ob + d0 * p.os[3]] = from_float<T>(val);
+    }
+    if (d1 < D) {
+        const float val = A1 / L;
+        if (p.out_f32) ((float *)p.out)[ob + d1 * p.os[3]] = val;
+        else ((T *)p.out)[ob + d1 * p.os[3]] = from_float<T>(val);
     }
 }
 
 template <typename T, int LPK>
-static void launch_pass1(const AttnParams &p, dim3 grid, hipStream_t stream, int gt) {
+static void launch_vec(const AttnParams &p, dim3 grid, hipStream_t stream, int gt) {
     dim3 block(64 * DEC_WAVES);
     switch (gt) {
-        case 1: hipLaunchKernelGGL((decode_splitkv_kernel<T, LPK, 1>), grid, block, 0, stream, p); break;
-        case 2: hipLaunchKernelGGL((decode_splitkv_kernel<T, LPK, 2>), grid, block, 0, stream, p); break;
-        case 4: hipLaunchKernelGGL((decode_splitkv_kernel<T, LPK, 4>), grid, block, 0, stream, p); break;
-        default: hipLaunchKernelGGL((decode_splitkv_kernel<T, LPK, 8>), grid, block, 0, stream, p); break;
+        case 1: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 1>), grid, block, 0, stream, p); break;
+        case 2: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 2>), grid, block, 0, stream, p); break;
+        case 4: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 4>), grid, block, 0, stream, p); break;
+        default: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 8>), grid, block, 0, stream, p); break;
     }
 }
 
 template <typename T>
 static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
-    const int gt = decode_gt(p.G);
+    const int gt = decode_gt(p.G, p.D);
     const int hb = (p.G + gt - 1) / gt;
     const long gy = (long)p.B * p.Hkv * hb;
     if (gy > 65535 || p.nsplit > 0x7fffffff) {
         set_error("decode: batch * kv_heads * head_blocks = %ld exceeds the grid limit 65535", gy);
         return FHIP_ERR_UNSUPPORTED;
     }
-    dim3 grid((unsigned)p.nsplit, (unsigned)gy);
-    if (p.D <= 32) launch_pass1<T, 4>(p, grid, stream, gt);
-    else if (p.D <= 64) launch_pass1<T, 8>(p, grid, stream, gt);
-    else launch_pass1<T, 16>(p, grid, stream, gt);
+    dim3 grid((unsigned)p.nsplit, (unsigned)gy), block(64 * DEC_WAVES);
+    if (decode_use_mfma(p.D)) {
+        switch (p.D) {
+            case 32: hipLaunchKernelGGL((decode_mfma_kernel<T, 32>), grid, block, 0, stream, p); break;
+            case 64: hipLaunchKernelGGL((decode_mfma_kernel<T, 64>), grid, block, 0, stream, p); break;
+            case 96: hipLaunchKernelGGL((decode_mfma_kernel<T, 96>), grid, block, 0, stream, p); break;
+            default: hipLaunchKernelGGL((decode_mfma_kernel<T, 128>), grid, block, 0, stream, p); break;
+        }
+    } else if (p.D <= 32) {
+        launch_vec<T, 4>(p, grid, stream, gt);
+    } else if (p.D <= 64) {
+        launch_vec<T, 8>(p, grid, stream, gt);
+    } else {
+        launch_vec<T, 16>(p, grid, stream, gt);
+    }
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
     if (p.nsplit > 1) {

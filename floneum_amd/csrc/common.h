@@ -23,7 +23,7 @@ struct AttnParams {
     float scale;
     int32_t out_f32;        // 1: out is f32 although the inputs are 16-bit
     // split-KV decode only
-    void *workspace;
+    float *partials;        // [B, H, nsplit, D + 2] per-split (acc, m, l)
     int32_t chunk;          // keys per split
     int32_t nsplit;         // splits per (batch, kv head) over Skv
     hipEvent_t main_done;   // host-side only: recorded after the main kernel when not null
@@ -47,11 +47,12 @@ int launch_prefill_f32(const AttnParams &p, hipStream_t stream);
 
 // decode planning (host): keys per split and number of splits
 void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, int *chunk, int *nsplit);
-size_t decode_workspace_bytes(int B, int H, int D, int nsplit);
+size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 
 // KV cache copies
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream);
+int launch_fill_zero_bytes(void *dst, size_t bytes, hipStream_t stream);
 int launch_fill_zero_rows(void *dst, const int64_t dstride[4], const uint32_t shape[4], int elem_bytes,
                           hipStream_t stream);
 

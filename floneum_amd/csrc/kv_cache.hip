@@ -102,6 +102,23 @@ static int copy_or_zero(const void *src, const int64_t *ss, void *dst, const int
     return FHIP_OK;
 }
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *dst, size_t words) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256) dst[i] = 0u;
+}
+
+// Zero fill by a kernel (not a memset node), so a caller may record it into a HIP graph.
+int launch_fill_zero_bytes(void *dst, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return FHIP_OK;
+    if (((uintptr_t)dst & 3) != 0 || (bytes & 3) != 0) {
+        set_error("zero fill needs a 4-byte aligned pointer and size");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const size_t words = bytes / 4;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for((int64_t)words)), dim3(256), 0, stream, (uint32_t *)dst, words);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream) {
     return copy_or_zero(src, sstride, dst, dstride, shape, elem_bytes, false, stream);

@@ -107,8 +107,9 @@ typedef struct {
     /* Optional device array of B int32: keys j >= kv_lens[b] are masked for batch b.  Equivalent
      * to a 0 / -inf BatchKeyMask; it exists so a ragged batch needs no [B,Skv] mask tensor. */
     const int32_t *kv_lens;
-    void *workspace; /* device scratch, >= fhip_flash_attention_workspace_bytes(); may be NULL
-                        when that reports 0                                                         */
+    void *workspace; /* device scratch, >= fhip_flash_attention_workspace_bytes(), 16-byte aligned,
+                        contents irrelevant; may be NULL when the size query reports 0.  Calls that
+                        share a workspace must not overlap.                                          */
     size_t workspace_bytes;
     int32_t force_kernel; /* 0 = choose; otherwise a fhip_kernel_id (testing / benchmarking)       */
     /* Optional profiling hook: when non-NULL the event is recorded on the stream right after the
