@@ -184,6 +184,12 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     if (!(a->scale > 0.0f)) return false;
     if (a->mask_kind != FHIP_MASK_NONE) return false;  // dense additive masks take the generic kernel
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
+    // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv
+    // head) slice must span less than 2 GiB
+    const uint64_t Skv = a->k.shape[2];
+    if (a->k.stride[2] < (int64_t)D || a->v.stride[2] < (int64_t)D) return false;
+    if (Skv * (uint64_t)a->k.stride[2] * 2 >= 0x7fffffffull || Skv * (uint64_t)a->v.stride[2] * 2 >= 0x7fffffffull)
+        return false;
     return true;
 }
 
@@ -552,6 +558,9 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     fill_params(args, &p);
     FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+#ifdef EXP_TRACE
+    p.partials = (float *)args->workspace;
+#endif
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;

@@ -1,14 +1,20 @@
 // Prefill attention for f16 / bf16 on the gfx950 matrix cores.
 //
-// Workgroup = 4 wavefronts = 128 query rows of one (batch, head); each wavefront owns 32 rows.
-// Keys/values are walked in tiles of 64 rows staged through LDS.  Per tile and wavefront:
+// Workgroup = 8 wavefronts = 256 query rows of one (batch, head); each wavefront owns 32 rows.
+// Keys/values are walked in tiles of 64 rows staged through double-buffered LDS.  Per tile and
+// wavefront:
 //   S^T (64 keys x 32 queries)  = K_tile . Q^T      v_mfma_f32_32x32x16  (A = K from LDS, B = Q in registers)
 //   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of
 //   it per 32-key block, so the row max / row sum are in-lane folds plus one exchange with the
-//   lane 32 away (v_permlane32_swap)
+//   lane 32 away (v_permlane32_swap); the rescale of O is skipped while the running maximum moves
+//   by less than 2^8
 //   O^T (D x 32 queries)       += V_tile^T . P^T    A = V^T read from row-major LDS with the
 //   transposing LDS load ds_read_b64_tr_b16, B = P^T taken straight from the S^T accumulator
 //   registers (the contraction index is permuted identically on both operands)
+// The two wavefronts that share a SIMD (w and w + 4) run half a tile out of phase: while one is in
+// its matrix phase (P.V of the previous tile, then S^T of the current one) the other is in its
+// vector phase (softmax), so the MFMA pipe and the VALU are busy at the same time.  Phases are
+// separated by workgroup barriers; the tile loads ride on the same barriers.
 // All accumulation is f32; P is rounded to the input type for the second product.
 // Masking is analytic (causal with offset, sliding window, per-batch kv length, tail of the key
 // axis); key tiles that are invisible to the whole workgroup are never loaded, and tiles fully
@@ -17,12 +23,14 @@
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199, f32 accumulation
 // of 16-bit inputs as fusor-ml/core/src/composite/flash_attention.rs:186-203,323-327; head
 // mapping kv_head = head / (H / Hkv) (core :135-137,163-167).
+#include <type_traits>
+
 #include "common.h"
 #include "device_utils.h"
 
 namespace fhip {
 
-constexpr int PF_WAVES = 4;
+constexpr int PF_WAVES = 8;
 constexpr int PF_BM = 32 * PF_WAVES;  // query rows per workgroup
 constexpr int PF_BN = 64;             // key rows per tile
 constexpr float PF_LOG2E = 1.4426950408889634f;
@@ -60,7 +68,7 @@ struct PfCfg {
     static constexpr int K_BYTES = PF_BN * KP;
     static constexpr int V_BYTES = PF_BN * VP;
     static constexpr int CPR = D / 8;                                // 16-byte chunks per row
-    static constexpr int NCH = PF_BN * CPR / (64 * PF_WAVES);        // chunks per thread per tile
+    static constexpr int NCH = PF_BN * CPR / 256;                    // chunks per thread of the 4 moving wavefronts
 };
 
 __device__ __forceinline__ float half_swap_max(float x) {
@@ -73,18 +81,37 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+template <typename T>
+__device__ __forceinline__ float packed_pair_sum(uint32_t pk, float acc);
+template <>
+__device__ __forceinline__ float packed_pair_sum<half_t>(uint32_t pk, float acc) {
+    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, pk), ones, acc, false);  // acc + lo + hi in f32
+}
+template <>
+__device__ __forceinline__ float packed_pair_sum<bf16_t>(uint32_t pk, float acc) {
+    return acc + __uint_as_float(pk << 16) + __uint_as_float(pk & 0xffff0000u);
+}
+
+// Rows whose running maximum is stale by at most this much (log2 domain) keep it: probabilities
+// then reach 2^8 at most, well inside f16/bf16 range, and the 64-register rescale of O is skipped
+// on almost every tile.
+constexpr float PF_RESCALE_SLACK = 8.0f;
+
 template <typename T, int D>
-__global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnParams p, int nqb) {
+__global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnParams p, int nqb, int out_vec) {
     typedef PfCfg<D> C;
     typedef typename Mma<T>::vec8 vec8;
-    __shared__ __attribute__((aligned(16))) char smem[C::K_BYTES + C::V_BYTES];
+    constexpr int STAGE = C::K_BYTES + C::V_BYTES;
+    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    const int ln = lane & 31;  // query column / key row owned inside a 32-wide MFMA block
-    const int h2 = lane >> 5;  // which half of the contraction slice
+    const int ln = lane & 31;      // query column / key row owned inside a 32-wide MFMA block
+    const int h2 = lane >> 5;      // which half of the contraction slice
+    const int group = wave >> 2;   // wavefronts w and w + 4 share a SIMD and run out of phase
 
     // workgroup -> (query block, batch, head): long query blocks first, and heads laid out so
     // the workgroups that land on one XCD (id % 8) share a KV head whenever H is a multiple of 8
@@ -100,31 +127,32 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int q0 = qb * PF_BM;
     const int qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
-    const int off = (int)p.q_pos_offset;
+    const int64_t off = p.q_pos_offset;
 
     int kv_hi = p.Skv;
     if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
 
-    // key range visible to the workgroup / to this wavefront
+    // visible key interval [klo, khi) of a query row r:  j < kv_hi, j <= r + off (causal),
+    // j + window > r + off (sliding window)
+    auto row_lo = [&](int r) __attribute__((always_inline)) -> int {
+        return (p.analytic && p.window > 0) ? (int)max((int64_t)0, (int64_t)r + off - p.window + 1) : 0;
+    };
+    auto row_hi = [&](int r) __attribute__((always_inline)) -> int {
+        return (p.analytic && p.causal) ? (int)min((int64_t)kv_hi, (int64_t)r + off + 1) : kv_hi;
+    };
     const int q_last_wg = min(q0 + PF_BM - 1, p.Sq - 1);
     const int q_last_w = min(qw0 + 31, p.Sq - 1);
-    int hi_wg = kv_hi, lo_wg = 0, hi_w = kv_hi, lo_w = 0;
-    if (p.analytic) {
-        if (p.causal) {
-            hi_wg = (int)min((int64_t)kv_hi, (int64_t)q_last_wg + off + 1);
-            hi_w = (int)min((int64_t)kv_hi, (int64_t)q_last_w + off + 1);
-        }
-        if (p.window > 0) {
-            lo_wg = (int)max((int64_t)0, (int64_t)q0 + off - p.window + 1);
-            lo_w = (int)max((int64_t)0, (int64_t)qw0 + off - p.window + 1);
-        }
-    }
+    const int q_first_w = min(qw0, p.Sq - 1);
+    const int lo_wg = row_lo(q0), hi_wg = row_hi(q_last_wg);        // union over the workgroup's rows
+    const int lo_w = row_lo(q_first_w), hi_w = row_hi(q_last_w);    // union over this wavefront's rows
+    const int full_lo_w = row_lo(q_last_w), full_hi_w = row_hi(q_first_w);  // intersection
+    const int qrow = min(query, p.Sq - 1);
+    const int klo = row_lo(qrow), khi = row_hi(qrow);               // this lane's row
     const bool wave_has_rows = qw0 < p.Sq;
 
     // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel
     vec8 qreg[D / 16];
     {
-        const int qrow = min(query, p.Sq - 1);
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
@@ -133,8 +161,18 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         }
     }
 
+    const int j_begin = (lo_wg / PF_BN) * PF_BN;
+    const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PF_BN - 1) / PF_BN : 0;
+
+    // K and V of this (batch, kv head) as raw buffers: a row beyond the end of the key axis reads as
+    // zero, so the tile loop needs neither clamps nor 64-bit address arithmetic
     const uint16_t *kg = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
     const uint16_t *vg = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
+    const int krow_bytes = (int)p.ks[2] * 2, vrow_bytes = (int)p.vs[2] * 2;
+    const __amdgpu_buffer_rsrc_t krs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)kg, 0, (p.Skv - 1) * krow_bytes + D * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)vg, 0, (p.Skv - 1) * vrow_bytes + D * 2, 0x00020000);
 
     float16_t o[D / 32];
 #pragma unroll
@@ -144,41 +182,38 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     float m = -INFINITY, l = 0.0f;
     const float scale2 = p.scale * PF_LOG2E;
 
-    uint4_t kst[C::NCH], vst[C::NCH];
-    auto load_tile = [&](int j0) {
+    // ---- tile movement: global -> registers -> LDS ---------------------------------------------------
+    // The four wavefronts of a group move one whole tile: group 1 moves the K tiles, group 0 the V
+    // tiles, each during its own vector phase (the matrix-phase wavefronts do nothing but MFMA work).
+    uint4_t st[C::NCH];
+    int gofs[C::NCH], lofs[C::NCH];  // per-thread global / LDS byte offsets of its chunks
+    const int mrow_bytes = group ? krow_bytes : vrow_bytes;
+    const __amdgpu_buffer_rsrc_t mrs = group ? krs : vrs;
 #pragma unroll
-        for (int i = 0; i < C::NCH; i++) {
-            const int cid = tid + 64 * PF_WAVES * i;
-            const int row = cid / C::CPR, col = cid % C::CPR;
-            const int key = min(j0 + row, p.Skv - 1);
-            kst[i] = *(const uint4_t *)(kg + (int64_t)key * p.ks[2] + col * 8);
-            vst[i] = *(const uint4_t *)(vg + (int64_t)key * p.vs[2] + col * 8);
-        }
-    };
-    auto store_tile = [&]() {
+    for (int i = 0; i < C::NCH; i++) {
+        const int cid = (tid & 255) + 256 * i;
+        const int row = cid / C::CPR, col = cid % C::CPR;
+        gofs[i] = row * mrow_bytes + col * 16;
+        lofs[i] = group ? row * C::KP + col * 16 : C::K_BYTES + row * C::VP + col * 16;
+    }
+    // a tile that starts beyond the key axis is never used: clamp the (uniform) offset so it stays
+    // inside 32 bits; rows past Skv inside a used tile are out of range of the buffer and read 0
+    auto load_tile = [&](int tile) __attribute__((always_inline)) {
+        const int soff = min(j_begin + tile * PF_BN, p.Skv) * mrow_bytes;
 #pragma unroll
-        for (int i = 0; i < C::NCH; i++) {
-            const int cid = tid + 64 * PF_WAVES * i;
-            const int row = cid / C::CPR, col = cid % C::CPR;
-            *LDS_PTR(uint4_t, row * C::KP + col * 16) = kst[i];
-            *LDS_PTR(uint4_t, C::K_BYTES + row * C::VP + col * 16) = vst[i];
-        }
+        for (int i = 0; i < C::NCH; i++) st[i] = __builtin_amdgcn_raw_buffer_load_b128(mrs, gofs[i], soff, 0);
+    };
+    auto store_tile = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < C::NCH; i++) *LDS_PTR(uint4_t, (tile & 1) * STAGE + lofs[i]) = st[i];
     };
 
-    const int j_begin = (lo_wg / PF_BN) * PF_BN;
-    if (j_begin < hi_wg) load_tile(j_begin);
+    float16_t s[2];     // S^T of the tile in flight
+    uint32_t pk[2][8];  // its probabilities, packed pairs in the MFMA operand order
 
-    for (int j0 = j_begin; j0 < hi_wg; j0 += PF_BN) {
-        __syncthreads();  // everyone finished reading the previous tile
-        store_tile();
-        __syncthreads();
-        if (j0 + PF_BN < hi_wg) load_tile(j0 + PF_BN);
-
-        const bool tile_visible = wave_has_rows && j0 < hi_w && j0 + PF_BN > lo_w;
-        if (!tile_visible) continue;
-
-        // ---- S^T = K . Q^T --------------------------------------------------------------------
-        float16_t s[2];
+    // S^T = K . Q^T for tile i
+    auto qk = [&](int i) __attribute__((always_inline)) {
+        const int stage = i & 1;
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -187,99 +222,296 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         for (int kb = 0; kb < D / 16; kb++) {
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                uint4_t raw = *LDS_PTR(uint4_t, (32 * t + ln) * C::KP + kb * 32 + h2 * 16);
+                uint4_t raw = *LDS_PTR(uint4_t, stage * STAGE + (32 * t + ln) * C::KP + kb * 32 + h2 * 16);
                 s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], s[t]);
             }
         }
-
-        // ---- mask ------------------------------------------------------------------------------
-        // element r of block t is key j0 + 32 t + 8 (r / 4) + 4 h2 + r % 4 for query `query`
-        bool full = j0 + PF_BN <= kv_hi;
-        if (p.analytic) {
-            if (p.causal) full = full && (j0 + PF_BN - 1 <= qw0 + off);
-            if (p.window > 0) full = full && ((int64_t)j0 + p.window > (int64_t)q_last_w + off);
-        }
-        if (!full) {
-            const int qpos = query + off;
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = j0 + 32 * t + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                    bool vis = key < kv_hi;
-                    if (p.analytic) {
-                        if (p.causal) vis = vis && key <= qpos;
-                        if (p.window > 0) vis = vis && ((int64_t)key + p.window > (int64_t)qpos);
-                    }
-                    s[t][r] = vis ? s[t][r] : -INFINITY;
-                }
-        }
-
-        // ---- online softmax (log2 domain) ------------------------------------------------------
-        float mx = s[0][0];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-        mx = half_swap_max(mx);
-        const float m_new = fmaxf(m, mx * scale2);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
-        m = m_new;
-        float psum = 0.0f;
-        uint32_t pk[2][8];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[t][r], scale2, -m_safe));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[t][r + 1], scale2, -m_safe));
-                psum += p0 + p1;
-                pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
-            }
-        l = l * corr + psum;
-#pragma unroll
-        for (int db = 0; db < D / 32; db++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[db][r] *= corr;
-
-        // ---- O^T += V^T . P^T ------------------------------------------------------------------
-        // contraction slice (t, kk): this half-wave's keys are 32 t + 16 kk + 4 h2 + {0..3} and + 8
+    };
+    // O^T += V^T . P^T for tile i: contraction slice (t, kk) holds this half-wave's keys
+    // 32 t + 16 kk + 4 h2 + {0..3} and + 8
+    auto pv = [&](int i) __attribute__((always_inline)) {
+        const int stage = i & 1;
         const int i16 = lane & 15;
         const int bl = (lane & 31) >> 4;
 #pragma unroll
         for (int t = 0; t < 2; t++) {
 #pragma unroll
             for (int kk = 0; kk < 2; kk++) {
-                uint4_t braw = {pk[t][4 * kk], pk[t][4 * kk + 1], pk[t][4 * kk + 2], pk[t][4 * kk + 3]};
+                const uint4_t braw = {pk[t][4 * kk], pk[t][4 * kk + 1], pk[t][4 * kk + 2], pk[t][4 * kk + 3]};
                 const vec8 bop = __builtin_bit_cast(vec8, braw);
                 const int krow = 32 * t + 16 * kk + 4 * h2 + (i16 >> 2);
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
                     const int colb = (32 * db + 16 * bl + 4 * (i16 & 3)) * 2;
                     short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        LDS_PTR(short4_t, C::K_BYTES + krow * C::VP + colb));
+                        LDS_PTR(short4_t, stage * STAGE + C::K_BYTES + krow * C::VP + colb));
                     short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        LDS_PTR(short4_t, C::K_BYTES + (krow + 8) * C::VP + colb));
-                    uint4_t araw = {__builtin_bit_cast(uint2_t, a0)[0], __builtin_bit_cast(uint2_t, a0)[1],
-                                    __builtin_bit_cast(uint2_t, a1)[0], __builtin_bit_cast(uint2_t, a1)[1]};
+                        LDS_PTR(short4_t, stage * STAGE + C::K_BYTES + (krow + 8) * C::VP + colb));
+                    const uint2_t u0 = __builtin_bit_cast(uint2_t, a0), u1 = __builtin_bit_cast(uint2_t, a1);
+                    uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
                     o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, araw), bop, o[db]);
                 }
             }
         }
+    };
+    // Matrix phase in one basic block: P.V of tile ip, then S^T of tile ik, with the LDS operand
+    // reads issued two MFMA groups ahead of their use (the order is pinned by the scheduling groups
+    // at the end; without them the reads sit right in front of their MFMAs and the pipe waits out the
+    // LDS latency every four instructions).
+    auto pv_qk = [&](int ip, int ik) __attribute__((always_inline)) {
+        constexpr int NDB = D / 32, NKB = D / 16;
+        const int vstage = (ip & 1) * STAGE + C::K_BYTES, kstage = (ik & 1) * STAGE;
+        const int i16 = lane & 15;
+        const int bl = (lane & 31) >> 4;
+        const int vbase = vstage + (4 * h2 + (i16 >> 2)) * C::VP + (16 * bl + 4 * (i16 & 3)) * 2;
+        const int kbase = kstage + ln * C::KP + h2 * 16;
+        uint4_t va[2][NDB];
+        auto read_v = [&](int gq, uint4_t (&a)[NDB]) {  // gq = 2 t + kk: rows 32 t + 16 kk (+8)
+#pragma unroll
+            for (int db = 0; db < NDB; db++) {
+                const int addr = vbase + (16 * gq) * C::VP + db * 64;
+                short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr));
+                short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VP));
+                const uint2_t u0 = __builtin_bit_cast(uint2_t, a0), u1 = __builtin_bit_cast(uint2_t, a1);
+                a[db] = uint4_t{u0[0], u0[1], u1[0], u1[1]};
+            }
+        };
+        auto mfma_v = [&](int gq, const uint4_t (&a)[NDB]) {
+            const int t = gq >> 1, kk = gq & 1;
+            const uint4_t braw = {pk[t][4 * kk], pk[t][4 * kk + 1], pk[t][4 * kk + 2], pk[t][4 * kk + 3]};
+            const vec8 bop = __builtin_bit_cast(vec8, braw);
+#pragma unroll
+            for (int db = 0; db < NDB; db++) o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, a[db]), bop, o[db]);
+        };
+        uint4_t ka[4][2];
+        auto read_k = [&](int kb, uint4_t (&a)[2]) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + 32 * t * C::KP + kb * 32);
+        };
+        read_v(0, va[0]);
+        read_v(1, va[1]);
+        mfma_v(0, va[0]);
+        read_v(2, va[0]);
+        mfma_v(1, va[1]);
+        read_v(3, va[1]);
+        mfma_v(2, va[0]);
+#pragma unroll
+        for (int kb = 0; kb < 4 && kb < NKB; kb++) read_k(kb, ka[kb]);
+        mfma_v(3, va[1]);
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[t][r] = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < NKB; kb++) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, ka[kb & 3][t]), qreg[kb], s[t]);
+            if (kb + 4 < NKB) read_k(kb + 4, ka[kb & 3]);
+        }
+        // scheduling groups: 0x100 = LDS read, 0x008 = MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 4 * NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+#pragma unroll
+        for (int kb = 0; kb < NKB; kb++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            if (kb + 4 < NKB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+    };
+    // mask + online softmax (log2 domain, lazily rescaled) of tile i: s -> pk
+    auto softmax = [&](int i) __attribute__((always_inline)) {
+        const int j0 = j_begin + i * PF_BN;
+        if (!(j0 >= full_lo_w && j0 + PF_BN <= full_hi_w)) {
+            // element r of block t is key j0 + 32 t + 8 (r / 4) + 4 h2 + r % 4
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = j0 + 32 * t + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                    s[t][r] = (key >= klo && key < khi) ? s[t][r] : -INFINITY;
+                }
+        }
+        float mx = s[0][0];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+        mx = half_swap_max(mx) * scale2;
+        const bool grow = mx > m + PF_RESCALE_SLACK;  // also true for the first visible tile (m = -inf)
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float m_new = grow ? mx : m;
+            const float corr = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m - m_new);
+            m = m_new;
+            l *= corr;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= corr;
+        }
+        const float m_safe = (m == -INFINITY) ? 0.0f : m;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[t][r], scale2, -m_safe));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[t][r + 1], scale2, -m_safe));
+                pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
+                l = packed_pair_sum<T>(pk[t][r >> 1], l);  // the rounded values the MFMA will use
+            }
+    };
+    auto tile_visible = [&](int i) __attribute__((always_inline)) {
+        const int j0 = j_begin + i * PF_BN;
+        return i >= 0 && i < ntiles && wave_has_rows && j0 < hi_w && j0 + PF_BN > lo_w;
+    };
+
+    // ---- slot schedule ---------------------------------------------------------------------------------
+    // Slots are separated by workgroup barriers.  Group 0 is in its matrix phase in even slots and in
+    // its vector phase in odd slots; group 1 the other way round, one slot later.  Matrix phase of
+    // tile i: P.V of tile i-1 (reads V(i-1)), then S^T of tile i (reads K(i)).  Vector phase: the tile
+    // movement, then the softmax of tile i.  K(i) and V(i-1) are read in slots 2i and 2i+1.
+    // In even slot 2j group 1 moves K(j+1) from registers to LDS and fetches K(j+2); in odd slot 2j+1
+    // group 0 moves V(j) and fetches V(j+1).  Each buffer is rewritten after the barrier that follows
+    // its last reader and a full slot before its next reader.
+    // The tiles visible to a wavefront form one contiguous range [ia, ib).  Each group walks the slot
+    // sequence in five static segments (nothing / first tile / steady state / last tile / nothing) so
+    // that the steady-state loop body is branch-free and no state changes registers between phases.
+    int ia = 0, ib = 0;
+    if (wave_has_rows && hi_w > lo_w) {
+        ia = (lo_w - j_begin) / PF_BN;
+        ib = min(ntiles, (hi_w - j_begin + PF_BN - 1) / PF_BN);
+        if (ib < ia) ib = ia;
+    }
+    // MODE bit 0: S^T of tile i; bit 1: P.V of tile i-1; bit 2: softmax of tile i (group 0) / i-1 (group 1)
+    auto matrix_phase = [&](int i, auto mode) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode)::value;
+        __builtin_amdgcn_s_setprio(1);
+#ifndef EXP_NO_MFMA
+        if constexpr ((MODE & 3) == 3) pv_qk(i - 1, i);
+        else if constexpr ((MODE & 3) == 2) pv(i - 1);
+        else if constexpr ((MODE & 3) == 1) qk(i);
+#endif
+        __builtin_amdgcn_s_setprio(0);
+    };
+    auto vector_phase = [&](int i, int tile_to_store, auto mode) __attribute__((always_inline)) {
+        constexpr int MODE = decltype(mode)::value;
+        store_tile(tile_to_store);
+        load_tile(tile_to_store + 1);
+#ifndef EXP_NO_SOFTMAX
+        if constexpr ((MODE & 4) != 0) softmax(i);
+#endif
+    };
+    auto segment0 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 0: slot 2i matrix, slot 2i+1 vector + V(i)
+        for (int i = i0; i < i1; i++) {
+            matrix_phase(i, mode);
+            lds_barrier();
+            vector_phase(i, i, mode);
+            lds_barrier();
+        }
+    };
+    auto segment1 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 1: slot 2i vector (tile i-1) + K(i+1), slot 2i+1 matrix
+        for (int i = i0; i < i1; i++) {
+            vector_phase(i - 1, i + 1, mode);
+            lds_barrier();
+            matrix_phase(i, mode);
+            lds_barrier();
+        }
+    };
+    using std::integral_constant;
+    if (ntiles > 0) {
+        if (group) {
+            load_tile(0);
+            store_tile(0);
+            load_tile(1);
+        } else {
+            load_tile(0);
+        }
+        lds_barrier();
+        if (group == 0) {
+            // iteration i: S^T(i), softmax(i), P.V(i-1)
+            segment0(0, ia, integral_constant<int, 0>{});
+            if (ia < ib) {
+                segment0(ia, ia + 1, integral_constant<int, 1 | 4>{});
+                segment0(ia + 1, ib, integral_constant<int, 1 | 2 | 4>{});
+                segment0(ib, ib + 1, integral_constant<int, 2>{});
+                segment0(ib + 1, ntiles + 1, integral_constant<int, 0>{});
+            } else {
+                segment0(ia, ntiles + 1, integral_constant<int, 0>{});
+            }
+        } else {
+            // iteration i: softmax(i-1), then S^T(i) and P.V(i-1)
+            segment1(0, ia, integral_constant<int, 0>{});
+            if (ia < ib) {
+                segment1(ia, ia + 1, integral_constant<int, 1>{});
+                segment1(ia + 1, ib, integral_constant<int, 1 | 2 | 4>{});
+                segment1(ib, ib + 1, integral_constant<int, 2 | 4>{});
+                segment1(ib + 1, ntiles + 1, integral_constant<int, 0>{});
+            } else {
+                segment1(ia, ntiles + 1, integral_constant<int, 0>{});
+            }
+        }
     }
 
-    // ---- epilogue: out[query][dim] = O^T[dim][query] / l ----------------------------------------
+    // ---- epilogue: out[query][dim] = O^T[dim][query] / l ----------------------------------------------
     const float l_tot = half_swap_sum(l);
-    if (query < p.Sq) {
-        const float inv = 1.0f / l_tot;  // no visible key: l = 0 -> 0 * inf = NaN, like the reference
+    const float inv = 1.0f / l_tot;
+    const bool dead = (l_tot == 0.0f);  // no visible key: the reference gives NaN (0/0)
+    if (out_vec) {
+        // transpose through a wavefront-private slice of the LDS so that every global store is a
+        // 16-byte piece of a contiguous row; 32 rows per round for 2-byte outputs, 16 for f32
+        const int esz = p.out_f32 ? 4 : 2;
+        const int pitch = D * esz + 16;                      // rows stay 16-byte aligned, 4 banks apart
+        constexpr int SLICE = 32 * (D * 2 + 16);             // bytes per wavefront
+        static_assert(PF_WAVES * SLICE <= 2 * STAGE, "epilogue staging exceeds the tile buffers");
+        auto wbase = lds_base + wave * SLICE;
+        const int rounds = p.out_f32 ? 2 : 1;
+        const int rows_per_round = 32 / rounds;
+        const int cpr = D * esz / 16;
+        char *og = (char *)p.out;
+        for (int rd = 0; rd < rounds; rd++) {
+            const int row_lo_ = rd * rows_per_round;
+            if (ln >= row_lo_ && ln < row_lo_ + rows_per_round) {
+#pragma unroll
+                for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        float v4[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v4[e] = dead ? __builtin_nanf("") : o[db][4 * rq + e] * inv;
+                        const int dim = 32 * db + 8 * rq + 4 * h2;
+                        if (p.out_f32) {
+                            *(__attribute__((address_space(3))) float4_t *)(wbase + (ln - row_lo_) * pitch + dim * 4) =
+                                float4_t{v4[0], v4[1], v4[2], v4[3]};
+                        } else {
+                            const uint2_t pk2 = {Mma<T>::pack2(v4[0], v4[1]), Mma<T>::pack2(v4[2], v4[3])};
+                            *(__attribute__((address_space(3))) uint2_t *)(wbase + ln * pitch + dim * 2) = pk2;
+                        }
+                    }
+            }
+            wave_lds_sync();
+            for (int c = lane; c < rows_per_round * cpr; c += 64) {
+                const int row = c / cpr, col = c % cpr;
+                const int qr = qw0 + row_lo_ + row;
+                if (qr < p.Sq) {
+                    const uint4_t val = *(__attribute__((address_space(3))) uint4_t *)(wbase + row * pitch + col * 16);
+                    const int64_t eidx = b * p.os[0] + h * p.os[1] + (int64_t)qr * p.os[2];
+                    *(uint4_t *)(og + eidx * esz + col * 16) = val;
+                }
+            }
+            wave_lds_sync();
+        }
+    } else if (query < p.Sq) {
         const int64_t obase = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                const float val = (l_tot == 0.0f) ? __builtin_nanf("") : o[db][r] * inv;
+                const float val = dead ? __builtin_nanf("") : o[db][r] * inv;
                 if (p.out_f32) ((float *)p.out)[obase + dim * p.os[3]] = val;
                 else ((T *)p.out)[obase + dim * p.os[3]] = from_float<T>(val);
             }
@@ -295,10 +527,15 @@ static int launch_t(const AttnParams &p, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     dim3 grid((unsigned)blocks), block(64 * PF_WAVES);
+    // rows of the output can be written in 16-byte pieces when they are contiguous and aligned
+    const int oeb = p.out_f32 ? 4 : 2;
+    int out_vec = (p.os[3] == 1 || p.D == 1) && ((uintptr_t)p.out % 16 == 0);
+    for (int i = 0; i < 3; i++)
+        if ((p.os[i] * oeb) % 16 != 0) out_vec = 0;
     switch (p.D) {
-        case 64: hipLaunchKernelGGL((prefill_mfma_kernel<T, 64>), grid, block, 0, stream, p, nqb); break;
-        case 96: hipLaunchKernelGGL((prefill_mfma_kernel<T, 96>), grid, block, 0, stream, p, nqb); break;
-        case 128: hipLaunchKernelGGL((prefill_mfma_kernel<T, 128>), grid, block, 0, stream, p, nqb); break;
+        case 64: hipLaunchKernelGGL((prefill_mfma_kernel<T, 64>), grid, block, 0, stream, p, nqb, out_vec); break;
+        case 96: hipLaunchKernelGGL((prefill_mfma_kernel<T, 96>), grid, block, 0, stream, p, nqb, out_vec); break;
+        case 128: hipLaunchKernelGGL((prefill_mfma_kernel<T, 128>), grid, block, 0, stream, p, nqb, out_vec); break;
         default: set_error("prefill MFMA kernel: head_dim %d not in {64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
