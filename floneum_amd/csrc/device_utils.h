@@ -57,7 +57,13 @@ __device__ __forceinline__ void wave_lds_sync() {
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory
 // counter, i.e. it waits for every global load in flight, which would serialise a tile prefetch
 // with the math it is meant to overlap.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// The scheduling fences keep register-only work (e.g. a softmax tail) from drifting across the
+// barrier into the neighbouring phase.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
