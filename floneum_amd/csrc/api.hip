@@ -558,9 +558,6 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     fill_params(args, &p);
     FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
-#ifdef EXP_TRACE
-    p.partials = (float *)args->workspace;
-#endif
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;

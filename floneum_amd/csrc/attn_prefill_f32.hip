@@ -124,9 +124,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     if (j_begin < hi_wg) load_tile(j_begin);
 
     for (int j0 = j_begin; j0 < hi_wg; j0 += PF32_BN) {
-        __syncthreads();
-        store_tile();
-        __syncthreads();
+        lds_barrier();  // everyone finished reading the previous tile (LDS-only barrier: the prefetch
+        store_tile();   // issued below stays in flight across the math)
+        lds_barrier();
         if (j0 + PF32_BN < hi_wg) load_tile(j0 + PF32_BN);
 
         const bool tile_visible = wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;

@@ -111,11 +111,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int lane = tid & 63;
     const int ln = lane & 31;      // query column / key row owned inside a 32-wide MFMA block
     const int h2 = lane >> 5;      // which half of the contraction slice
-#ifdef EXP_FLIP
-    const int group = 1 - (wave >> 2);
-#else
     const int group = wave >> 2;   // wavefronts w and w + 4 share a SIMD and run out of phase
-#endif
 
     // workgroup -> (query block, batch, head): long query blocks first, and heads laid out so
     // the workgroups that land on one XCD (id % 8) share a KV head whenever H is a multiple of 8
@@ -191,11 +187,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // tiles, each during its own vector phase (the matrix-phase wavefronts do nothing but MFMA work).
     uint4_t st[C::NCH];
     int gofs[C::NCH], lofs[C::NCH];  // per-thread global / LDS byte offsets of its chunks
-#ifdef EXP_SWAP
-    const bool moves_k = group == 0;
-#else
     const bool moves_k = group == 1;
-#endif
     const int mrow_bytes = moves_k ? krow_bytes : vrow_bytes;
     const __amdgpu_buffer_rsrc_t mrs = moves_k ? krs : vrs;
 #pragma unroll
@@ -373,10 +365,6 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                 l = packed_pair_sum<T>(pk[t][r >> 1], l);  // the rounded values the MFMA will use
             }
     };
-    auto tile_visible = [&](int i) __attribute__((always_inline)) {
-        const int j0 = j_begin + i * PF_BN;
-        return i >= 0 && i < ntiles && wave_has_rows && j0 < hi_w && j0 + PF_BN > lo_w;
-    };
 
     // ---- slot schedule ---------------------------------------------------------------------------------
     // Slots are separated by workgroup barriers.  Group 0 is in its matrix phase in even slots and in
@@ -398,66 +386,32 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // MODE bit 0: S^T of tile i; bit 1: P.V of tile i-1; bit 2: softmax of tile i (group 0) / i-1 (group 1)
     auto matrix_phase = [&](int i, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
-#ifndef EXP_PRIO_M
-#define EXP_PRIO_M 1
-#endif
-        __builtin_amdgcn_s_setprio(EXP_PRIO_M);
-#ifndef EXP_NO_MFMA
+        __builtin_amdgcn_s_setprio(1);
         if constexpr ((MODE & 3) == 3) pv_qk(i - 1, i);
         else if constexpr ((MODE & 3) == 2) pv(i - 1);
         else if constexpr ((MODE & 3) == 1) qk(i);
-#endif
         __builtin_amdgcn_s_setprio(0);
     };
     auto vector_phase = [&](int i, int tile_to_store, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
         store_tile(tile_to_store);
         load_tile(tile_to_store + 1);
-#ifndef EXP_NO_SOFTMAX
         if constexpr ((MODE & 4) != 0) softmax(i);
-#endif
     };
-#ifdef EXP_TRACE
-    long long *trace = (long long *)p.partials;
-    const bool tracing = trace && blockIdx.x == 8 && lane == 0;
-#define TRACE_AT(slot, k) if (tracing && (slot) < 300) trace[(wave * 300 + (slot)) * 4 + (k)] = clock64();
-#else
-#define TRACE_AT(slot, k)
-#endif
     auto segment0 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 0: slot 2i matrix, slot 2i+1 vector + V(i)
         for (int i = i0; i < i1; i++) {
-            TRACE_AT(2 * i, 0)
             matrix_phase(i, mode);
-            TRACE_AT(2 * i, 1)
             lds_barrier();
-            TRACE_AT(2 * i, 2)
-            TRACE_AT(2 * i + 1, 0)
-#ifdef EXP_SWAP
-            vector_phase(i, i + 1, mode);
-#else
             vector_phase(i, i, mode);
-#endif
-            TRACE_AT(2 * i + 1, 1)
             lds_barrier();
-            TRACE_AT(2 * i + 1, 2)
         }
     };
     auto segment1 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 1: slot 2i vector (tile i-1) + K(i+1), slot 2i+1 matrix
         for (int i = i0; i < i1; i++) {
-            TRACE_AT(2 * i, 0)
-#ifdef EXP_SWAP
-            vector_phase(i - 1, i, mode);
-#else
             vector_phase(i - 1, i + 1, mode);
-#endif
-            TRACE_AT(2 * i, 1)
             lds_barrier();
-            TRACE_AT(2 * i, 2)
-            TRACE_AT(2 * i + 1, 0)
             matrix_phase(i, mode);
-            TRACE_AT(2 * i + 1, 1)
             lds_barrier();
-            TRACE_AT(2 * i + 1, 2)
         }
     };
     using std::integral_constant;
@@ -482,41 +436,6 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                 segment0(ia, ntiles + 1, integral_constant<int, 0>{});
             }
         } else {
-#ifdef EXP_SAMELOOP
-            // same loop as group 0, one slot later: slot 2i+1 matrix(i), slot 2i+2 vector(i) + K(i+2)
-            auto segment1b = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {
-                for (int i = i0; i < i1; i++) {
-                    TRACE_AT(2 * i + 1, 0)
-                    matrix_phase(i, mode);
-                    TRACE_AT(2 * i + 1, 1)
-                    lds_barrier();
-                    TRACE_AT(2 * i + 1, 2)
-                    TRACE_AT(2 * i + 2, 0)
-                    vector_phase(i, i + 2, mode);
-                    TRACE_AT(2 * i + 2, 1)
-                    lds_barrier();
-                    TRACE_AT(2 * i + 2, 2)
-                }
-            };
-            // slot 0: vector phase with nothing to do but move K(1)
-            store_tile(1);
-            load_tile(2);
-            lds_barrier();
-            segment1b(0, ia, integral_constant<int, 0>{});
-            if (ia < ib) {
-                segment1b(ia, ia + 1, integral_constant<int, 1 | 4>{});
-                segment1b(ia + 1, ib, integral_constant<int, 1 | 2 | 4>{});
-                if (ib < ntiles) {
-                    segment1b(ib, ib + 1, integral_constant<int, 2>{});
-                    segment1b(ib + 1, ntiles, integral_constant<int, 0>{});
-                } else {
-                    matrix_phase(ntiles, integral_constant<int, 2>{});  // last slot: P.V of the last tile
-                }
-            } else {
-                segment1b(ia, ntiles, integral_constant<int, 0>{});
-            }
-            lds_barrier();  // last slot 2 ntiles + 1
-#else
             // iteration i: softmax(i-1), then S^T(i) and P.V(i-1)
             segment1(0, ia, integral_constant<int, 0>{});
             if (ia < ib) {
@@ -527,7 +446,6 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             } else {
                 segment1(ia, ntiles + 1, integral_constant<int, 0>{});
             }
-#endif
         }
     }
 
