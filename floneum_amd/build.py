@@ -38,6 +38,13 @@ def build(verbose=True):
     if os.path.exists(STATIC):
         os.remove(STATIC)
     subprocess.check_call(["ar", "rcs", STATIC] + objs)
+    # the C++ host mirror's test program (runs on the GPU box, started by tests/test_host_mirror_gpu.py)
+    root = os.path.dirname(HERE)
+    cpp = os.path.join(root, "tests", "cpp", "test_host_mirror.cpp")
+    if os.path.exists(cpp):
+        subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(root, "include"), cpp,
+                               "-o", os.path.join(root, "tests", "cpp", "test_host_mirror"),
+                               "-L", HERE, "-lfusor_hip", "-Wl,-rpath,$ORIGIN/../../floneum_amd"])
     if verbose:
         print(f"built {LIB}")
     return LIB

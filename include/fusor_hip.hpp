@@ -1,0 +1,346 @@
+// fusor_hip.hpp -- C++ host side above the C ABI of fusor_hip.h.
+//
+// Header-only mirror of the fusor types that sit on the attention path, with the reference's
+// names, argument order and failure behaviour, so code written against
+//     fusor::Tensor<4, D>::flash_attention(&k, &v, scale, Option<(&mask, MaskKind)>)
+//                                   fusor-ml/fusor/src/composite/flash_attention.rs:52-73
+//     fusor::cache::{AttentionMask, MaskCache, KvCache}
+//                                   fusor-ml/fusor/src/cache/{attention_mask,mask_cache,kv_cache}.rs
+// reads the same here.  Where the reference panics (assert!/panic!) these functions throw
+// fusor_hip::Panic carrying the reference's message; HIP failures throw fusor_hip::GpuError (the
+// reference's fusor::Error::Gpu, fusor-ml/fusor/src/lib.rs:391-403).
+// Tensors are reference-counted views {buffer, offset, shape, strides} in element units
+// (fusor-ml/types/src/layout.rs:88-129); layout operations never copy.
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "fusor_hip.h"
+
+namespace fusor_hip {
+
+struct Panic : std::logic_error {
+    using std::logic_error::logic_error;
+};
+struct GpuError : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+inline void check(int status) {
+    if (status == FHIP_OK) return;
+    const std::string msg = fhip_last_error();
+    if (status == FHIP_ERR_INVALID_ARG) throw Panic(msg);
+    throw GpuError(msg);
+}
+
+enum class DType { F32 = FHIP_F32, F16 = FHIP_F16, BF16 = FHIP_BF16 };
+inline size_t dtype_bytes(DType d) { return d == DType::F32 ? 4 : 2; }
+
+/// fusor::MaskKind (flash_attention.rs:11-19)
+enum class MaskKind { QKMask = FHIP_MASK_QK, BatchKeyMask = FHIP_MASK_BATCH_KEY };
+
+/// One GPU plus one stream.  Cheap to copy (shared handle), like fusor's Device.
+class Device {
+    struct Inner {
+        fhip_device *dev = nullptr;
+        fhip_stream *stream = nullptr;
+        fhip_device_info info{};
+        void *workspace = nullptr;
+        size_t workspace_bytes = 0;
+        ~Inner() {
+            if (workspace) fhip_free(dev, workspace);
+            if (stream) fhip_stream_destroy(stream);
+            if (dev) fhip_device_destroy(dev);
+        }
+    };
+    std::shared_ptr<Inner> in_;
+
+   public:
+    explicit Device(int ordinal = 0) : in_(std::make_shared<Inner>()) {
+        check(fhip_device_create(ordinal, &in_->dev));
+        check(fhip_stream_create(in_->dev, &in_->stream));
+        check(fhip_device_get_info(in_->dev, &in_->info));
+    }
+    fhip_device *handle() const { return in_->dev; }
+    fhip_stream *stream() const { return in_->stream; }
+    const fhip_device_info &info() const { return in_->info; }
+    void synchronize() const { check(fhip_stream_synchronize(in_->stream)); }
+    bool same(const Device &o) const { return in_ == o.in_; }
+    /// grow-only scratch for the split-KV decode (the caller of the C ABI owns the workspace)
+    void *workspace(size_t bytes) const {
+        if (bytes > in_->workspace_bytes) {
+            if (in_->workspace) {
+                synchronize();
+                check(fhip_free(in_->dev, in_->workspace));
+                in_->workspace = nullptr;
+            }
+            check(fhip_malloc(in_->dev, bytes, &in_->workspace));
+            in_->workspace_bytes = bytes;
+        }
+        return in_->workspace;
+    }
+    size_t workspace_bytes() const { return in_->workspace_bytes; }
+};
+
+/// Owning device allocation, freed with the last tensor that views it.
+class Buffer {
+    Device dev_;
+    void *ptr_ = nullptr;
+    bool owned_ = true;
+
+   public:
+    Buffer(const Device &dev, size_t bytes) : dev_(dev) { check(fhip_malloc(dev.handle(), bytes, &ptr_)); }
+    Buffer(const Device &dev, void *borrowed) : dev_(dev), ptr_(borrowed), owned_(false) {}
+    Buffer(const Buffer &) = delete;
+    Buffer &operator=(const Buffer &) = delete;
+    ~Buffer() {
+        if (owned_ && ptr_) fhip_free(dev_.handle(), ptr_);
+    }
+    void *ptr() const { return ptr_; }
+    const Device &device() const { return dev_; }
+};
+
+/// Rank-R strided view of device memory.
+template <int R>
+class Tensor {
+    std::shared_ptr<Buffer> buf_;
+    std::shared_ptr<void> keepalive_;  // e.g. the KV cache that owns a borrowed buffer
+    DType dtype_ = DType::F32;
+    uint64_t offset_ = 0;
+    uint32_t shape_[R]{};
+    int64_t stride_[R]{};
+
+   public:
+    Tensor() = default;
+    Tensor(std::shared_ptr<Buffer> buf, DType dt, const uint32_t (&shape)[R], const int64_t *strides = nullptr,
+           uint64_t offset = 0, std::shared_ptr<void> keepalive = nullptr)
+        : buf_(std::move(buf)), keepalive_(std::move(keepalive)), dtype_(dt), offset_(offset) {
+        int64_t acc = 1;
+        for (int i = R - 1; i >= 0; i--) {
+            shape_[i] = shape[i];
+            stride_[i] = strides ? strides[i] : acc;
+            acc *= shape[i];
+        }
+    }
+    /// Tensor::zeros-like allocation without initialisation (the kernels overwrite it)
+    static Tensor empty(const Device &dev, DType dt, const uint32_t (&shape)[R]) {
+        size_t n = 1;
+        for (int i = 0; i < R; i++) n *= shape[i];
+        return Tensor(std::make_shared<Buffer>(dev, n * dtype_bytes(dt)), dt, shape);
+    }
+    /// Tensor::from_slice: uploads contiguous host elements of the tensor's dtype
+    static Tensor from_slice(const Device &dev, DType dt, const uint32_t (&shape)[R], const void *host) {
+        Tensor t = empty(dev, dt, shape);
+        check(fhip_memcpy_h2d(dev.stream(), t.buf_->ptr(), host, t.numel() * dtype_bytes(dt)));
+        return t;
+    }
+    size_t numel() const {
+        size_t n = 1;
+        for (int i = 0; i < R; i++) n *= shape_[i];
+        return n;
+    }
+    const uint32_t *shape() const { return shape_; }
+    const int64_t *strides() const { return stride_; }
+    uint64_t offset() const { return offset_; }
+    DType dtype() const { return dtype_; }
+    const Device &device() const { return buf_->device(); }
+    void *data() const { return buf_->ptr(); }
+    bool is_contiguous() const {
+        int64_t acc = 1;
+        for (int i = R - 1; i >= 0; i--) {
+            if (shape_[i] != 1 && stride_[i] != acc) return false;
+            acc *= shape_[i];
+        }
+        return true;
+    }
+    /// Layout::transpose (types/src/layout.rs): swaps two dimensions, no copy
+    Tensor transpose(int a, int b) const {
+        Tensor t = *this;
+        std::swap(t.shape_[a], t.shape_[b]);
+        std::swap(t.stride_[a], t.stride_[b]);
+        return t;
+    }
+    /// Layout::narrow: a window along one dimension, no copy
+    Tensor narrow(int dim, uint32_t start, uint32_t len) const {
+        if (start + (uint64_t)len > shape_[dim]) throw Panic("narrow out of range");
+        Tensor t = *this;
+        t.shape_[dim] = len;
+        t.offset_ += (uint64_t)start * (uint64_t)stride_[dim];
+        return t;
+    }
+    /// as_slice().await: contiguous readback of this view (synchronises the stream)
+    void to_host(void *host) const {
+        if (!is_contiguous()) throw Panic("to_host needs a contiguous view");
+        const size_t eb = dtype_bytes(dtype_);
+        check(fhip_memcpy_d2h(device().stream(), host, (const char *)buf_->ptr() + offset_ * eb, numel() * eb));
+    }
+
+    fhip_tensor4 c4() const {
+        static_assert(R == 4, "rank-4 only");
+        fhip_tensor4 t{};
+        t.ptr = buf_->ptr();
+        t.offset = offset_;
+        for (int i = 0; i < 4; i++) {
+            t.shape[i] = shape_[i];
+            t.stride[i] = stride_[i];
+        }
+        return t;
+    }
+    fhip_tensor2 c2() const {
+        static_assert(R == 2, "rank-2 only");
+        fhip_tensor2 t{};
+        t.ptr = buf_->ptr();
+        t.offset = offset_;
+        for (int i = 0; i < 2; i++) {
+            t.shape[i] = shape_[i];
+            t.stride[i] = stride_[i];
+        }
+        return t;
+    }
+
+    /// fusor::Tensor<4,D>::flash_attention(&self, k, v, scale, mask) -> Self
+    /// (fusor flash_attention.rs:52-73).  `analytic` is the extension MaskCache::get_analytic hands
+    /// out when it built the mask itself; it replaces the dense mask tensor.
+    Tensor flash_attention(const Tensor &k, const Tensor &v, float scale,
+                           std::optional<std::pair<const Tensor<2> *, MaskKind>> mask = std::nullopt,
+                           const fhip_analytic_mask *analytic = nullptr, const int32_t *kv_lens = nullptr) const {
+        static_assert(R == 4, "flash_attention takes rank-4 tensors");
+        if (!device().same(k.device()) || !device().same(v.device()))
+            throw Panic("Cannot mix tensors of different devices");  // fusor lib.rs:265
+        fhip_attn_args a{};
+        Tensor out = empty(device(), dtype_, shape_);  // fresh, contiguous, Q's shape (core :505-507)
+        a.q = c4();
+        a.k = k.c4();
+        a.v = v.c4();
+        a.out = out.c4();
+        a.dtype = a.out_dtype = (fhip_dtype)dtype_;
+        a.scale = scale;
+        if (mask) {
+            if (!device().same(mask->first->device()))
+                throw Panic("Mask must be on the same device as other tensors");  // fusor flash_attention.rs:64
+            a.mask = mask->first->c2();
+            a.mask_kind = (fhip_mask_kind)mask->second;
+        }
+        if (analytic) a.analytic = *analytic;
+        a.kv_lens = kv_lens;
+        size_t need = 0;
+        check(fhip_flash_attention_workspace_bytes(&a, device().info().compute_units, &need));
+        if (need) {
+            a.workspace = device().workspace(need);
+            a.workspace_bytes = device().workspace_bytes();
+        }
+        check(fhip_flash_attention(device().stream(), &a));
+        return out;
+    }
+
+    template <int>
+    friend class Tensor;
+    friend class KvCache;
+};
+
+/// fusor::cache::AttentionMask (attention_mask.rs:9-83)
+class AttentionMask {
+    Tensor<2> mask_;
+    std::optional<fhip_analytic_mask> analytic_;
+
+   public:
+    AttentionMask() = default;
+    explicit AttentionMask(Tensor<2> mask, std::optional<fhip_analytic_mask> analytic = std::nullopt)
+        : mask_(std::move(mask)), analytic_(analytic) {}
+    /// AttentionMask::causal(device, seq_len): mask[i][j] = -inf if j > i else 0
+    static AttentionMask causal(const Device &dev, uint32_t seq_len, DType dt = DType::F32) {
+        std::vector<char> host((size_t)seq_len * seq_len * dtype_bytes(dt));
+        check(fhip_mask_causal((fhip_dtype)dt, seq_len, host.data()));
+        const uint32_t shape[2] = {seq_len, seq_len};
+        fhip_analytic_mask am{1, 1, 0, 0};
+        return AttentionMask(Tensor<2>::from_slice(dev, dt, shape, host.data()), am);
+    }
+    const Tensor<2> &mask() const { return mask_; }
+    const std::optional<fhip_analytic_mask> &analytic() const { return analytic_; }
+};
+
+/// fusor::cache::MaskCache (mask_cache.rs:9-116): base masks cached by (seq_len, window)
+class MaskCache {
+    DType dtype_;
+    std::map<std::pair<uint32_t, int64_t>, AttentionMask> masks_;
+
+   public:
+    explicit MaskCache(DType dt = DType::F32) : dtype_(dt) {}
+    /// get_mask(seq_len, seqlen_offset, sliding_window_size, device)
+    AttentionMask get_mask(uint32_t seq_len, uint64_t seqlen_offset, std::optional<uint64_t> sliding_window_size,
+                           const Device &dev) {
+        const int has_w = sliding_window_size.has_value();
+        const uint64_t w = has_w ? *sliding_window_size : 0;
+        uint32_t rows;
+        uint64_t cols;
+        check(fhip_mask_get_mask_shape(seq_len, seqlen_offset, has_w, w, &rows, &cols));
+        fhip_analytic_mask am{};
+        const bool have_am = fhip_mask_get_analytic(seq_len, seqlen_offset, has_w, w, &am) == FHIP_OK;
+        const auto key = std::make_pair(seq_len, has_w ? (int64_t)w : (int64_t)-1);
+        auto it = masks_.find(key);
+        if (it == masks_.end()) {
+            std::vector<char> host((size_t)seq_len * seq_len * dtype_bytes(dtype_));
+            if (has_w) check(fhip_mask_sliding_window((fhip_dtype)dtype_, seq_len, w, host.data()));
+            else check(fhip_mask_causal((fhip_dtype)dtype_, seq_len, host.data()));
+            const uint32_t shape[2] = {seq_len, seq_len};
+            it = masks_.emplace(key, AttentionMask(Tensor<2>::from_slice(dev, dtype_, shape, host.data()))).first;
+        }
+        std::optional<fhip_analytic_mask> oam;
+        if (have_am) oam = am;
+        if (cols > seq_len) {  // left padding with zeros (mask_cache.rs:73-85)
+            std::vector<char> host((size_t)rows * cols * dtype_bytes(dtype_));
+            check(fhip_mask_get_mask((fhip_dtype)dtype_, seq_len, seqlen_offset, has_w, w, host.data()));
+            const uint32_t shape[2] = {rows, (uint32_t)cols};
+            return AttentionMask(Tensor<2>::from_slice(dev, dtype_, shape, host.data()), oam);
+        }
+        return AttentionMask(it->second.mask(), oam);
+    }
+};
+
+/// fusor::cache::KvCache over device memory (kv_cache.rs:13-68, tensor_cache.rs:9-124)
+class KvCache {
+    struct Inner {
+        fhip_kv_cache *c = nullptr;
+        ~Inner() {
+            if (c) fhip_kv_cache_destroy(c);
+        }
+    };
+    std::shared_ptr<Inner> in_;
+    Device dev_;
+    DType dtype_;
+
+   public:
+    /// KvCache::new(concat_dim, max_sequence_len); the device cache concatenates along dim 2
+    KvCache(const Device &dev, int concat_dim, uint64_t max_sequence_len, DType dt = DType::F32)
+        : in_(std::make_shared<Inner>()), dev_(dev), dtype_(dt) {
+        if (concat_dim != 2) throw GpuError("the device KV cache concatenates [B, Hkv, seq, D] along dim 2");
+        check(fhip_kv_cache_create(dev.handle(), (fhip_dtype)dt, max_sequence_len, &in_->c));
+    }
+    void reset() { check(fhip_kv_cache_reset(in_->c)); }
+    uint64_t current_seq_len() const {
+        uint64_t n;
+        check(fhip_kv_cache_current_seq_len(in_->c, &n));
+        return n;
+    }
+    /// append(device, k, v) -> (keys, values) including the new rows
+    std::pair<Tensor<4>, Tensor<4>> append(const Device &, const Tensor<4> &k, const Tensor<4> &v) {
+        fhip_tensor4 kn = k.c4(), vn = v.c4(), ka{}, va{};
+        check(fhip_kv_cache_append(in_->c, dev_.stream(), &kn, &vn, &ka, &va));
+        auto wrap = [&](const fhip_tensor4 &t) {
+            Tensor<4> r(std::make_shared<Buffer>(dev_, t.ptr), dtype_, t.shape, t.stride, t.offset, in_);
+            return r;
+        };
+        return {wrap(ka), wrap(va)};
+    }
+};
+
+}  // namespace fusor_hip

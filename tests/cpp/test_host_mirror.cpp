@@ -1,0 +1,146 @@
+// Runs on the GPU box: the C++ host mirror (include/fusor_hip.hpp) exercised with the inputs and
+// assertions of the reference's own tests.
+//   fusor-ml/fusor/src/composite/flash_attention.rs:207-358  (attention, CPU arm tests)
+//   fusor-ml/fusor/src/cache/attention_mask.rs:88-111        (causal mask)
+//   fusor-ml/fusor/src/cache/mask_cache.rs:122-175           (mask cache)
+//   fusor-ml/fusor/src/cache/kv_cache.rs:74-157, tensor_cache.rs:130-186  (KV cache)
+#include <cmath>
+#include <cstdio>
+#include <limits>
+#include <vector>
+
+#include "fusor_hip.hpp"
+
+using namespace fusor_hip;
+static int failures = 0;
+#define EXPECT(cond, ...)                                             \
+    do {                                                              \
+        if (!(cond)) {                                                \
+            failures++;                                               \
+            printf("FAIL %s:%d: %s : ", __FILE__, __LINE__, #cond);   \
+            printf(__VA_ARGS__);                                      \
+            printf("\n");                                             \
+        }                                                             \
+    } while (0)
+
+static const float NEG_INF = -std::numeric_limits<float>::infinity();
+
+static Tensor<4> t4(const Device &d, std::vector<float> v, uint32_t a, uint32_t b, uint32_t c, uint32_t e) {
+    const uint32_t shape[4] = {a, b, c, e};
+    return Tensor<4>::from_slice(d, DType::F32, shape, v.data());
+}
+static std::vector<float> host(const Tensor<4> &t) {
+    std::vector<float> h(t.numel());
+    t.to_host(h.data());
+    return h;
+}
+static std::vector<float> host2(const Tensor<2> &t) {
+    std::vector<float> h(t.numel());
+    t.to_host(h.data());
+    return h;
+}
+
+static void test_flash_attention_cpu(const Device &d) {  // flash_attention.rs:207-239
+    auto q = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), k = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), v = t4(d, {1, 2, 3, 4}, 1, 1, 2, 2);
+    auto out = q.flash_attention(k, v, 1.0f / std::sqrt(2.0f));
+    EXPECT(out.shape()[0] == 1 && out.shape()[1] == 1 && out.shape()[2] == 2 && out.shape()[3] == 2, "shape");
+    for (float x : host(out)) EXPECT(std::isfinite(x), "non-finite %f", x);
+}
+
+static void test_flash_attention_cpu_with_mask(const Device &d) {  // :241-276
+    auto q = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), k = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), v = t4(d, {1, 2, 3, 4}, 1, 1, 2, 2);
+    const float m[4] = {0, NEG_INF, 0, 0};
+    const uint32_t ms[2] = {2, 2};
+    auto mask = Tensor<2>::from_slice(d, DType::F32, ms, m);
+    auto out = host(q.flash_attention(k, v, 1.0f / std::sqrt(2.0f), std::make_pair(&mask, MaskKind::QKMask)));
+    EXPECT(std::fabs(out[0] - 1.0f) < 0.01f, "row 0 should equal V[0]: %f", out[0]);
+    EXPECT(std::fabs(out[1] - 2.0f) < 0.01f, "row 0 should equal V[0]: %f", out[1]);
+}
+
+static void test_flash_attention_gqa_cpu(const Device &d) {  // :278-313
+    std::vector<float> q(16), k(8), v(8);
+    for (int i = 0; i < 16; i++) q[i] = i * 0.1f;
+    for (int i = 0; i < 8; i++) k[i] = i * 0.1f + 1.0f, v[i] = i * 0.1f + 2.0f;
+    auto out = t4(d, q, 1, 4, 2, 2).flash_attention(t4(d, k, 1, 2, 2, 2), t4(d, v, 1, 2, 2, 2), 1.0f / std::sqrt(2.0f));
+    EXPECT(out.shape()[1] == 4, "output keeps Q's head count");
+    for (float x : host(out)) EXPECT(std::isfinite(x), "non-finite %f", x);
+    // Q heads (3) not divisible by K/V heads (2): the reference asserts (:94-99)
+    bool threw = false;
+    try {
+        t4(d, std::vector<float>(12, 0.f), 1, 3, 2, 2).flash_attention(t4(d, k, 1, 2, 2, 2), t4(d, v, 1, 2, 2, 2), 1.0f);
+    } catch (const Panic &e) {
+        threw = std::string(e.what()) == "Number of Q heads (3) must be divisible by number of K/V heads (2)";
+    }
+    EXPECT(threw, "divisibility panic with the reference's message");
+}
+
+static void test_flash_attention_cpu_with_batch_key_mask(const Device &d) {  // :315-358
+    std::vector<float> q(12), k(12), v(12);
+    for (int i = 0; i < 12; i++) q[i] = i * 0.1f, k[i] = i * 0.1f + 1.0f, v[i] = i * 0.1f + 2.0f;
+    const float m[6] = {0, 0, 0, 0, 0, NEG_INF};
+    const uint32_t ms[2] = {2, 3};
+    auto mask = Tensor<2>::from_slice(d, DType::F32, ms, m);
+    auto out = t4(d, q, 2, 1, 3, 2).flash_attention(t4(d, k, 2, 1, 3, 2), t4(d, v, 2, 1, 3, 2), 1.0f / std::sqrt(2.0f),
+                                                    std::make_pair(&mask, MaskKind::BatchKeyMask));
+    EXPECT(out.shape()[0] == 2 && out.shape()[2] == 3, "shape");
+    for (float x : host(out)) EXPECT(std::isfinite(x), "non-finite %f", x);
+}
+
+static void test_attention_mask_causal(const Device &d) {  // attention_mask.rs:88-111
+    auto m = host2(AttentionMask::causal(d, 3).mask());
+    const float want[9] = {0, NEG_INF, NEG_INF, 0, 0, NEG_INF, 0, 0, 0};
+    for (int i = 0; i < 9; i++) EXPECT(m[i] == want[i], "causal[%d] = %f", i, m[i]);
+}
+
+static void test_mask_cache(const Device &d) {  // mask_cache.rs:122-175
+    MaskCache cache;
+    EXPECT(cache.get_mask(3, 0, std::nullopt, d).mask().shape()[0] == 3, "3x3");
+    EXPECT(cache.get_mask(5, 0, std::nullopt, d).mask().shape()[1] == 5, "5x5");
+    auto padded = cache.get_mask(2, 3, std::nullopt, d);
+    EXPECT(padded.mask().shape()[0] == 2 && padded.mask().shape()[1] == 5, "offset pads to [2, 5]");
+    auto sw = cache.get_mask(4, 0, 2, d);
+    auto m = host2(sw.mask());
+    auto at = [&](int i, int j) { return m[i * 4 + j]; };
+    EXPECT(at(0, 0) == 0 && at(0, 1) == NEG_INF && at(1, 0) == 0 && at(1, 1) == 0, "rows 0-1");
+    EXPECT(at(2, 0) == NEG_INF && at(2, 1) == 0 && at(2, 2) == 0, "row 2");
+    EXPECT(at(3, 1) == NEG_INF && at(3, 2) == 0 && at(3, 3) == 0, "row 3");
+}
+
+static void test_kv_cache(const Device &d) {  // kv_cache.rs:74-157, tensor_cache.rs:130-186
+    KvCache cache(d, 2, 3);
+    auto k1 = t4(d, {1, 2}, 1, 1, 1, 2), v1 = t4(d, {5, 6}, 1, 1, 1, 2);
+    auto r1 = cache.append(d, k1, v1);
+    EXPECT(r1.first.shape()[2] == 1 && cache.current_seq_len() == 1, "first append stores the tensor");
+    auto k2 = t4(d, {3, 4}, 1, 1, 1, 2), v2 = t4(d, {7, 8}, 1, 1, 1, 2);
+    auto r2 = cache.append(d, k2, v2);
+    EXPECT(r2.first.shape()[2] == 2 && cache.current_seq_len() == 2, "second append");
+    auto kh = host(r2.first), vh = host(r2.second);
+    EXPECT(kh[0] == 1 && kh[1] == 2 && kh[2] == 3 && kh[3] == 4, "keys 1 2 3 4");
+    EXPECT(vh[0] == 5 && vh[3] == 8, "values 5..8");
+    // growth beyond max_sequence_len keeps the last positions (tensor_cache.rs:55-78)
+    auto k3 = t4(d, {9, 10, 11, 12}, 1, 1, 2, 2), v3 = t4(d, {13, 14, 15, 16}, 1, 1, 2, 2);
+    auto r3 = cache.append(d, k3, v3);
+    EXPECT(r3.first.shape()[2] == 3 && cache.current_seq_len() == 3, "truncated to max_sequence_len");
+    kh = host(r3.first);
+    EXPECT(kh[0] == 3 && kh[1] == 4 && kh[2] == 9 && kh[5] == 12, "last three positions kept");
+    cache.reset();
+    EXPECT(cache.current_seq_len() == 0, "reset");
+}
+
+int main() {
+    try {
+        Device d(0);
+        test_flash_attention_cpu(d);
+        test_flash_attention_cpu_with_mask(d);
+        test_flash_attention_gqa_cpu(d);
+        test_flash_attention_cpu_with_batch_key_mask(d);
+        test_attention_mask_causal(d);
+        test_mask_cache(d);
+        test_kv_cache(d);
+    } catch (const std::exception &e) {
+        printf("exception: %s\n", e.what());
+        return 2;
+    }
+    printf("%s (%d failures)\n", failures ? "FAILED" : "ok", failures);
+    return failures ? 1 : 0;
+}
