@@ -27,6 +27,9 @@ PEAK_HBM_GBS = 8000.0
 PEAK_MFMA_F16_TFLOPS = 2500.0
 PEAK_MFMA_F32_TFLOPS = 157.3
 SEED = 0xF10E0000
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# same counter reads for a 256 MiB copy (profiles/decode_splitkv_C2.txt, profiles/prefill_mfma_C3.txt)
+MEASURED_TRAFFIC_BYTES = {"C2": 270.2e6, "C3": 213.7e6}
 
 
 def configs():
@@ -289,7 +292,7 @@ def run_config(name, steps, warmup, with_cpu=True):
         value, unit = flops / (wall_ms * 1e-3) / 1e12, "TFLOP/s"
         roof = dict(bound="mfma", achieved=flops / (main_ms_mean * 1e-3) / 1e12, peak=peak, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
     roof["kernel"] = kernel
     roof["kernel_ms_mean"] = main_ms_mean
     roof["kernel_ms_median"] = main_ms_med
@@ -306,6 +309,20 @@ def run_config(name, steps, warmup, with_cpu=True):
     return res
 
 
+def calibration_copy(mib=256, reps=3):
+    """A first KvCache.append is a plain copy of the appended tensor: reads `mib` MiB, writes `mib` MiB."""
+    import floneum_amd as fa
+    dev = fa.Device.default()
+    rows = mib * (1 << 20) // (2 * 128)  # f16 rows of 128 elements
+    src = fa.Tensor.empty(dev, (1, 1, rows, 128), fa.F16)
+    fa.check(fa.lib().fhip_memset(dev.stream, ctypes.c_void_p(src.buffer.ptr), 0, rows * 256))
+    for _ in range(reps):
+        cache = fa.KvCache(2, rows, fa.F16, dev)
+        cache.append(dev, src, src)  # keys and values: two copies of `mib` MiB each
+        dev.synchronize()
+        del cache
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -314,6 +331,10 @@ def main():
     ap.add_argument("--config", default="C2", choices=sorted(configs()))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (prefill C3) figure")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (the KV-cache row copy kernel) three times, so a "
+                         "rocprofv3 --pmc run of this command has a kernel of known traffic to scale FETCH_SIZE / "
+                         "WRITE_SIZE with")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build runs on exactly one GPU (no sharding, no collectives); --gpus {a.gpus} is "
@@ -321,6 +342,8 @@ def main():
         sys.exit(2)
 
     main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
+    if a.calibration_copy:
+        calibration_copy()
     line = {"metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": a.steps,
             "warmup": a.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (seeded SplitMix64 normals)",
