@@ -354,7 +354,9 @@ def main():
         line["cpu_baseline"] = main_res["cpu_baseline"]
     if not a.no_extra and a.config == "C2":
         # the other half of the metric: C3 prefill on the matrix cores
-        pre = run_config("C3", max(5, a.steps // 5), max(2, a.warmup // 5), with_cpu=not a.no_cpu)
+        # the shader clock needs some tens of milliseconds of matrix load to settle: warm the prefill
+        # leg up for longer than the (much shorter) decode steps need
+        pre = run_config("C3", max(20, a.steps // 2), max(100, a.warmup), with_cpu=not a.no_cpu)
         line["prefill"] = {k: pre[k] for k in ("value", "unit", "ms_per_step", "roofline", "config", "dtype",
                                                "frac_of_roofline", "spot_check_max_abs_err") if k in pre}
         if "cpu_baseline" in pre:

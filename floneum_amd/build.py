@@ -11,7 +11,7 @@ SOURCES = ["api.hip", "attn_generic.hip", "attn_decode.hip", "attn_prefill_mfma.
 LIB = os.path.join(HERE, "libfusor_hip.so")
 STATIC = os.path.join(HERE, "libfusor_hip.a")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Wall", "-Wno-unused-function",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
          # packed-f32 VALU forms are kept out of the generated code on purpose
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

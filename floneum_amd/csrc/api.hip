@@ -181,7 +181,9 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     if (a->dtype == FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
     if (!(D == 64 || D == 96 || D == 128)) return false;
-    if (!(a->scale > 0.0f)) return false;
+    // the kernel folds scale * log2(e) into Q (rounded back to the input type): the factor must not
+    // be able to push a finite element out of range
+    if (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f)) return false;
     if (a->mask_kind != FHIP_MASK_NONE) return false;  // dense additive masks take the generic kernel
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
     // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv

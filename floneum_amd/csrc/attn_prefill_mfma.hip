@@ -1,20 +1,25 @@
 // Prefill attention for f16 / bf16 on the gfx950 matrix cores.
 //
 // Workgroup = 8 wavefronts = 256 query rows of one (batch, head); each wavefront owns 32 rows.
-// Keys/values are walked in tiles of 64 rows staged through double-buffered LDS.  Per tile and
-// wavefront:
+// Keys/values are walked in tiles of 64 rows that go from global memory straight into a three-stage
+// LDS ring (direct-to-LDS buffer loads, no staging registers).  Per tile and wavefront:
 //   S^T (64 keys x 32 queries)  = K_tile . Q^T      v_mfma_f32_32x32x16  (A = K from LDS, B = Q in registers)
+//   Q is multiplied by scale * log2(e) once, and the first MFMA of a tile takes -m (the running row
+//   maximum) as its C operand, so the accumulators come out as base-2 exponents relative to the
+//   maximum and go straight into exp2: no multiply or subtract per score
 //   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of
 //   it per 32-key block, so the row max / row sum are in-lane folds plus one exchange with the
-//   lane 32 away (v_permlane32_swap); the rescale of O is skipped while the running maximum moves
-//   by less than 2^8
+//   lane 32 away (v_permlane32_swap); the running maximum is only moved (and O rescaled) when a
+//   tile exceeds it by more than 2^8
 //   O^T (D x 32 queries)       += V_tile^T . P^T    A = V^T read from row-major LDS with the
 //   transposing LDS load ds_read_b64_tr_b16, B = P^T taken straight from the S^T accumulator
 //   registers (the contraction index is permuted identically on both operands)
 // The two wavefronts that share a SIMD (w and w + 4) run half a tile out of phase: while one is in
-// its matrix phase (P.V of the previous tile, then S^T of the current one) the other is in its
-// vector phase (softmax), so the MFMA pipe and the VALU are busy at the same time.  Phases are
-// separated by workgroup barriers; the tile loads ride on the same barriers.
+// its matrix phase (S^T of the current tile, then P.V of the previous one) the other is in its
+// vector phase (softmax, tile loads), so the MFMA pipe and the VALU are busy at the same time.
+// Phases are separated by workgroup barriers; the tile loads ride on the same barriers.  The vector
+// phase uses no dot-product instructions: on this chip they queue behind the MFMAs of the other
+// wavefront instead of running beside them.
 // All accumulation is f32; P is rounded to the input type for the second product.
 // Masking is analytic (causal with offset, sliding window, per-batch kv length, tail of the key
 // axis); key tiles that are invisible to the whole workgroup are never loaded, and tiles fully
@@ -49,6 +54,11 @@ struct Mma<half_t> {
         half2_t h = {(half_t)x, (half_t)y};
         return __builtin_bit_cast(uint32_t, h);
     }
+    static __device__ __forceinline__ vec8 scaled(vec8 q, float c) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = (half_t)((float)q[e] * c);
+        return q;
+    }
 };
 template <>
 struct Mma<bf16_t> {
@@ -57,18 +67,34 @@ struct Mma<bf16_t> {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ uint32_t pack2(float x, float y) {
-        return (uint32_t)from_float<bf16_t>(x).bits | ((uint32_t)from_float<bf16_t>(y).bits << 16);
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        const bf16x2_t h = {(__bf16)x, (__bf16)y};  // v_cvt_pk_bf16_f32: round to nearest even
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    static __device__ __forceinline__ vec8 scaled(vec8 q, float c) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = (__bf16)((float)q[e] * c);
+        return q;
     }
 };
 
+// LDS image of a 64-row tile.  Rows are kept in 16 groups of 4: row r sits in group r % 16 at
+// position r / 16.  A group is exactly what one wavefront-wide direct-to-LDS load writes (4 rows of
+// head_dim 16-bit values, contiguous), and groups are padded apart so that
+//   - the 16 rows a quarter-wavefront reads for the S^T operand (rows r .. r+15, same 16-byte
+//     column) fall 16 bytes apart modulo the 256-byte bank period            (K: pitch 8 D + 16)
+//   - the 4 rows x 64 bytes a half-wavefront reads with the transposing load fall 64 bytes apart
+//                                                                            (V: pitch 8 D + 64)
 template <int D>
 struct PfCfg {
-    static constexpr int KP = D * 2 + 16;                            // K tile row pitch, bytes
-    static constexpr int VP = (D == 64) ? 192 : 320;                 // V tile row pitch, bytes
-    static constexpr int K_BYTES = PF_BN * KP;
-    static constexpr int V_BYTES = PF_BN * VP;
+    static constexpr int ROWB = D * 2;                               // bytes per tile row
+    static constexpr int KG = 4 * ROWB + 16;                         // K group pitch, bytes
+    static constexpr int VG = 4 * ROWB + 64;                         // V group pitch, bytes
+    static constexpr int K_BYTES = 16 * KG;
+    static constexpr int V_BYTES = 16 * VG;
     static constexpr int CPR = D / 8;                                // 16-byte chunks per row
-    static constexpr int NCH = PF_BN * CPR / 256;                    // chunks per thread of the 4 moving wavefronts
+    static constexpr int LOAD_LANES = 4 * CPR;                       // lanes of a wavefront-wide tile load (<= 64)
+    static constexpr int NS = 3;                                     // tile stages in LDS
 };
 
 __device__ __forceinline__ float half_swap_max(float x) {
@@ -81,18 +107,6 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <typename T>
-__device__ __forceinline__ float packed_pair_sum(uint32_t pk, float acc);
-template <>
-__device__ __forceinline__ float packed_pair_sum<half_t>(uint32_t pk, float acc) {
-    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, pk), ones, acc, false);  // acc + lo + hi in f32
-}
-template <>
-__device__ __forceinline__ float packed_pair_sum<bf16_t>(uint32_t pk, float acc) {
-    return acc + __uint_as_float(pk << 16) + __uint_as_float(pk & 0xffff0000u);
-}
-
 // Rows whose running maximum is stale by at most this much (log2 domain) keep it: probabilities
 // then reach 2^8 at most, well inside f16/bf16 range, and the 64-register rescale of O is skipped
 // on almost every tile.
@@ -103,7 +117,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     typedef PfCfg<D> C;
     typedef typename Mma<T>::vec8 vec8;
     constexpr int STAGE = C::K_BYTES + C::V_BYTES;
-    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    constexpr int NS = C::NS;
+    __shared__ __attribute__((aligned(16))) char smem[NS * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     const int tid = threadIdx.x;
@@ -150,14 +165,17 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int klo = row_lo(qrow), khi = row_hi(qrow);               // this lane's row
     const bool wave_has_rows = qw0 < p.Sq;
 
-    // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel
+    // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel, already
+    // multiplied by scale * log2(e) (rounded back to the input type): the S^T accumulators then hold
+    // base-2 exponents and the softmax needs no multiply per score
+    const float scale2 = p.scale * PF_LOG2E;
     vec8 qreg[D / 16];
     {
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
             uint4_t raw = *(const uint4_t *)(qp + 16 * kb + 8 * h2);
-            qreg[kb] = __builtin_bit_cast(vec8, raw);
+            qreg[kb] = Mma<T>::scaled(__builtin_bit_cast(vec8, raw), scale2);
         }
     }
 
@@ -169,44 +187,57 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const uint16_t *kg = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
     const uint16_t *vg = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
     const int krow_bytes = (int)p.ks[2] * 2, vrow_bytes = (int)p.vs[2] * 2;
-    const __amdgpu_buffer_rsrc_t krs =
-        __builtin_amdgcn_make_buffer_rsrc((void *)kg, 0, (p.Skv - 1) * krow_bytes + D * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrs =
-        __builtin_amdgcn_make_buffer_rsrc((void *)vg, 0, (p.Skv - 1) * vrow_bytes + D * 2, 0x00020000);
 
     float16_t o[D / 32];
 #pragma unroll
     for (int db = 0; db < D / 32; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    // m: running row maximum (base-2 exponent units); negm = -m in every element (0 while m is still
+    // -inf): it is the C operand of the first S^T MFMA of every tile, so the accumulators come out as
+    // s - m and go straight into exp2
     float m = -INFINITY, l = 0.0f;
-    const float scale2 = p.scale * PF_LOG2E;
+    float16_t negm;
+#pragma unroll
+    for (int r = 0; r < 16; r++) negm[r] = 0.0f;
 
-    // ---- tile movement: global -> registers -> LDS ---------------------------------------------------
-    // The four wavefronts of a group move one whole tile: group 1 moves the K tiles, group 0 the V
-    // tiles, each during its own vector phase (the matrix-phase wavefronts do nothing but MFMA work).
-    uint4_t st[C::NCH];
-    int gofs[C::NCH], lofs[C::NCH];  // per-thread global / LDS byte offsets of its chunks
+    using std::integral_constant;
+    // ---- tile movement: global -> LDS directly (no registers) --------------------------------------
+    // The four wavefronts of a group move one whole tile with four loads each: group 1 moves the K
+    // tiles, group 0 the V tiles.  Load j of wavefront w writes LDS group w + 4 j; lane i of it
+    // fetches row 16 (i / CPR) + w + 4 j, 16-byte column i % CPR, so the lanes of one load land
+    // contiguously (which is what the hardware does with a direct load) and the four loads of a
+    // wavefront differ by a uniform offset only.
     const bool moves_k = group == 1;
     const int mrow_bytes = moves_k ? krow_bytes : vrow_bytes;
-    const __amdgpu_buffer_rsrc_t mrs = moves_k ? krs : vrs;
-#pragma unroll
-    for (int i = 0; i < C::NCH; i++) {
-        const int cid = (tid & 255) + 256 * i;
-        const int row = cid / C::CPR, col = cid % C::CPR;
-        gofs[i] = row * mrow_bytes + col * 16;
-        lofs[i] = moves_k ? row * C::KP + col * 16 : C::K_BYTES + row * C::VP + col * 16;
-    }
+    // the moved tensor as a raw buffer descriptor (base, no stride, size in bytes, 32-bit raw format)
+    const uint64_t mptr = (uint64_t)(moves_k ? kg : vg);
+    const uint4_t mrs = {(uint32_t)mptr, (uint32_t)(mptr >> 32) & 0xffffu,
+                         (uint32_t)((p.Skv - 1) * mrow_bytes + D * 2), 0x00020000u};
+    const int wv = wave & 3;
+    const int gofs = (16 * (lane / C::CPR) + wv) * mrow_bytes + (lane % C::CPR) * 16;
+    const int lds_move_base = (moves_k ? 0 : C::K_BYTES) + wv * (moves_k ? C::KG : C::VG);
+    const int lds_move_step = 4 * (moves_k ? C::KG : C::VG);
     // a tile that starts beyond the key axis is never used: clamp the (uniform) offset so it stays
     // inside 32 bits; rows past Skv inside a used tile are out of range of the buffer and read 0
-    auto load_tile = [&](int tile) __attribute__((always_inline)) {
+    auto issue_tile = [&](int tile) __attribute__((always_inline)) {
         const int soff = min(j_begin + tile * PF_BN, p.Skv) * mrow_bytes;
+        const int lbase = (tile % NS) * STAGE + lds_move_base;
+        if (C::LOAD_LANES == 64 || lane < C::LOAD_LANES) {
+            // written as assembly on purpose: the compiler would otherwise make every later LDS read
+            // of this wavefront wait for these loads, whose data is not due before the next barrier
 #pragma unroll
-        for (int i = 0; i < C::NCH; i++) st[i] = __builtin_amdgcn_raw_buffer_load_b128(mrs, gofs[i], soff, 0);
+            for (int j = 0; j < 4; j++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                             :
+                             : "s"(lbase + j * lds_move_step), "v"(gofs), "s"(mrs), "s"(soff + 4 * j * mrow_bytes)
+                             : "memory", "m0");
+        }
     };
-    auto store_tile = [&](int tile) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < C::NCH; i++) *LDS_PTR(uint4_t, (tile & 1) * STAGE + lofs[i]) = st[i];
+    // all but the `newer` most recent tile loads of this wavefront have landed
+    auto wait_tiles = [&](auto newer) __attribute__((always_inline)) {
+        if constexpr (decltype(newer)::value == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     };
 
     float16_t s[2];     // S^T of the tile in flight
@@ -214,65 +245,67 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 
     // S^T = K . Q^T for tile i
     auto qk = [&](int i) __attribute__((always_inline)) {
-        const int stage = i & 1;
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[t][r] = 0.0f;
+        const int kbase = (i % NS) * STAGE + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                uint4_t raw = *LDS_PTR(uint4_t, stage * STAGE + (32 * t + ln) * C::KP + kb * 32 + h2 * 16);
-                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], s[t]);
+                uint4_t raw = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
+                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], kb == 0 ? negm : s[t]);
             }
         }
     };
     // O^T += V^T . P^T for tile i: contraction slice (t, kk) holds this half-wave's keys
     // 32 t + 16 kk + 4 h2 + {0..3} and + 8
     auto pv = [&](int i) __attribute__((always_inline)) {
-        const int stage = i & 1;
         const int i16 = lane & 15;
         const int bl = (lane & 31) >> 4;
+        const int vbase = (i % NS) * STAGE + C::K_BYTES + (4 * h2 + (i16 >> 2)) * C::VG + (16 * bl + 4 * (i16 & 3)) * 2;
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
+        for (int gq = 0; gq < 4; gq++) {  // gq = 2 t + kk: rows 16 gq + 4 h2 + {0..3} and + 8
+            const int t = gq >> 1, kk = gq & 1;
+            const uint4_t braw = {pk[t][4 * kk], pk[t][4 * kk + 1], pk[t][4 * kk + 2], pk[t][4 * kk + 3]};
+            const vec8 bop = __builtin_bit_cast(vec8, braw);
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
-                const uint4_t braw = {pk[t][4 * kk], pk[t][4 * kk + 1], pk[t][4 * kk + 2], pk[t][4 * kk + 3]};
-                const vec8 bop = __builtin_bit_cast(vec8, braw);
-                const int krow = 32 * t + 16 * kk + 4 * h2 + (i16 >> 2);
-#pragma unroll
-                for (int db = 0; db < D / 32; db++) {
-                    const int colb = (32 * db + 16 * bl + 4 * (i16 & 3)) * 2;
-                    short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        LDS_PTR(short4_t, stage * STAGE + C::K_BYTES + krow * C::VP + colb));
-                    short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        LDS_PTR(short4_t, stage * STAGE + C::K_BYTES + (krow + 8) * C::VP + colb));
-                    const uint2_t u0 = __builtin_bit_cast(uint2_t, a0), u1 = __builtin_bit_cast(uint2_t, a1);
-                    uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
-                    o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, araw), bop, o[db]);
-                }
+            for (int db = 0; db < D / 32; db++) {
+                const int addr = vbase + gq * C::ROWB + db * 64;
+                short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr));
+                short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VG));
+                const uint2_t u0 = __builtin_bit_cast(uint2_t, a0), u1 = __builtin_bit_cast(uint2_t, a1);
+                uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
+                o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, araw), bop, o[db]);
             }
         }
     };
-    // Matrix phase in one basic block: P.V of tile ip, then S^T of tile ik, with the LDS operand
-    // reads issued two MFMA groups ahead of their use (the order is pinned by the scheduling groups
-    // at the end; without them the reads sit right in front of their MFMAs and the pipe waits out the
-    // LDS latency every four instructions).
-    auto pv_qk = [&](int ip, int ik) __attribute__((always_inline)) {
+    // Matrix phase in one basic block: S^T of tile ik, then P.V of tile ip.  The first four K operand
+    // slices are already in `ka` (read before the barrier that opens the phase, see prefetch_k), so the
+    // matrix pipe starts at once; the remaining LDS reads are issued several MFMAs ahead of their use
+    // (the order is pinned by the scheduling groups at the end; without them the reads sit right in
+    // front of their MFMAs and the pipe waits out the LDS latency every few instructions).
+    constexpr int PFK = (D == 128) ? 2 : 4;  // K operand slices in flight (register budget)
+    uint4_t ka[PFK][2];
+    auto prefetch_k = [&](int ik) __attribute__((always_inline)) {
+        const int kbase = (ik % NS) * STAGE + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
+#pragma unroll
+        for (int kb = 0; kb < PFK; kb++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) ka[kb][t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
+    };
+    auto qk_pv = [&](int ip, int ik, auto do_pv) __attribute__((always_inline)) {
+        constexpr bool PV = decltype(do_pv)::value;
         constexpr int NDB = D / 32, NKB = D / 16;
-        const int vstage = (ip & 1) * STAGE + C::K_BYTES, kstage = (ik & 1) * STAGE;
+        const int vstage = (ip % NS) * STAGE + C::K_BYTES, kstage = (ik % NS) * STAGE;
         const int i16 = lane & 15;
         const int bl = (lane & 31) >> 4;
-        const int vbase = vstage + (4 * h2 + (i16 >> 2)) * C::VP + (16 * bl + 4 * (i16 & 3)) * 2;
-        const int kbase = kstage + ln * C::KP + h2 * 16;
+        const int vbase = vstage + (4 * h2 + (i16 >> 2)) * C::VG + (16 * bl + 4 * (i16 & 3)) * 2;
+        const int kbase = kstage + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
         uint4_t va[2][NDB];
         auto read_v = [&](int gq, uint4_t (&a)[NDB]) {  // gq = 2 t + kk: rows 32 t + 16 kk (+8)
 #pragma unroll
             for (int db = 0; db < NDB; db++) {
-                const int addr = vbase + (16 * gq) * C::VP + db * 64;
+                const int addr = vbase + gq * C::ROWB + db * 64;
                 short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr));
-                short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VP));
+                short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VG));
                 const uint2_t u0 = __builtin_bit_cast(uint2_t, a0), u1 = __builtin_bit_cast(uint2_t, a1);
                 a[db] = uint4_t{u0[0], u0[1], u1[0], u1[1]};
             }
@@ -284,44 +317,44 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
             for (int db = 0; db < NDB; db++) o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, a[db]), bop, o[db]);
         };
-        uint4_t ka[4][2];
         auto read_k = [&](int kb, uint4_t (&a)[2]) {
 #pragma unroll
-            for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + 32 * t * C::KP + kb * 32);
+            for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
         };
-        read_v(0, va[0]);
-        read_v(1, va[1]);
-        mfma_v(0, va[0]);
-        read_v(2, va[0]);
-        mfma_v(1, va[1]);
-        read_v(3, va[1]);
-        mfma_v(2, va[0]);
-#pragma unroll
-        for (int kb = 0; kb < 4 && kb < NKB; kb++) read_k(kb, ka[kb]);
-        mfma_v(3, va[1]);
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[t][r] = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-            for (int t = 0; t < 2; t++) s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, ka[kb & 3][t]), qreg[kb], s[t]);
-            if (kb + 4 < NKB) read_k(kb + 4, ka[kb & 3]);
+            for (int t = 0; t < 2; t++)
+                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, ka[kb % PFK][t]), qreg[kb], kb == 0 ? negm : s[t]);
+            if (kb + PFK < NKB) read_k(kb + PFK, ka[kb % PFK]);
+            if (PV && kb >= NKB - 4 && kb < NKB - 2) read_v(kb + 4 - NKB, va[kb + 4 - NKB]);
+        }
+        if constexpr (PV) {
+            mfma_v(0, va[0]);
+            read_v(2, va[0]);
+            mfma_v(1, va[1]);
+            read_v(3, va[1]);
+            mfma_v(2, va[0]);
+            mfma_v(3, va[1]);
         }
         // scheduling groups: 0x100 = LDS read, 0x008 = MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 4 * NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+        auto constexpr_reads = [&](int kb) __attribute__((always_inline)) {
+            const bool rk = kb + PFK < NKB, rv = PV && kb >= NKB - 4 && kb < NKB - 2;
+            if (rk && rv) __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * NDB, 0);
+            else if (rk) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            else if (rv) __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
+        };
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            if (kb + 4 < NKB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            constexpr_reads(kb);
+        }
+        if constexpr (PV) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NDB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * NDB, 0);
         }
     };
     // mask + online softmax (log2 domain, lazily rescaled) of tile i: s -> pk
@@ -337,43 +370,54 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                     s[t][r] = (key >= klo && key < khi) ? s[t][r] : -INFINITY;
                 }
         }
+        // s holds (score - m) already; mx is the tile maximum relative to the running maximum
         float mx = s[0][0];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-        mx = half_swap_max(mx) * scale2;
-        const bool grow = mx > m + PF_RESCALE_SLACK;  // also true for the first visible tile (m = -inf)
+        mx = half_swap_max(mx);
+        const bool first = (m == -INFINITY);  // no visible key so far (negm is 0 then)
+        const bool grow = first ? (mx > -INFINITY) : (mx > PF_RESCALE_SLACK);
         if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float m_new = grow ? mx : m;
-            const float corr = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m - m_new);
-            m = m_new;
+            const float delta = grow ? mx : 0.0f;
+            const float corr = first ? 0.0f : __builtin_amdgcn_exp2f(-delta);
+            m = grow ? (first ? mx : m + mx) : m;
             l *= corr;
 #pragma unroll
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[db][r] *= corr;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[t][r] -= delta;
+            const float nm = (m == -INFINITY) ? 0.0f : -m;
+#pragma unroll
+            for (int r = 0; r < 16; r++) negm[r] = nm;
         }
-        const float m_safe = (m == -INFINITY) ? 0.0f : m;
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[t][r], scale2, -m_safe));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[t][r + 1], scale2, -m_safe));
+                const float p0 = __builtin_amdgcn_exp2f(s[t][r]);
+                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
                 pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
-                l = packed_pair_sum<T>(pk[t][r >> 1], l);  // the rounded values the MFMA will use
+                l += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
             }
     };
 
     // ---- slot schedule ---------------------------------------------------------------------------------
     // Slots are separated by workgroup barriers.  Group 0 is in its matrix phase in even slots and in
     // its vector phase in odd slots; group 1 the other way round, one slot later.  Matrix phase of
-    // tile i: P.V of tile i-1 (reads V(i-1)), then S^T of tile i (reads K(i)).  Vector phase: the tile
-    // movement, then the softmax of tile i.  K(i) and V(i-1) are read in slots 2i and 2i+1.
-    // In even slot 2j group 1 moves K(j+1) from registers to LDS and fetches K(j+2); in odd slot 2j+1
-    // group 0 moves V(j) and fetches V(j+1).  Each buffer is rewritten after the barrier that follows
-    // its last reader and a full slot before its next reader.
+    // tile i: S^T of tile i (reads K(i)), then P.V of tile i-1 (reads V(i-1)); K(i) is read in slots 2i
+    // and 2i+1, V(i) in slots 2i+2 and 2i+3.  Vector phase: issue a tile load, softmax, read the first
+    // K operands of the next matrix phase, wait for the tile load issued one vector phase earlier.
+    // Tile t lives in stage t % 3.  In even slot 2j group 1 issues K(j+2) (its stage was last read for
+    // K(j-1) in slot 2j-1) and makes sure K(j+1) has landed; in odd slot 2j+1 group 0 issues V(j+1)
+    // (stage last read for V(j-2) in slot 2j-1) and makes sure V(j) has landed.  Every tile is thus
+    // complete, and published by a barrier, before the slot of its first reader, and has had two
+    // slots to arrive.
     // The tiles visible to a wavefront form one contiguous range [ia, ib).  Each group walks the slot
     // sequence in five static segments (nothing / first tile / steady state / last tile / nothing) so
     // that the steady-state loop body is branch-free and no state changes registers between phases.
@@ -383,53 +427,59 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         ib = min(ntiles, (hi_w - j_begin + PF_BN - 1) / PF_BN);
         if (ib < ia) ib = ia;
     }
-    // MODE bit 0: S^T of tile i; bit 1: P.V of tile i-1; bit 2: softmax of tile i (group 0) / i-1 (group 1)
+    // MODE bit 0: S^T of tile i; bit 1: P.V of tile i-1; bit 2: softmax of tile i (group 0) / i-1 (group 1);
+    // bit 3: the K operands of tile i were prefetched by the preceding vector phase
     auto matrix_phase = [&](int i, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
         __builtin_amdgcn_s_setprio(1);
-        if constexpr ((MODE & 3) == 3) pv_qk(i - 1, i);
-        else if constexpr ((MODE & 3) == 2) pv(i - 1);
-        else if constexpr ((MODE & 3) == 1) qk(i);
+        if constexpr ((MODE & 11) == 11) qk_pv(i - 1, i, std::true_type{});
+        else if constexpr ((MODE & 11) == 9) qk_pv(i - 1, i, std::false_type{});
+        else {
+            if constexpr ((MODE & 2) != 0) pv(i - 1);
+            if constexpr ((MODE & 1) != 0) qk(i);
+        }
         __builtin_amdgcn_s_setprio(0);
     };
-    auto vector_phase = [&](int i, int tile_to_store, auto mode) __attribute__((always_inline)) {
+    // next_k: the tile whose S^T this wavefront computes in its next matrix phase
+    auto vector_phase = [&](int i, int tile_to_load, int next_k, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
-        store_tile(tile_to_store);
-        load_tile(tile_to_store + 1);
+        issue_tile(tile_to_load);
         if constexpr ((MODE & 4) != 0) softmax(i);
+        if constexpr ((MODE & 16) != 0) prefetch_k(next_k);
+        wait_tiles(integral_constant<int, 1>{});  // the tile issued one vector phase ago has landed
     };
+    // MODE bit 4: prefetch the K operands for the next matrix phase at the end of the vector phase
     auto segment0 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 0: slot 2i matrix, slot 2i+1 vector + V(i)
         for (int i = i0; i < i1; i++) {
             matrix_phase(i, mode);
             lds_barrier();
-            vector_phase(i, i, mode);
+            vector_phase(i, i + 1, i + 1, mode);
             lds_barrier();
         }
     };
     auto segment1 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 1: slot 2i vector (tile i-1) + K(i+1), slot 2i+1 matrix
         for (int i = i0; i < i1; i++) {
-            vector_phase(i - 1, i + 1, mode);
+            vector_phase(i - 1, i + 2, i, mode);
             lds_barrier();
             matrix_phase(i, mode);
             lds_barrier();
         }
     };
-    using std::integral_constant;
     if (ntiles > 0) {
         if (moves_k) {
-            load_tile(0);
-            store_tile(0);
-            load_tile(1);
+            issue_tile(0);
+            issue_tile(1);
         } else {
-            load_tile(0);
+            issue_tile(0);
         }
+        wait_tiles(integral_constant<int, 0>{});
         lds_barrier();
         if (group == 0) {
             // iteration i: S^T(i), softmax(i), P.V(i-1)
             segment0(0, ia, integral_constant<int, 0>{});
             if (ia < ib) {
-                segment0(ia, ia + 1, integral_constant<int, 1 | 4>{});
-                segment0(ia + 1, ib, integral_constant<int, 1 | 2 | 4>{});
+                segment0(ia, ia + 1, integral_constant<int, 1 | 4 | 16>{});
+                segment0(ia + 1, ib, integral_constant<int, 1 | 2 | 4 | 8 | 16>{});
                 segment0(ib, ib + 1, integral_constant<int, 2>{});
                 segment0(ib + 1, ntiles + 1, integral_constant<int, 0>{});
             } else {
@@ -439,8 +489,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             // iteration i: softmax(i-1), then S^T(i) and P.V(i-1)
             segment1(0, ia, integral_constant<int, 0>{});
             if (ia < ib) {
-                segment1(ia, ia + 1, integral_constant<int, 1>{});
-                segment1(ia + 1, ib, integral_constant<int, 1 | 2 | 4>{});
+                segment1(ia, ia + 1, integral_constant<int, 1 | 8 | 16>{});
+                segment1(ia + 1, ib, integral_constant<int, 1 | 2 | 4 | 8 | 16>{});
                 segment1(ib, ib + 1, integral_constant<int, 2 | 4>{});
                 segment1(ib + 1, ntiles + 1, integral_constant<int, 0>{});
             } else {
@@ -449,6 +499,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         }
     }
 
+    // the epilogue reuses the tile buffers: no tile load may still be on its way into them
+    wait_tiles(integral_constant<int, 0>{});
+    lds_barrier();
     // ---- epilogue: out[query][dim] = O^T[dim][query] / l ----------------------------------------------
     const float l_tot = half_swap_sum(l);
     const float inv = 1.0f / l_tot;
@@ -459,7 +512,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         const int esz = p.out_f32 ? 4 : 2;
         const int pitch = D * esz + 16;                      // rows stay 16-byte aligned, 4 banks apart
         constexpr int SLICE = 32 * (D * 2 + 16);             // bytes per wavefront
-        static_assert(PF_WAVES * SLICE <= 2 * STAGE, "epilogue staging exceeds the tile buffers");
+        static_assert(PF_WAVES * SLICE <= NS * STAGE, "epilogue staging exceeds the tile buffers");
         auto wbase = lds_base + wave * SLICE;
         const int rounds = p.out_f32 ? 2 : 1;
         const int rows_per_round = 32 / rounds;
