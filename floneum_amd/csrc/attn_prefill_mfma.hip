@@ -168,15 +168,14 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel, already
     // multiplied by scale * log2(e) (rounded back to the input type): the S^T accumulators then hold
     // base-2 exponents and the softmax needs no multiply per score
+    // (the loads are issued here, the scaling waits until the first K/V tiles are on their way too)
     const float scale2 = p.scale * PF_LOG2E;
     vec8 qreg[D / 16];
     {
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) {
-            uint4_t raw = *(const uint4_t *)(qp + 16 * kb + 8 * h2);
-            qreg[kb] = Mma<T>::scaled(__builtin_bit_cast(vec8, raw), scale2);
-        }
+        for (int kb = 0; kb < D / 16; kb++)
+            qreg[kb] = __builtin_bit_cast(vec8, *(const uint4_t *)(qp + 16 * kb + 8 * h2));
     }
 
     const int j_begin = (lo_wg / PF_BN) * PF_BN;
@@ -291,8 +290,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
             for (int t = 0; t < 2; t++) ka[kb][t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
     };
-    auto qk_pv = [&](int ip, int ik, auto do_pv) __attribute__((always_inline)) {
+    auto qk_pv = [&](int ip, int ik, auto do_pv, auto prefetched) __attribute__((always_inline)) {
         constexpr bool PV = decltype(do_pv)::value;
+        constexpr bool PRE = decltype(prefetched)::value;
         constexpr int NDB = D / 32, NKB = D / 16;
         const int vstage = (ip % NS) * STAGE + C::K_BYTES, kstage = (ik % NS) * STAGE;
         const int i16 = lane & 15;
@@ -321,6 +321,10 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
             for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
         };
+        if constexpr (!PRE) {
+#pragma unroll
+            for (int kb = 0; kb < PFK; kb++) read_k(kb, ka[kb]);
+        }
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
@@ -344,6 +348,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             else if (rk) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             else if (rv) __builtin_amdgcn_sched_group_barrier(0x100, 2 * NDB, 0);
         };
+        if constexpr (!PRE) __builtin_amdgcn_sched_group_barrier(0x100, 2 * PFK, 0);
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
@@ -432,8 +437,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     auto matrix_phase = [&](int i, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
         __builtin_amdgcn_s_setprio(1);
-        if constexpr ((MODE & 11) == 11) qk_pv(i - 1, i, std::true_type{});
-        else if constexpr ((MODE & 11) == 9) qk_pv(i - 1, i, std::false_type{});
+        if constexpr ((MODE & 11) == 11) qk_pv(i - 1, i, std::true_type{}, std::true_type{});
+        else if constexpr ((MODE & 11) == 9) qk_pv(i - 1, i, std::false_type{}, std::true_type{});
         else {
             if constexpr ((MODE & 2) != 0) pv(i - 1);
             if constexpr ((MODE & 1) != 0) qk(i);
@@ -472,6 +477,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         } else {
             issue_tile(0);
         }
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) qreg[kb] = Mma<T>::scaled(qreg[kb], scale2);
         wait_tiles(integral_constant<int, 0>{});
         lds_barrier();
         if (group == 0) {
