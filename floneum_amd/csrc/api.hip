@@ -184,7 +184,6 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     // the kernel folds scale * log2(e) into Q (rounded back to the input type): the factor must not
     // be able to push a finite element out of range
     if (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f)) return false;
-    if (a->mask_kind != FHIP_MASK_NONE) return false;  // dense additive masks take the generic kernel
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
     // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv
     // head) slice must span less than 2 GiB
@@ -200,24 +199,38 @@ static bool prefill_f32_eligible(const fhip_attn_args *a) {
     const uint32_t D = a->q.shape[3];
     if (!(D == 32 || D == 64 || D == 96 || D == 128)) return false;
     if (!(a->scale > 0.0f)) return false;
-    if (a->mask_kind != FHIP_MASK_NONE) return false;
     if (!rows_vectorizable(a->q, 4) || !rows_vectorizable(a->k, 4) || !rows_vectorizable(a->v, 4)) return false;
     return true;
 }
 
-static int select_kernel(const fhip_attn_args *a, int32_t *id) {
+// A dense mask reaches the tiled prefill kernels in interval form (mask_intervals.hip), which needs
+// device scratch: 16 bytes for the count of rows that are not intervals, then {lo, hi} per row.
+static size_t mask_scratch_bytes(const fhip_attn_args *a) {
+    if (a->mask_kind == FHIP_MASK_NONE) return 0;
+    return mask_intervals_bytes(a->mask_kind == FHIP_MASK_QK ? (int)a->q.shape[2] : (int)a->q.shape[0]);
+}
+static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
+    if (a->mask_kind == FHIP_MASK_NONE || assume_workspace) return true;
+    return a->workspace && ((uintptr_t)a->workspace & 15) == 0 && a->workspace_bytes >= mask_scratch_bytes(a);
+}
+
+// assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
+// (the size query); otherwise a masked call without enough scratch takes the general kernel.
+static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_workspace = false) {
     const int f = a->force_kernel;
+    const bool mask_ok = mask_scratch_ok(a, assume_workspace);
     if (f != FHIP_KERNEL_AUTO) {
         bool ok = false;
         switch (f) {
             case FHIP_KERNEL_GENERIC: ok = true; break;
-            case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a); break;
-            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a); break;
+            case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a) && mask_ok; break;
+            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a) && mask_ok; break;
             case FHIP_KERNEL_DECODE_SPLITKV: ok = decode_eligible(a); break;
             default: set_error("unknown force_kernel %d", f); return FHIP_ERR_INVALID_ARG;
         }
         if (!ok) {
-            set_error("force_kernel %d cannot run these arguments (dtype/head_dim/stride/mask constraints)", f);
+            set_error("force_kernel %d cannot run these arguments (dtype/head_dim/stride constraints, or a mask without "
+                      "the workspace its interval form needs)", f);
             return FHIP_ERR_UNSUPPORTED;
         }
         *id = f;
@@ -225,9 +238,9 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id) {
     }
     if (decode_eligible(a))
         *id = FHIP_KERNEL_DECODE_SPLITKV;
-    else if (prefill_mfma_eligible(a))
+    else if (prefill_mfma_eligible(a) && mask_ok)
         *id = FHIP_KERNEL_PREFILL_MFMA;
-    else if (prefill_f32_eligible(a))
+    else if (prefill_f32_eligible(a) && mask_ok)
         *id = FHIP_KERNEL_PREFILL_F32;
     else
         *id = FHIP_KERNEL_GENERIC;
@@ -534,8 +547,9 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     int rc = validate(args);
     if (rc) return rc;
     int32_t id;
-    rc = select_kernel(args, &id);
+    rc = select_kernel(args, &id, true);
     if (rc) return rc;
+    if (id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) *bytes = mask_scratch_bytes(args);
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
         int chunk, nsplit;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
@@ -560,6 +574,23 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     fill_params(args, &p);
     FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
+        // dense mask: reduce it to one visible interval per row on the device; the tiled kernel runs
+        // if every row is of that form, the general kernel (queued right behind it) if not
+        int32_t *bad = (int32_t *)args->workspace;
+        int2 *iv = (int2 *)((char *)args->workspace + 16);
+        rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
+        if (rc) return rc;
+        AttnParams pt = p;
+        pt.iv = iv;
+        pt.iv_bad = bad;
+        rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, s->s);
+        if (rc) return rc;
+        if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+        AttnParams pg = p;
+        pg.only_if_bad = bad;
+        return launch_generic(pg, args->dtype, s->s);
+    }
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;

@@ -13,6 +13,7 @@
 //
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199; this is the data
 // type kalosm-llama always calls with (models/kalosm-llama/src/raw/attention_layer.rs:400-448).
+#include "attn_bounds.h"
 #include "common.h"
 #include "device_utils.h"
 
@@ -43,6 +44,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     __shared__ __attribute__((aligned(16))) char smem[2 * K_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
+    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -61,23 +63,8 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int q0 = qb * PF32_BM;
     const int qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
-    const int off = (int)p.q_pos_offset;
-
-    int kv_hi = p.Skv;
-    if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
-    const int q_last_wg = min(q0 + PF32_BM - 1, p.Sq - 1);
-    const int q_last_w = min(qw0 + 31, p.Sq - 1);
-    int hi_wg = kv_hi, lo_wg = 0, hi_w = kv_hi, lo_w = 0;
-    if (p.analytic) {
-        if (p.causal) {
-            hi_wg = (int)min((int64_t)kv_hi, (int64_t)q_last_wg + off + 1);
-            hi_w = (int)min((int64_t)kv_hi, (int64_t)q_last_w + off + 1);
-        }
-        if (p.window > 0) {
-            lo_wg = (int)max((int64_t)0, (int64_t)q0 + off - p.window + 1);
-            lo_w = (int)max((int64_t)0, (int64_t)qw0 + off - p.window + 1);
-        }
-    }
+    const RowBounds rb = row_bounds(p, b, q0, PF32_BM, qw0, lane);
+    const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const bool wave_has_rows = qw0 < p.Sq;
 
     // Q operand: Q[query][8 kc + 4 h2 .. +4]
@@ -144,22 +131,11 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         }
 
         // element r is key j0 + 8 (r / 4) + 4 h2 + r % 4 for query `query`
-        bool full = j0 + PF32_BN <= kv_hi;
-        if (p.analytic) {
-            if (p.causal) full = full && (j0 + PF32_BN - 1 <= qw0 + off);
-            if (p.window > 0) full = full && ((int64_t)j0 + p.window > (int64_t)q_last_w + off);
-        }
-        if (!full) {
-            const int qpos = query + off;
+        if (!(j0 >= rb.full_lo_w && j0 + PF32_BN <= rb.full_hi_w)) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                bool vis = key < kv_hi;
-                if (p.analytic) {
-                    if (p.causal) vis = vis && key <= qpos;
-                    if (p.window > 0) vis = vis && ((int64_t)key + p.window > (int64_t)qpos);
-                }
-                s[r] = vis ? s[r] : -INFINITY;
+                s[r] = (key >= rb.klo && key < rb.khi) ? s[r] : -INFINITY;
             }
         }
 

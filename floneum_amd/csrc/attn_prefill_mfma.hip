@@ -21,15 +21,17 @@
 // phase uses no dot-product instructions: on this chip they queue behind the MFMAs of the other
 // wavefront instead of running beside them.
 // All accumulation is f32; P is rounded to the input type for the second product.
-// Masking is analytic (causal with offset, sliding window, per-batch kv length, tail of the key
-// axis); key tiles that are invisible to the whole workgroup are never loaded, and tiles fully
-// visible to a wavefront skip the per-element test.
+// Masking is by interval: every query row sees one range of keys, known analytically (causal with
+// offset, sliding window, per-batch kv length, tail of the key axis) or read from the interval form
+// of a dense mask tensor (attn_bounds.h, mask_intervals.hip); key tiles that are invisible to the
+// whole workgroup are never loaded, and tiles fully visible to a wavefront skip the per-element test.
 //
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199, f32 accumulation
 // of 16-bit inputs as fusor-ml/core/src/composite/flash_attention.rs:186-203,323-327; head
 // mapping kv_head = head / (H / Hkv) (core :135-137,163-167).
 #include <type_traits>
 
+#include "attn_bounds.h"
 #include "common.h"
 #include "device_utils.h"
 
@@ -121,6 +123,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     __shared__ __attribute__((aligned(16))) char smem[NS * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
+    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it is uniform
     const int lane = tid & 63;
@@ -142,27 +145,10 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int q0 = qb * PF_BM;
     const int qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
-    const int64_t off = p.q_pos_offset;
-
-    int kv_hi = p.Skv;
-    if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
-
-    // visible key interval [klo, khi) of a query row r:  j < kv_hi, j <= r + off (causal),
-    // j + window > r + off (sliding window)
-    auto row_lo = [&](int r) __attribute__((always_inline)) -> int {
-        return (p.analytic && p.window > 0) ? (int)max((int64_t)0, (int64_t)r + off - p.window + 1) : 0;
-    };
-    auto row_hi = [&](int r) __attribute__((always_inline)) -> int {
-        return (p.analytic && p.causal) ? (int)min((int64_t)kv_hi, (int64_t)r + off + 1) : kv_hi;
-    };
-    const int q_last_wg = min(q0 + PF_BM - 1, p.Sq - 1);
-    const int q_last_w = min(qw0 + 31, p.Sq - 1);
-    const int q_first_w = min(qw0, p.Sq - 1);
-    const int lo_wg = row_lo(q0), hi_wg = row_hi(q_last_wg);        // union over the workgroup's rows
-    const int lo_w = row_lo(q_first_w), hi_w = row_hi(q_last_w);    // union over this wavefront's rows
-    const int full_lo_w = row_lo(q_last_w), full_hi_w = row_hi(q_first_w);  // intersection
+    const RowBounds rb = row_bounds(p, b, q0, PF_BM, qw0, lane);
+    const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
+    const int full_lo_w = rb.full_lo_w, full_hi_w = rb.full_hi_w, klo = rb.klo, khi = rb.khi;
     const int qrow = min(query, p.Sq - 1);
-    const int klo = row_lo(qrow), khi = row_hi(qrow);               // this lane's row
     const bool wave_has_rows = qw0 < p.Sq;
 
     // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel, already

@@ -27,7 +27,20 @@ struct AttnParams {
     int32_t chunk;          // keys per split
     int32_t nsplit;         // splits per (batch, kv head) over Skv
     hipEvent_t main_done;   // host-side only: recorded after the main kernel when not null
+    // Dense additive mask reduced to intervals (see mask_intervals.hip).  iv[r] = {lo, hi}: row r of the
+    // mask is 0 on keys [lo, hi) and -inf elsewhere; r is the query row (FHIP_MASK_QK) or the batch
+    // (FHIP_MASK_BATCH_KEY).  *iv_bad counts the rows that are NOT of that form.  A tiled kernel given
+    // `iv` does nothing when *iv_bad != 0; the general kernel given `only_if_bad` does nothing when
+    // *only_if_bad == 0: exactly one of the two computes the result.
+    const int2 *iv;
+    const int32_t *iv_bad;
+    const int32_t *only_if_bad;
 };
+
+// bytes of device scratch the interval form of a dense mask needs
+size_t mask_intervals_bytes(int rows);
+// fills iv[rows] and *bad (zeroed first) from the mask described by p.mask / p.ms0 / p.ms1 / p.mask_kind
+int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32_t *bad, hipStream_t stream);
 
 // thread-local error text
 void set_error(const char *fmt, ...);

@@ -1,0 +1,105 @@
+// Dense additive masks as intervals.
+//
+// fusor hands the attention operator its masks as tensors (fusor-ml/fusor/src/cache/mask_cache.rs:36-116,
+// attention_mask.rs:26-46): 0 where a key is visible, -inf where it is not.  Every mask those builders
+// produce (causal, sliding window, their concatenation with a cached prefix) and every padding mask
+// has, per row, ONE run of zeros.  This kernel checks that per row and writes the run as {lo, hi}; the
+// tiled attention kernels then mask by interval and never read the [rows, kv_seq_len] tensor again.  A
+// row that is anything else (finite biases, several runs, NaN) is counted in *bad and the call falls
+// back to the general kernel, which adds the mask values as the reference does
+// (fusor-ml/fusor/src/composite/flash_attention.rs:161-176).
+#include "common.h"
+#include "device_utils.h"
+
+namespace fhip {
+
+constexpr int MI_WAVES = 4;
+
+// EB: element bytes; NINF16: the 16-bit pattern of -inf (0xFC00 f16, 0xFF80 bf16), unused for EB == 4
+template <int EB>
+__global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const char *mask, int64_t ms0, int64_t ms1,
+                                                                      int rows, int cols, uint32_t ninf16, int vec_ok,
+                                                                      int2 *iv, int32_t *bad) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * MI_WAVES + (threadIdx.x >> 6);
+    if (row >= rows) return;  // whole wavefront
+    const char *mrow = mask + (int64_t)row * ms0 * EB;
+    int lo = 0x7fffffff, hi = 0, zeros = 0, others = 0;
+    auto take = [&](int j, uint32_t bits) {
+        bool ninf, zero;
+        if (EB == 4) {
+            ninf = bits == 0xFF800000u;
+            zero = (bits & 0x7FFFFFFFu) == 0;
+        } else {
+            ninf = bits == ninf16;
+            zero = (bits & 0x7FFFu) == 0;
+        }
+        if (!ninf) {
+            lo = min(lo, j);
+            hi = max(hi, j + 1);
+            zeros += zero ? 1 : 0;
+            others += zero ? 0 : 1;
+        }
+    };
+    if (vec_ok) {
+        // contiguous, 16-byte aligned rows: 16 bytes per lane and step
+        constexpr int EPV = 16 / EB;
+        const int nvec = cols / EPV;
+        for (int c = lane; c < nvec; c += 64) {
+            const uint4_t raw = __builtin_nontemporal_load((const uint4_t *)(mrow) + c);
+#pragma unroll
+            for (int e = 0; e < EPV; e++) {
+                uint32_t bits;
+                if (EB == 4) bits = raw[e];
+                else bits = (raw[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+                take(c * EPV + e, bits);
+            }
+        }
+        for (int j = nvec * EPV + lane; j < cols; j += 64) {
+            uint32_t bits = EB == 4 ? *(const uint32_t *)(mrow + (int64_t)j * 4) : *(const uint16_t *)(mrow + (int64_t)j * 2);
+            take(j, bits);
+        }
+    } else {
+        for (int j = lane; j < cols; j += 64) {
+            const char *e = mrow + (int64_t)j * ms1 * EB;
+            uint32_t bits = EB == 4 ? *(const uint32_t *)e : *(const uint16_t *)e;
+            take(j, bits);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        lo = min(lo, __shfl_xor(lo, o, 64));
+        hi = max(hi, __shfl_xor(hi, o, 64));
+        zeros += __shfl_xor(zeros, o, 64);
+        others += __shfl_xor(others, o, 64);
+    }
+    if (lane == 0) {
+        if (hi == 0) lo = 0;  // no visible key at all: the empty interval
+        const bool ok = others == 0 && zeros == hi - lo;  // only zeros and -inf, and the zeros are one run
+        iv[row] = int2{lo, hi};
+        if (!ok) atomicAdd(bad, 1);
+    }
+}
+
+size_t mask_intervals_bytes(int rows) { return ((size_t)rows * sizeof(int2) + 16 + 15) & ~(size_t)15; }
+
+int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32_t *bad, hipStream_t stream) {
+    const int rows = p.mask_kind == FHIP_MASK_QK ? p.Sq : p.B;
+    const int cols = p.Skv;
+    int rc = launch_fill_zero_bytes(bad, 16, stream);
+    if (rc) return rc;
+    if (rows == 0) return FHIP_OK;
+    const int eb = dtype == FHIP_F32 ? 4 : 2;
+    const int vec_ok = (p.ms1 == 1 || cols <= 1) && ((uintptr_t)p.mask % 16 == 0) && ((p.ms0 * eb) % 16 == 0);
+    dim3 grid((rows + MI_WAVES - 1) / MI_WAVES), block(64 * MI_WAVES);
+    if (eb == 4)
+        hipLaunchKernelGGL(mask_intervals_kernel<4>, grid, block, 0, stream, (const char *)p.mask, p.ms0, p.ms1, rows, cols,
+                           0u, vec_ok, iv, bad);
+    else
+        hipLaunchKernelGGL(mask_intervals_kernel<2>, grid, block, 0, stream, (const char *)p.mask, p.ms0, p.ms1, rows, cols,
+                           dtype == FHIP_F16 ? 0xFC00u : 0xFF80u, vec_ok, iv, bad);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+}  // namespace fhip

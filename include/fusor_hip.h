@@ -109,7 +109,13 @@ typedef struct {
     const int32_t *kv_lens;
     void *workspace; /* device scratch, >= fhip_flash_attention_workspace_bytes(), 16-byte aligned,
                         contents irrelevant; may be NULL when the size query reports 0.  Calls that
-                        share a workspace must not overlap.                                          */
+                        share a workspace must not overlap.  Split-KV decode needs it for its partial
+                        results.  A prefill call with a mask TENSOR uses it to reduce the mask to one
+                        visible interval per row on the device (every mask fusor builds, and every
+                        padding mask, has that form) and then runs the tiled kernel; a mask that is
+                        not of that form, or a call that brings no workspace, is served by the general
+                        kernel, which adds the mask values like the reference.  Same results either
+                        way.                                                                          */
     size_t workspace_bytes;
     int32_t force_kernel; /* 0 = choose; otherwise a fhip_kernel_id (testing / benchmarking)       */
     /* Optional profiling hook: when non-NULL the event is recorded on the stream right after the
@@ -173,7 +179,10 @@ int fhip_event_elapsed_ms(fhip_event *start, fhip_event *stop, float *ms);
  * GPU.  Same status and message fhip_flash_attention would return. */
 int fhip_flash_attention_validate(const fhip_attn_args *args);
 
-/* Which kernel fhip_flash_attention will run for these arguments (host-only). */
+/* Which kernel fhip_flash_attention will run for these arguments (host-only).  For a prefill call
+ * with a mask tensor and a sufficient workspace in `args` this names the tiled kernel, which runs if
+ * the mask turns out to be made of intervals (decided on the device); without the workspace it
+ * names the general kernel. */
 int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id);
 
 /* Bytes of device workspace the call needs (0 for the single-pass kernels).  `compute_units`

@@ -1,0 +1,148 @@
+"""GPU tests of dense mask tensors on the tiled prefill kernels.
+
+fusor passes its masks as tensors (MaskCache::get_mask, fusor-ml/fusor/src/cache/mask_cache.rs:36-116;
+the padding masks of the BatchKeyMask kind, fusor flash_attention.rs:161-176).  The library reduces
+such a tensor to one visible interval per row on the device and runs the tiled kernel when every
+row has that form, the general kernel otherwise.  Both outcomes are checked against the CPU checker,
+and the interval outcome is checked to be the tiled kernel by bit-equality with the analytic call.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import floneum_amd as fa
+import oracle
+from conftest import TOL_16, TOL_F32, assert_parity
+from test_attention_gpu import _normal_qkv, rounded
+
+pytestmark = pytest.mark.gpu
+
+NEG_INF = float("-inf")
+TOL_BF16 = dict(max_abs=2e-2, rel_l2=1e-2)
+
+
+def _tol(dtype):
+    return TOL_F32 if dtype == fa.F32 else (TOL_BF16 if dtype == fa.BF16 else TOL_16)
+
+
+def _tensors(device, dtype, *arrays):
+    return [fa.Tensor.from_numpy(device, a, dtype) for a in arrays]
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.F16, 64), (fa.BF16, 96), (fa.F32, 64), (fa.F32, 128)])
+@pytest.mark.parametrize("seq,offset,window", [(257, 0, None), (130, 270, None), (300, 0, 100), (96, 500, 200),
+                                               (64, 1000, 64)])
+def test_get_mask_tensor_runs_the_tiled_kernel(device, dtype, D, seq, offset, window):
+    """The tensors MaskCache::get_mask builds give bit for bit what the analytic description gives."""
+    mask = oracle.get_mask(seq, offset, window)
+    Skv = mask.shape[1]
+    q, k, v = _normal_qkv(21, 2, 4, 2, seq, Skv, D)
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    scale = D ** -0.5
+    out = tq.flash_attention(tk, tv, scale, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale, mask, "qk")
+    assert_parity(out, ref, _tol(dtype), f"dense get_mask({seq},{offset},{window}) D{D}")
+    analytic = (True, Skv - seq, window or 0)  # what get_mask builds: causal after Skv - seq cached keys, plus the window
+    out_a = tq.flash_attention(tk, tv, scale, analytic=analytic).to_numpy()
+    assert np.array_equal(out.view(np.uint8), out_a.view(np.uint8)), "dense interval mask did not take the tiled kernel"
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.F32, 64)])
+def test_padding_batch_key_mask(device, dtype, D):
+    """Left and right padding per sequence (BatchKeyMask): the tiled kernel with a key range per batch."""
+    B, H, Hkv, Sq, Skv = 3, 4, 2, 130, 333
+    q, k, v = _normal_qkv(22, B, H, Hkv, Sq, Skv, D)
+    mask = np.zeros((B, Skv), np.float32)
+    mask[0, 300:] = NEG_INF          # right padding
+    mask[1, :77] = NEG_INF           # left padding
+    mask[2, :5] = NEG_INF
+    mask[2, 200:] = NEG_INF          # both
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.BatchKeyMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "batch_key")
+    assert_parity(out, ref, _tol(dtype), "padding mask")
+    # the same call, sequence by sequence on the un-padded keys (tiled kernel, no mask at all)
+    for b, (lo, hi) in enumerate([(0, 300), (77, Skv), (5, 200)]):
+        tqb, tkb, tvb = _tensors(device, dtype, q[b:b + 1], k[b:b + 1, :, lo:hi], v[b:b + 1, :, lo:hi])
+        out_b = tqb.flash_attention(tkb, tvb, D ** -0.5).to_numpy()
+        assert_parity(out[b:b + 1], out_b, dict(max_abs=1e-6 if dtype == fa.F32 else 2e-3, rel_l2=1e-5 if dtype == fa.F32 else 1e-3),
+                      f"un-padded sequence {b}")
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.BF16, 64), (fa.F32, 64)])
+@pytest.mark.parametrize("shape", ["bias", "two_runs", "nan", "positive_inf"])
+def test_masks_that_are_not_intervals_fall_back(device, dtype, D, shape):
+    """Finite biases, several visible runs, NaN or +inf entries: the general kernel adds the values as the
+    reference does (fusor flash_attention.rs:161-176)."""
+    B, H, Hkv, Sq, Skv = 1, 2, 1, 140, 200
+    q, k, v = _normal_qkv(23, B, H, Hkv, Sq, Skv, D)
+    rng = np.random.default_rng(5)
+    mask = np.zeros((Sq, Skv), np.float32)
+    if shape == "bias":
+        mask = rng.normal(0, 1, (Sq, Skv)).astype(np.float32)
+        mask[:, 150:] = NEG_INF
+    elif shape == "two_runs":
+        mask[:, 40:60] = NEG_INF
+        mask[7, :] = 0.0
+    elif shape == "nan":
+        mask[:, 100:] = NEG_INF
+        mask[3, 5] = np.nan
+    else:
+        mask[:, 100:] = NEG_INF
+        mask[9, 120] = np.inf
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 rounded(mask, dtype), "qk")
+    bad_rows = {"nan": [3], "positive_inf": [9]}.get(shape, [])
+    keep = [r for r in range(Sq) if r not in bad_rows]
+    assert_parity(out[:, :, keep], ref[:, :, keep], _tol(dtype), f"fallback {shape}")
+    for r in bad_rows:
+        assert np.isnan(out[0, :, r]).all() and np.isnan(ref[0, :, r]).all()
+
+
+def test_rows_without_visible_keys_and_negative_zero(device):
+    """Empty rows give NaN like the reference; -0.0 counts as zero; a one-key row works."""
+    D, Sq, Skv = 128, 70, 90
+    q, k, v = _normal_qkv(24, 1, 2, 2, Sq, Skv, D)
+    mask = np.full((Sq, Skv), NEG_INF, np.float32)
+    for r in range(Sq):
+        if r % 7 == 3:
+            continue                      # nothing visible
+        lo = (r * 5) % 40
+        mask[r, lo:lo + 1 + r] = -0.0 if r % 2 else 0.0
+    tq, tk, tv, tm = _tensors(device, fa.F16, q, k, v, mask)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), D ** -0.5, mask, "qk")
+    empty = [r for r in range(Sq) if r % 7 == 3]
+    keep = [r for r in range(Sq) if r % 7 != 3]
+    assert np.isnan(out[:, :, empty]).all() and np.isnan(ref[:, :, empty]).all()
+    assert_parity(out[:, :, keep], ref[:, :, keep], TOL_16, "interval rows")
+
+
+def test_strided_and_broadcast_mask_views(device):
+    """A mask that is a transposed view, and one with a zero row stride, go through the scan as well."""
+    D, S = 64, 150
+    q, k, v = _normal_qkv(25, 1, 2, 1, S, S, D)
+    causal = oracle.get_mask(S, 0)
+    tq, tk, tv = _tensors(device, fa.F16, q, k, v)
+    # the transpose of the anti-causal mask is the causal mask
+    t_anti = fa.Tensor.from_numpy(device, np.ascontiguousarray(causal.T), fa.F16).transpose(0, 1)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (t_anti, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), D ** -0.5, causal, "qk")
+    assert_parity(out, ref, TOL_16, "transposed mask view")
+
+
+def test_without_workspace_the_general_kernel_runs(device):
+    """The C ABI never allocates: a masked call that brings no scratch is served by the general kernel."""
+    D, S = 64, 100
+    q, k, v = _normal_qkv(26, 1, 2, 1, S, S, D)
+    mask = oracle.get_mask(S, 0)
+    tq, tk, tv, tm = _tensors(device, fa.F16, q, k, v, mask)
+    assert tq.selected_kernel(tk, tv, 0.1, (tm, fa.MaskKind.QKMask)) == fa.KERNEL_GENERIC
+    out_t = fa.Tensor.empty(device, (1, 2, S, D), fa.F16)
+    args = tq._attn_args(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask), None, None, None, fa.KERNEL_AUTO, out_t)
+    fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), D ** -0.5, mask, "qk")
+    assert_parity(out_t.to_numpy(), ref, TOL_16, "no workspace")
