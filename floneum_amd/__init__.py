@@ -78,6 +78,11 @@ class CDeviceInfo(ctypes.Structure):
 # every symbol include/fusor_hip.h declares: name -> (restype, argtypes)
 _P = ctypes.c_void_p
 _PP = ctypes.POINTER(ctypes.c_void_p)
+class CRopeTables(ctypes.Structure):
+    _fields_ = [("cos", ctypes.c_void_p), ("sin", ctypes.c_void_p), ("table_rows", ctypes.c_uint64),
+                ("start_pos", ctypes.c_uint64), ("interleaved", ctypes.c_int32)]
+
+
 SYMBOLS = {
     "fhip_last_error": (ctypes.c_char_p, []),
     "fhip_version": (ctypes.c_char_p, []),
@@ -120,6 +125,11 @@ SYMBOLS = {
     "fhip_kv_cache_allocated_seq_len": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_uint64)]),
     "fhip_kv_cache_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CTensor4), ctypes.POINTER(CTensor4),
                                             ctypes.POINTER(CTensor4), ctypes.POINTER(CTensor4)]),
+    "fhip_rope": (ctypes.c_int, [_P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4), ctypes.c_int,
+                                 ctypes.POINTER(CTensor4), ctypes.c_int]),
+    "fhip_kv_cache_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
+                                                 ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
+                                                 ctypes.POINTER(CTensor4)]),
 }
 
 _LIB = None
@@ -563,3 +573,68 @@ class KvCache:
             return Tensor(_View(self.device, c.ptr, self), self.dtype, tuple(c.shape), tuple(c.stride), c.offset)
 
         return wrap(ka), wrap(va)
+
+    def append_rope(self, rope, k, v, start_pos, interleaved=False):
+        """append(rope(k), v) in one pass: the keys are rotated (RopeCache.forward semantics) and both
+        tensors converted from their own element type to the cache's on the way into the cache."""
+        assert k.dtype == v.dtype
+        ck, cv = k._c4(), v._c4()
+        ka, va = CTensor4(), CTensor4()
+        tables = rope._tables(start_pos, interleaved)
+        check(lib().fhip_kv_cache_rope_append(self.handle, self.device.stream, ctypes.byref(tables), ctypes.byref(ck),
+                                              ctypes.byref(cv), k.dtype, ctypes.byref(ka), ctypes.byref(va)))
+
+        def wrap(c):
+            return Tensor(_View(self.device, c.ptr, self), self.dtype, tuple(c.shape), tuple(c.stride), c.offset)
+
+        return wrap(ka), wrap(va)
+
+
+def base_inverse_frequency(dim, rope_theta):
+    """fusor::base_inverse_frequency (rope.rs:188-196): 1 / theta^(i / dim) for even i, in f32."""
+    theta = np.float32(rope_theta)
+    return np.array([np.float32(1.0) / np.power(theta, np.float32(i) / np.float32(dim), dtype=np.float32)
+                     for i in range(0, dim, 2)], np.float32)
+
+
+class RopeCache:
+    """fusor::RopeCache (rope.rs:180-265): [context_length, head_dim/2] f32 cos/sin tables on the device."""
+
+    def __init__(self, head_dim, context_length, rope_theta, device=None, inverse_frequency=None):
+        self.device = device or Device.default()
+        inv = base_inverse_frequency(head_dim, rope_theta) if inverse_frequency is None \
+            else np.asarray(inverse_frequency, np.float32)
+        pos = np.arange(context_length, dtype=np.float32)[:, None]
+        outer = (pos * inv[None, :]).astype(np.float32)  # a [n,1] x [1,h] matmul: one product per element
+        self.cos_host, self.sin_host = np.cos(outer).astype(np.float32), np.sin(outer).astype(np.float32)
+        self.cos = Tensor.from_numpy(self.device, self.cos_host, F32)
+        self.sin = Tensor.from_numpy(self.device, self.sin_host, F32)
+        self.rows = context_length
+
+    @classmethod
+    def from_parts(cls, cos, sin, device=None):
+        self = cls.__new__(cls)
+        self.device = device or Device.default()
+        self.cos_host, self.sin_host = np.asarray(cos, np.float32), np.asarray(sin, np.float32)
+        self.cos = Tensor.from_numpy(self.device, self.cos_host, F32)
+        self.sin = Tensor.from_numpy(self.device, self.sin_host, F32)
+        self.rows = self.cos_host.shape[0]
+        return self
+
+    def _tables(self, start_pos, interleaved):
+        return CRopeTables(self.cos.buffer.ptr, self.sin.buffer.ptr, self.rows, start_pos, 1 if interleaved else 0)
+
+    def apply(self, x, start_pos, interleaved=False, out_dtype=None):
+        """Tensor::rope_normal_fused / rope_fused with the tables narrowed to start_pos.. (rope.rs:139-175)."""
+        out = Tensor.empty(self.device, x.shape, out_dtype if out_dtype is not None else x.dtype)
+        cx, co = x._c4(), out._c4()
+        tables = self._tables(start_pos, interleaved)
+        check(lib().fhip_rope(self.device.stream, ctypes.byref(tables), ctypes.byref(cx), x.dtype, ctypes.byref(co),
+                              out.dtype))
+        return out
+
+    def forward(self, q, k, start_pos):
+        return self.apply(q, start_pos), self.apply(k, start_pos)
+
+    def forward_interleaved(self, q, k, start_pos):
+        return self.apply(q, start_pos, True), self.apply(k, start_pos, True)

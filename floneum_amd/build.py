@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SOURCES = ["api.hip", "attn_generic.hip", "attn_decode.hip", "attn_prefill_mfma.hip", "attn_prefill_f32.hip",
-           "kv_cache.hip", "mask_intervals.hip"]
+           "kv_cache.hip", "mask_intervals.hip", "rope.hip"]
 LIB = os.path.join(HERE, "libfusor_hip.so")
 STATIC = os.path.join(HERE, "libfusor_hip.a")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -17,11 +17,13 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", 
 
 
 EXTRA = os.environ.get("FHIP_EXTRA_FLAGS", "").split()  # e.g. -D switches while tuning
+# the rotary embedding must round every product and sum on its own (bit parity with the reference's CPU path)
+PER_FILE = {"rope.hip": ["-ffp-contract=off"]}
 
 
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + EXTRA + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + PER_FILE.get(src, []) + EXTRA + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

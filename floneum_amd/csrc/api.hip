@@ -742,6 +742,25 @@ static uint64_t next_pow2(uint64_t x) {
     return p;
 }
 
+// How the new rows of an append reach the cache: copied as they are (src_dtype == cache dtype, no
+// tables), or converted on the way, the keys rotated by the rotary embedding first.
+struct NewRows {
+    fhip_dtype src_dtype;
+    const fhip_rope_tables *rope;  // nullptr: plain copy
+};
+
+// rows [first, first + count) of the new block `src` -> dst (cache dtype, strides dst_st); side 0 = keys
+static int write_new_rows(const fhip_kv_cache *c, hipStream_t st, int side, const fhip_tensor4 *src, uint64_t first,
+                          uint32_t count, void *dst, const int64_t dst_st[4], const NewRows &nr) {
+    const uint32_t shp[4] = {c->B, c->Hkv, count, c->D};
+    const int seb = fhip::elem_bytes(nr.src_dtype);
+    const char *sp = (const char *)src->ptr + (src->offset + first * src->stride[2]) * (uint64_t)seb;
+    if (!nr.rope) return launch_copy_rows(sp, src->stride, dst, dst_st, shp, seb, st);
+    const int mode = side == 0 ? (nr.rope->interleaved ? 1 : 0) : 2;
+    return launch_rope_rows(sp, src->stride, nr.src_dtype, dst, dst_st, c->dtype, shp, nr.rope->cos, nr.rope->sin,
+                            (int64_t)(nr.rope->start_pos + first), mode, st);
+}
+
 extern "C" {
 
 int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequence_len, fhip_kv_cache **out) {
@@ -815,8 +834,8 @@ int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len) {
     return FHIP_OK;
 }
 
-int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
-                         fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
+                          fhip_tensor4 *k_all, fhip_tensor4 *v_all, const NewRows &nr) {
     if (!c || !s || !k_new || !v_new || !k_all || !v_all) {
         set_error("kv_cache_append: NULL argument");
         return FHIP_ERR_INVALID_ARG;
@@ -875,11 +894,8 @@ int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k
                                           eb, s->s);
                 if (rc) return rc;
             }
-            const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)take_new, c->D};
-            const char *src = (const char *)news[sd]->ptr +
-                              (news[sd]->offset + (n - take_new) * news[sd]->stride[2]) * (uint64_t)eb;
-            int rc = launch_copy_rows(src, news[sd]->stride, (char *)S.spare + keep_old * c->D * eb, dst_st, shp, eb,
-                                      s->s);
+            int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
+                                    (char *)S.spare + keep_old * c->D * eb, dst_st, nr);
             if (rc) return rc;
             if (S.buf && c->allocated != mx) {
                 // the growing buffer is retired; hipFree waits for the copies above
@@ -903,9 +919,7 @@ int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k
             FHIP_HIP_CHECK(hipMalloc(&S.buf, row_elems * n * eb));
             int64_t dst_st[4];
             kv_contig_strides(c, n, dst_st);
-            const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)n, c->D};
-            const char *src = (const char *)news[sd]->ptr + news[sd]->offset * (uint64_t)eb;
-            int rc = launch_copy_rows(src, news[sd]->stride, S.buf, dst_st, shp, eb, s->s);
+            int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, S.buf, dst_st, nr);
             if (rc) return rc;
             kv_view(c, S.buf, n, n, alls[sd]);
         }
@@ -940,15 +954,72 @@ int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k
                 S.spare = nullptr;
             }
         }
-        const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)n, c->D};
-        const char *src = (const char *)news[sd]->ptr + news[sd]->offset * (uint64_t)eb;
-        int rc = launch_copy_rows(src, news[sd]->stride, (char *)S.buf + c->current * c->D * eb, dst_st, shp, eb, s->s);
+        int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, (char *)S.buf + c->current * c->D * eb, dst_st, nr);
         if (rc) return rc;
         kv_view(c, S.buf, alloc, required, alls[sd]);
     }
     c->current = required;
     c->allocated = alloc;
     return FHIP_OK;
+}
+
+int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
+                         fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    NewRows nr;
+    nr.src_dtype = c ? c->dtype : FHIP_F32;
+    nr.rope = nullptr;
+    return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
+}
+
+static int check_rope(const fhip_rope_tables *r, uint32_t head_dim, uint64_t rows) {
+    if (!r || !r->cos || !r->sin) {
+        set_error("rope: NULL tables");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (head_dim == 0 || head_dim % 2 != 0) {
+        set_error("rope: head_dim %u must be even", head_dim);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (r->start_pos + rows > r->table_rows) {
+        set_error("rope: positions %llu..%llu exceed the %llu rows of the tables", (unsigned long long)r->start_pos,
+                  (unsigned long long)(r->start_pos + rows), (unsigned long long)r->table_rows);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    return FHIP_OK;
+}
+
+int fhip_rope(fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *x, fhip_dtype x_dtype, const fhip_tensor4 *out,
+              fhip_dtype out_dtype) {
+    if (!s || !x || !out || !x->ptr || !out->ptr || !fhip::dtype_ok(x_dtype) || !fhip::dtype_ok(out_dtype)) {
+        set_error("rope: NULL argument or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (int i = 0; i < 4; i++)
+        if (x->shape[i] != out->shape[i]) {
+            set_error("rope: output shape differs from the input shape");
+            return FHIP_ERR_INVALID_ARG;
+        }
+    int rc = check_rope(rope, x->shape[3], x->shape[2]);
+    if (rc) return rc;
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    const char *sp = (const char *)x->ptr + x->offset * (uint64_t)fhip::elem_bytes(x_dtype);
+    char *dp = (char *)out->ptr + out->offset * (uint64_t)fhip::elem_bytes(out_dtype);
+    return launch_rope_rows(sp, x->stride, x_dtype, dp, out->stride, out_dtype, x->shape, rope->cos, rope->sin,
+                            (int64_t)rope->start_pos, rope->interleaved ? 1 : 0, s->s);
+}
+
+int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *k_new,
+                              const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    if (!k_new || !fhip::dtype_ok(in_dtype)) {
+        set_error("kv_cache_rope_append: NULL argument or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    int rc = check_rope(rope, k_new->shape[3], k_new->shape[2]);
+    if (rc) return rc;
+    NewRows nr;
+    nr.src_dtype = in_dtype;
+    nr.rope = rope;
+    return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
 }
 
 }  // extern "C"

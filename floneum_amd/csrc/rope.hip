@@ -1,0 +1,96 @@
+// Rotary position embedding, fused with the type conversion and the write into its destination
+// (a query tensor for the attention call, or the new rows of the KV cache).
+//
+// Semantics: fusor-ml/fusor/src/composite/rope.rs:46-137 in f32, one rounding per operation as the
+// reference's CPU path has (mul, mul, add are separate tensor ops there):
+//   normal (rope / rope_normal_fused):       y[i]        = x[i] * cos[p][i]        + (-x[i + D/2]) * sin[p][i]
+//                                            y[i + D/2]  = x[i + D/2] * cos[p][i]  +   x[i]        * sin[p][i]
+//   interleaved (rope_interleaved / rope_fused): y[2i]   = x[2i] * cos[p][i] - x[2i+1] * sin[p][i]
+//                                            y[2i+1]     = x[2i] * sin[p][i] + x[2i+1] * cos[p][i]
+// with p = start_pos + row (RopeCache::forward, rope.rs:232-265) and cos/sin the [positions, D/2]
+// f32 tables of fusor::RopeCache.  16-bit inputs are widened to f32 first and the result is rounded
+// to nearest even, which is what kalosm-llama's cast -> rope -> cast does
+// (models/kalosm-llama/src/raw/rope.rs:103-111).
+#include "common.h"
+#include "device_utils.h"
+
+namespace fhip {
+
+__device__ __forceinline__ float load_as_f32(const void *p, int64_t idx, int dtype) {
+    if (dtype == FHIP_F32) return ((const float *)p)[idx];
+    if (dtype == FHIP_F16) return (float)((const half_t *)p)[idx];
+    return to_float(((const bf16_t *)p)[idx]);
+}
+__device__ __forceinline__ void store_from_f32(void *p, int64_t idx, int dtype, float v) {
+    if (dtype == FHIP_F32) ((float *)p)[idx] = v;
+    else if (dtype == FHIP_F16) ((half_t *)p)[idx] = (half_t)v;
+    else ((bf16_t *)p)[idx] = from_float<bf16_t>(v);
+}
+
+struct RopeRows {
+    const void *src;
+    void *dst;
+    int64_t ss[4], ds[4];
+    uint32_t shape[4];  // [B, heads, rows, D]
+    int32_t src_dtype, dst_dtype;
+    const float *cos, *sin;
+    int64_t pos0;       // table row of row 0
+    int32_t mode;       // 0 normal, 1 interleaved, 2 convert only
+};
+
+__global__ __launch_bounds__(256) void rope_rows_kernel(RopeRows a) {
+    const uint32_t D = a.shape[3], half = D / 2;
+    const int64_t per_row = a.mode == 2 ? D : half;
+    const int64_t total = (int64_t)a.shape[0] * a.shape[1] * a.shape[2] * per_row;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const uint32_t i = (uint32_t)(idx % per_row);
+        int64_t t = idx / per_row;
+        const uint32_t r = (uint32_t)(t % a.shape[2]);
+        t /= a.shape[2];
+        const uint32_t h = (uint32_t)(t % a.shape[1]);
+        const uint32_t b = (uint32_t)(t / a.shape[1]);
+        const int64_t sb = b * a.ss[0] + h * a.ss[1] + r * a.ss[2];
+        const int64_t db = b * a.ds[0] + h * a.ds[1] + r * a.ds[2];
+        if (a.mode == 2) {
+            store_from_f32(a.dst, db + i * a.ds[3], a.dst_dtype, load_as_f32(a.src, sb + i * a.ss[3], a.src_dtype));
+            continue;
+        }
+        const float c = a.cos[(a.pos0 + r) * half + i], s = a.sin[(a.pos0 + r) * half + i];
+        const uint32_t d0 = a.mode == 0 ? i : 2 * i, d1 = a.mode == 0 ? i + half : 2 * i + 1;
+        const float x0 = load_as_f32(a.src, sb + d0 * a.ss[3], a.src_dtype);
+        const float x1 = load_as_f32(a.src, sb + d1 * a.ss[3], a.src_dtype);
+        // every product and sum is rounded on its own: this file is compiled with -ffp-contract=off
+        const float y0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+        const float y1 = a.mode == 0 ? __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, s))
+                                     : __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+        store_from_f32(a.dst, db + d0 * a.ds[3], a.dst_dtype, y0);
+        store_from_f32(a.dst, db + d1 * a.ds[3], a.dst_dtype, y1);
+    }
+}
+
+int launch_rope_rows(const void *src, const int64_t ss[4], fhip_dtype src_dtype, void *dst, const int64_t ds[4],
+                     fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos, const float *sin, int64_t pos0,
+                     int mode, hipStream_t stream) {
+    RopeRows a;
+    a.src = src;
+    a.dst = dst;
+    for (int i = 0; i < 4; i++) {
+        a.ss[i] = ss[i];
+        a.ds[i] = ds[i];
+        a.shape[i] = shape[i];
+    }
+    a.src_dtype = src_dtype;
+    a.dst_dtype = dst_dtype;
+    a.cos = cos;
+    a.sin = sin;
+    a.pos0 = pos0;
+    a.mode = mode;
+    const int64_t total = (int64_t)shape[0] * shape[1] * shape[2] * (mode == 2 ? shape[3] : shape[3] / 2);
+    if (total == 0) return FHIP_OK;
+    const int64_t blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, stream, a);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+}  // namespace fhip

@@ -233,6 +233,33 @@ int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len);
 int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new,
                          const fhip_tensor4 *v_new, fhip_tensor4 *k_all, fhip_tensor4 *v_all);
 
+/* ---- rotary position embedding, fused with its destination --------------------------------------
+ * The step right before attention in kalosm-llama (models/kalosm-llama/src/raw/attention_layer.rs:
+ * 272-278, raw/rope.rs:86-111): q and k are cast to f32, rotated with the [positions, head_dim/2]
+ * cos/sin tables of fusor::RopeCache (fusor-ml/fusor/src/composite/rope.rs:180-265), cast back, and k,
+ * v are appended to the cache.  Here the rotation, the casts and the cache write are one pass:
+ * arithmetic in f32 with one rounding per operation as on the reference's CPU path (rope.rs:46-137),
+ * results rounded to nearest even into the destination type. */
+typedef struct {
+    const float *cos;    /* device, [table_rows, head_dim/2] f32 row-major (RopeCache::cos)           */
+    const float *sin;    /* device, same shape (RopeCache::sin)                                        */
+    uint64_t table_rows;
+    uint64_t start_pos;  /* table row used by sequence position 0 of the tensor (RopeCache::forward)  */
+    int32_t interleaved; /* 0: pairs (i, i + head_dim/2)  (rope, rope_normal_fused)
+                            1: pairs (2i, 2i + 1)         (rope_interleaved, rope_fused)              */
+} fhip_rope_tables;
+
+/* out = rope(x): x, out [B, heads, seq, head_dim] strided device views of x_dtype / out_dtype; out may
+ * be x itself.  Replaces Tensor::rope_normal_fused / rope_fused (rope.rs:139-175). */
+int fhip_rope(fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *x, fhip_dtype x_dtype,
+              const fhip_tensor4 *out, fhip_dtype out_dtype);
+
+/* fhip_kv_cache_append with the new keys rotated and both tensors converted from in_dtype to the
+ * cache's type on the way in (no rotated copy of k, no separate cast pass). */
+int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *k_new,
+                              const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all,
+                              fhip_tensor4 *v_all);
+
 /* Library version string, e.g. "fusor-hip 0.1 (gfx950)". */
 const char *fhip_version(void);
 

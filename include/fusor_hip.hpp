@@ -341,6 +341,72 @@ class KvCache {
         };
         return {wrap(ka), wrap(va)};
     }
+    /// append(rope(k), v): the rotation of RopeCache::forward / forward_interleaved and the conversion to
+    /// the cache's element type happen in the pass that writes the new rows
+    std::pair<Tensor<4>, Tensor<4>> append_rope(const fhip_rope_tables &tables, const Tensor<4> &k, const Tensor<4> &v) {
+        if (k.dtype() != v.dtype()) throw Panic("append_rope: keys and values differ in element type");
+        fhip_tensor4 kn = k.c4(), vn = v.c4(), ka{}, va{};
+        check(fhip_kv_cache_rope_append(in_->c, dev_.stream(), &tables, &kn, &vn, (fhip_dtype)k.dtype(), &ka, &va));
+        auto wrap = [&](const fhip_tensor4 &t) {
+            Tensor<4> r(std::make_shared<Buffer>(dev_, t.ptr), dtype_, t.shape, t.stride, t.offset, in_);
+            return r;
+        };
+        return {wrap(ka), wrap(va)};
+    }
+};
+
+/// fusor::RopeCache (fusor-ml/fusor/src/composite/rope.rs:180-265): [context_length, head_dim/2] f32
+/// cos/sin tables on the device, applied by one fused kernel per tensor.
+class RopeCache {
+    Tensor<2> cos_, sin_;
+    Device dev_;
+    uint64_t rows_;
+
+   public:
+    /// RopeCache::from_parts(cos, sin): host tables, row-major [rows, head_dim / 2]
+    RopeCache(const Device &dev, uint32_t rows, uint32_t half_dim, const float *cos, const float *sin)
+        : cos_(Tensor<2>::from_slice(dev, DType::F32, {rows, half_dim}, cos)),
+          sin_(Tensor<2>::from_slice(dev, DType::F32, {rows, half_dim}, sin)), dev_(dev), rows_(rows) {}
+    /// RopeCache::new(head_dim, context_length, rope_theta, device) (rope.rs:198-221)
+    static RopeCache standard(const Device &dev, uint32_t head_dim, uint32_t context_length, float rope_theta) {
+        const uint32_t half = head_dim / 2;
+        std::vector<float> c((size_t)context_length * half), s(c.size());
+        for (uint32_t i = 0; i < half; i++) {
+            const float inv = 1.0f / std::pow(rope_theta, (float)(2 * i) / (float)head_dim);  // base_inverse_frequency
+            for (uint32_t p = 0; p < context_length; p++) {
+                const float a = (float)p * inv;
+                c[(size_t)p * half + i] = std::cos(a);
+                s[(size_t)p * half + i] = std::sin(a);
+            }
+        }
+        return RopeCache(dev, context_length, half, c.data(), s.data());
+    }
+    fhip_rope_tables tables(uint64_t start_pos, bool interleaved) const {
+        fhip_rope_tables t{};
+        t.cos = (const float *)cos_.c2().ptr;
+        t.sin = (const float *)sin_.c2().ptr;
+        t.table_rows = rows_;
+        t.start_pos = start_pos;
+        t.interleaved = interleaved ? 1 : 0;
+        return t;
+    }
+    Tensor<4> apply(const Tensor<4> &x, uint64_t start_pos, bool interleaved, std::optional<DType> out_dtype = std::nullopt) const {
+        const DType od = out_dtype.value_or(x.dtype());
+        const auto &shp = x.shape();
+        Tensor<4> out = Tensor<4>::empty(dev_, od, {shp[0], shp[1], shp[2], shp[3]});
+        const fhip_rope_tables t = tables(start_pos, interleaved);
+        const fhip_tensor4 cx = x.c4(), co = out.c4();
+        check(fhip_rope(dev_.stream(), &t, &cx, (fhip_dtype)x.dtype(), &co, (fhip_dtype)od));
+        return out;
+    }
+    /// RopeCache::forward(q, k, start_pos) -> (q, k)   (pairs (i, i + head_dim/2))
+    std::pair<Tensor<4>, Tensor<4>> forward(const Tensor<4> &q, const Tensor<4> &k, uint64_t start_pos) const {
+        return {apply(q, start_pos, false), apply(k, start_pos, false)};
+    }
+    /// RopeCache::forward_interleaved(q, k, start_pos) -> (q, k)   (pairs (2i, 2i + 1))
+    std::pair<Tensor<4>, Tensor<4>> forward_interleaved(const Tensor<4> &q, const Tensor<4> &k, uint64_t start_pos) const {
+        return {apply(q, start_pos, true), apply(k, start_pos, true)};
+    }
 };
 
 }  // namespace fusor_hip

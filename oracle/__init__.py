@@ -249,3 +249,58 @@ class KvCache:
 
     def current_seq_len(self):
         return self.key.current_seq_len
+
+
+# ---- rotary position embedding (fusor-ml/fusor/src/composite/rope.rs) --------------------------------
+# numpy float32 arithmetic rounds once per operation, exactly like the reference's CPU tensor ops
+# (mul_, add_, sub_ are separate passes there), so these restatements are bit-level statements of it.
+
+def rope_tables(head_dim, context_length, theta):
+    """RopeCache::new (rope.rs:198-221): outer product of positions and 1/theta^(i/dim), then cos/sin, in f32.
+    The last bit of cos/sin depends on the libm in use; the rotation itself takes the tables as inputs."""
+    th = np.float32(theta)
+    inv = np.array([np.float32(1.0) / np.power(th, np.float32(i) / np.float32(head_dim), dtype=np.float32)
+                    for i in range(0, head_dim, 2)], np.float32)
+    outer = (np.arange(context_length, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float32)
+    return np.cos(outer).astype(np.float32), np.sin(outer).astype(np.float32)
+
+
+def rope(x, cos, sin, start_pos=0):
+    """Tensor::rope (rope.rs:46-79) on rows start_pos.. of the tables: x*cos + rotate_half(x)*sin."""
+    x = np.asarray(x, np.float32)
+    n, d = x.shape[2], x.shape[3]
+    c = np.concatenate([cos, cos], 1)[start_pos:start_pos + n][None, None].astype(np.float32)
+    s = np.concatenate([sin, sin], 1)[start_pos:start_pos + n][None, None].astype(np.float32)
+    h = d // 2
+    rot = np.concatenate([-x[..., h:], x[..., :h]], -1)  # rotate_half (rope.rs:10-21)
+    return (x * c).astype(np.float32) + (rot * s).astype(np.float32)
+
+
+def rope_interleaved(x, cos, sin, start_pos=0):
+    """Tensor::rope_interleaved (rope.rs:81-137): pairs (2i, 2i+1)."""
+    x = np.asarray(x, np.float32)
+    n = x.shape[2]
+    c = cos[start_pos:start_pos + n][None, None].astype(np.float32)
+    s = sin[start_pos:start_pos + n][None, None].astype(np.float32)
+    x0, x1 = x[..., 0::2], x[..., 1::2]
+    y0 = (x0 * c).astype(np.float32) - (x1 * s).astype(np.float32)
+    y1 = (x0 * s).astype(np.float32) + (x1 * c).astype(np.float32)
+    out = np.empty_like(x)
+    out[..., 0::2], out[..., 1::2] = y0, y1
+    return out
+
+
+def rope_f64(x, cos, sin, start_pos=0, interleaved=False):
+    """The same rotation written from the textbook (complex multiplication) in float64."""
+    x = np.asarray(x, np.float64)
+    n, d = x.shape[2], x.shape[3]
+    ang_c = np.asarray(cos, np.float64)[start_pos:start_pos + n][None, None]
+    ang_s = np.asarray(sin, np.float64)[start_pos:start_pos + n][None, None]
+    z = (x[..., 0::2] + 1j * x[..., 1::2]) if interleaved else (x[..., :d // 2] + 1j * x[..., d // 2:])
+    w = z * (ang_c + 1j * ang_s)
+    out = np.empty_like(x)
+    if interleaved:
+        out[..., 0::2], out[..., 1::2] = w.real, w.imag
+    else:
+        out[..., :d // 2], out[..., d // 2:] = w.real, w.imag
+    return out

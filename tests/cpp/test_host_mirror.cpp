@@ -127,6 +127,45 @@ static void test_kv_cache(const Device &d) {  // kv_cache.rs:74-157, tensor_cach
     EXPECT(cache.current_seq_len() == 0, "reset");
 }
 
+static void test_rope(const Device &d) {  // rope.rs:270-400 (inputs), rope.rs:46-137 (values)
+    const uint32_t rows = 11, half = 32;
+    std::vector<float> c(rows * half), s(rows * half), x(3 * 11 * 64);
+    for (uint32_t i = 0; i < rows; i++)
+        for (uint32_t j = 0; j < half; j++) {
+            const float a = (float)i / std::pow(10000.0f, (float)(2 * j) / 64.0f);
+            c[i * half + j] = std::cos(a);
+            s[i * half + j] = std::sin(a);
+        }
+    for (size_t k = 0; k < x.size(); k++) x[k] = std::sin((float)(k % 64));
+    RopeCache rope(d, rows, half, c.data(), s.data());
+    auto t = t4(d, x, 1, 3, 11, 64);
+    auto qk = rope.forward(t, t, 0);
+    auto qi = rope.forward_interleaved(t, t, 0);
+    auto y = host(qk.first), yi = host(qi.second);
+    EXPECT(qk.first.shape()[1] == 3 && qk.first.shape()[2] == 11 && qk.first.shape()[3] == 64, "rope shape");
+    int bad = 0;
+    for (uint32_t h = 0; h < 3; h++)
+        for (uint32_t r = 0; r < 11; r++)
+            for (uint32_t i = 0; i < 32; i++) {
+                const size_t base = ((size_t)h * 11 + r) * 64;
+                const float cc = c[r * half + i], ss = s[r * half + i];
+                // the volatile temporaries keep the host compiler from fusing the products into the sums
+                volatile float a0 = x[base + i] * cc, a1 = x[base + i + 32] * ss, b0 = x[base + i + 32] * cc, b1 = x[base + i] * ss;
+                if (y[base + i] != a0 - a1 || y[base + i + 32] != b0 + b1 || !std::isfinite(y[base + i])) bad++;
+                volatile float e0 = x[base + 2 * i] * cc, e1 = x[base + 2 * i + 1] * ss, f0 = x[base + 2 * i] * ss, f1 = x[base + 2 * i + 1] * cc;
+                if (yi[base + 2 * i] != e0 - e1 || yi[base + 2 * i + 1] != f0 + f1) bad++;
+            }
+    EXPECT(bad == 0, "%d rope values differ from x*cos + rotate_half(x)*sin", bad);
+    // fused into the cache write: rope(k) lands in the cache, v unchanged
+    KvCache cache(d, 2, 64);
+    auto kv = cache.append_rope(rope.tables(0, false), t, t);
+    auto kc = host(kv.first), vc = host(kv.second);
+    bad = 0;
+    for (size_t k = 0; k < x.size(); k++)
+        if (kc[k] != y[k] || vc[k] != x[k]) bad++;
+    EXPECT(bad == 0, "%d cached values differ after append_rope", bad);
+}
+
 int main() {
     try {
         Device d(0);
@@ -137,6 +176,7 @@ int main() {
         test_attention_mask_causal(d);
         test_mask_cache(d);
         test_kv_cache(d);
+        test_rope(d);
     } catch (const std::exception &e) {
         printf("exception: %s\n", e.what());
         return 2;

@@ -1,0 +1,101 @@
+"""GPU tests of the fused rotary embedding (fhip_rope, fhip_kv_cache_rope_append) through the C ABI.
+
+Bit-exact against the CPU restatement of fusor's rope (rope.rs:46-137) for f32, and for 16-bit tensors
+against cast -> rope in f32 -> cast, which is what kalosm-llama does (raw/rope.rs:103-111).
+"""
+import numpy as np
+import pytest
+
+import floneum_amd as fa
+import oracle
+from test_attention_gpu import rounded
+
+pytestmark = pytest.mark.gpu
+
+
+def _cast_out(y, dtype):
+    """y rounded to the element type, in the form Tensor.to_numpy() returns it (bf16 comes back as f32)."""
+    if dtype == fa.F32:
+        return y.astype(np.float32)
+    if dtype == fa.F16:
+        return y.astype(np.float16)
+    return fa.bf16_bits_to_f32(fa.f32_to_bf16_bits(y)).reshape(y.shape)
+
+
+def _x(seed, shape):
+    return np.random.default_rng(seed).normal(0, 1, shape).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16, fa.BF16])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("D,start", [(64, 0), (128, 37), (96, 5), (2, 1)])
+def test_rope_bit_exact(device, dtype, interleaved, D, start):
+    rc = fa.RopeCache(D, 64, 10000.0, device)
+    x = _x(D + start, (2, 3, 11, D))
+    t = fa.Tensor.from_numpy(device, x, dtype)
+    out = rc.apply(t, start, interleaved).to_numpy()
+    fn = oracle.rope_interleaved if interleaved else oracle.rope
+    ref = _cast_out(fn(rounded(x, dtype), rc.cos_host, rc.sin_host, start), dtype)
+    assert np.array_equal(out.view(np.uint8), ref.view(np.uint8))
+
+
+def test_rope_reference_test_inputs(device):
+    # the inputs of fusor's rope tests (rope.rs:272-330)
+    i = np.arange(11, dtype=np.float32)[:, None]
+    j = np.arange(32, dtype=np.float32)[None, :]
+    ang = (i / np.power(np.float32(10000.0), (2 * j) / np.float32(64), dtype=np.float32)).astype(np.float32)
+    rc = fa.RopeCache.from_parts(np.cos(ang), np.sin(ang), device)
+    x = np.sin((np.arange(3 * 11 * 64) % 64).astype(np.float32)).astype(np.float32).reshape(1, 3, 11, 64)
+    t = fa.Tensor.from_numpy(device, x, fa.F32)
+    q, k = rc.forward(t, t, 0)
+    qi, ki = rc.forward_interleaved(t, t, 0)
+    assert q.shape == (1, 3, 11, 64) and np.isfinite(q.to_numpy()).all() and np.isfinite(qi.to_numpy()).all()
+    assert np.array_equal(q.to_numpy(), oracle.rope(x, rc.cos_host, rc.sin_host))
+    assert np.array_equal(ki.to_numpy(), oracle.rope_interleaved(x, rc.cos_host, rc.sin_host))
+
+
+def test_rope_on_the_transposed_projection_view_and_type_change(device):
+    """kalosm-llama's projections are [b, seq, heads, hd] transposed to [b, heads, seq, hd]
+    (attention_layer.rs:226-229): the op takes that view as it is, and can hand f16 to the attention call."""
+    B, S, H, D = 2, 9, 4, 64
+    rc = fa.RopeCache(D, 32, 500000.0, device)
+    proj = _x(7, (B, S, H, D))
+    t = fa.Tensor.from_numpy(device, proj, fa.F32).transpose(1, 2)
+    out = rc.apply(t, 3, False, out_dtype=fa.F16).to_numpy()
+    ref = oracle.rope(proj.transpose(0, 2, 1, 3), rc.cos_host, rc.sin_host, 3).astype(np.float16)
+    assert out.dtype == np.float16 and np.array_equal(out, ref)
+
+
+def test_rope_rejects_bad_arguments(device):
+    rc = fa.RopeCache(64, 8, 10000.0, device)
+    t = fa.Tensor.from_numpy(device, _x(1, (1, 1, 4, 64)), fa.F32)
+    with pytest.raises(AssertionError, match="exceed"):
+        rc.apply(t, 5)            # positions 5..9 of 8
+    odd = fa.Tensor.from_numpy(device, _x(1, (1, 1, 4, 63)), fa.F32)
+    with pytest.raises(AssertionError, match="even"):
+        rc.apply(odd, 0)
+
+
+@pytest.mark.parametrize("cache_dtype,in_dtype", [(fa.F32, fa.F32), (fa.F16, fa.F32), (fa.F16, fa.F16)])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_kv_cache_rope_append_equals_rope_then_append(device, cache_dtype, in_dtype, interleaved):
+    """Growth, in-place appends and truncation to max_sequence_len, with the rotation fused into the write."""
+    B, Hkv, D, max_len = 2, 2, 64, 40
+    rc = fa.RopeCache(D, 128, 10000.0, device)
+    fused = fa.KvCache(2, max_len, cache_dtype, device)
+    ref_cache = oracle.KvCache(2, max_len)
+    fn = oracle.rope_interleaved if interleaved else oracle.rope
+    pos = 0
+    for step, n in enumerate([5, 1, 1, 9, 1, 17, 1, 1, 12, 3]):
+        k = _x(100 + step, (B, Hkv, n, D))
+        v = _x(200 + step, (B, Hkv, n, D))
+        tk, tv = fa.Tensor.from_numpy(device, k, in_dtype), fa.Tensor.from_numpy(device, v, in_dtype)
+        ka, va = fused.append_rope(rc, tk, tv, pos, interleaved)
+        k_rot = _cast_out(fn(rounded(k, in_dtype), rc.cos_host, rc.sin_host, pos), cache_dtype)
+        v_cast = _cast_out(rounded(v, in_dtype), cache_dtype)
+        rk, rv = ref_cache.append(k_rot, v_cast)
+        assert ka.shape == rk.shape and va.shape == rv.shape
+        assert np.array_equal(ka.to_numpy().view(np.uint8), np.ascontiguousarray(rk).view(np.uint8)), f"keys, step {step}"
+        assert np.array_equal(va.to_numpy().view(np.uint8), np.ascontiguousarray(rv).view(np.uint8)), f"values, step {step}"
+        pos += n
+    assert fused.current_seq_len() == max_len
