@@ -283,3 +283,24 @@ def test_fully_masked_row_is_nan(device):
     assert np.isnan(out[0, 0, 2]).all() and np.isnan(ref[0, 0, 2]).all()
     keep = [0, 1, 3]
     assert_parity(out[:, :, keep], ref[:, :, keep], TOL_F32, "unmasked rows")
+
+
+@pytest.mark.parametrize("dtype,Sq", [(fa.F16, 200), (fa.F32, 200), (fa.F16, 1), (fa.BF16, 70)])
+def test_output_written_as_batch_seq_heads_dim(device, dtype, Sq):
+    """The layout kalosm-llama needs next: attention output transposed to [B, Sq, H, D] and flattened for
+    attention_wo (attention_layer.rs:450-454).  The caller passes that buffer as a strided [B, H, Sq, D]
+    view and the kernels (tiled prefill, split-KV decode, general) write it in place of a transpose pass."""
+    B, H, Hkv, D, Skv = 2, 8, 2, 128, 300
+    q, k, v = _normal_qkv(17, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    analytic = (True, Skv - Sq, 0)
+    plain = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    for kernel in (fa.KERNEL_AUTO, fa.KERNEL_GENERIC):
+        buf = fa.Tensor.empty(device, (B, Sq, H, D), dtype)           # [B, Sq, H*D] once flattened
+        tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out=buf.transpose(1, 2), force_kernel=kernel)
+        got = buf.to_numpy().transpose(0, 2, 1, 3)
+        if kernel == fa.KERNEL_AUTO:
+            assert np.array_equal(got, plain), "same kernel, different output strides: bits must agree"
+        else:
+            tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+            assert_parity(got.astype(np.float32), plain.astype(np.float32), tol, "general kernel, transposed output")
