@@ -30,13 +30,17 @@ def test_c1_llama32_1b_prefill_f32(device):
     assert np.array_equal(am.host, oracle.get_mask(S, 0))  # bit-exact mask
     tq, tk, tv = (fa.Tensor.from_numpy(device, a) for a in (q, k, v))
     ref = oracle.flash_attention(q, k, v, 0.125, am.host, "qk")
-    # the reference call: dense QKMask (generic kernel) ...
-    out = tq.flash_attention(tk, tv, 0.125, (am.mask(), fa.MaskKind.QKMask)).to_numpy()
-    assert_parity(out, ref, TOL_F32, "C1 dense mask")
-    # ... and the analytic descriptor of the same mask (f32 MFMA kernel)
+    # the reference call: dense QKMask (reduced to intervals on the device, f32 MFMA kernel) ...
+    out_dense = tq.flash_attention(tk, tv, 0.125, (am.mask(), fa.MaskKind.QKMask)).to_numpy()
+    assert_parity(out_dense, ref, TOL_F32, "C1 dense mask")
+    # ... the general kernel on the same tensor ...
+    out_gen = tq.flash_attention(tk, tv, 0.125, (am.mask(), fa.MaskKind.QKMask), force_kernel=fa.KERNEL_GENERIC).to_numpy()
+    assert_parity(out_gen, ref, TOL_F32, "C1 dense mask, general kernel")
+    # ... and the analytic descriptor of the same mask (f32 MFMA kernel): bit-identical to the dense call
     assert tq.selected_kernel(tk, tv, 0.125, analytic=am.analytic) == fa.KERNEL_PREFILL_F32
     out = tq.flash_attention(tk, tv, 0.125, analytic=am.analytic).to_numpy()
     assert_parity(out, ref, TOL_F32, "C1 analytic")
+    assert np.array_equal(out, out_dense)
     assert np.array_equal(out[:, :, 0], np.repeat(v, H // Hkv, axis=1)[:, :, 0])  # causal row 0 == V[0]
 
 
@@ -73,6 +77,12 @@ def test_c3_llama3_8b_prefill_f16(device):
     ref = oracle.flash_attention(f32(q)[:, :, rows], f32(k), f32(v), D ** -0.5, mask, "qk")
     assert_parity(out[:, :, rows], ref, TOL_16, "C3 f16 out")
     assert_parity(out32[:, :, rows], ref, TOL_16, "C3 f32 out")
+    # the call as the reference's caller makes it, with the [8192, 8192] mask tensor of MaskCache (f16, 128 MiB):
+    # reduced to intervals on the device, same kernel, same bits
+    dense = fa.MaskCache(fa.F16).get_mask(S, 0, None, device)
+    out_dense = tq.flash_attention(tk, tv, D ** -0.5, (dense.mask(), fa.MaskKind.QKMask)).to_numpy()
+    assert np.array_equal(out_dense, out)
+    del dense, out_dense
     # whole-tensor properties: no NaN, row 0 == V[0] exactly, every output inside the range of V (convex combination)
     assert not np.isnan(out).any()
     assert np.array_equal(out[:, :, 0], np.repeat(v, H // Hkv, axis=1)[:, :, 0])
