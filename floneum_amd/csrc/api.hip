@@ -168,11 +168,11 @@ static bool rows_vectorizable(const fhip_tensor4 &t, int eb) {
 }
 
 static bool decode_eligible(const fhip_attn_args *a) {
-    if (a->dtype == FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
     if (a->q.shape[2] != 1) return false;
     if (D % 8 != 0 || D < 8 || D > 128) return false;
-    if (!rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
+    const int eb = a->dtype == FHIP_F32 ? 4 : 2;
+    if (!rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;
     if (a->k.stride[2] < 0 || a->v.stride[2] < 0) return false;
     return true;
 }
@@ -554,7 +554,7 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
         int chunk, nsplit;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
         const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2];
-        decode_plan(B, Hkv, H / Hkv, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr, &chunk, &nsplit);
+        decode_plan(B, Hkv, H / Hkv, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr, args->dtype == FHIP_F32, &chunk, &nsplit);
         *bytes = decode_workspace_bytes(B, H, Hkv, D, nsplit);
     }
     return FHIP_OK;
@@ -596,7 +596,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
-            decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr, &p.chunk, &p.nsplit);
+            decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr, args->dtype == FHIP_F32, &p.chunk, &p.nsplit);
             const size_t need = decode_workspace_bytes(p.B, p.H, p.Hkv, p.D, p.nsplit);
             if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
                 set_error("decode needs a workspace of %zu bytes, got %zu", need,

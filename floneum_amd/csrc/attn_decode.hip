@@ -37,24 +37,24 @@ static int env_int(const char *name, int dflt) {
     return v > 0 ? v : dflt;
 }
 
-static int decode_gt(int G, int D);
-
-static bool decode_use_mfma(int D) {
-    return (D == 32 || D == 64 || D == 96 || D == 128) && env_int("FHIP_DECODE_VARIANT", 1) == 1;
+// the matrix-core variant takes 16-bit tensors; f32 tensors run on the vector variant
+static bool decode_use_mfma(int D, bool f32) {
+    return !f32 && (D == 32 || D == 64 || D == 96 || D == 128) && env_int("FHIP_DECODE_VARIANT", 1) == 1;
 }
 
 // query heads handled by one workgroup
-static int decode_gt(int G, int D) {
-    if (decode_use_mfma(D)) return 16;
+static int decode_gt(int G, int D, bool f32) {
+    if (decode_use_mfma(D, f32)) return 16;
     return G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
 }
 
-void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, int *chunk, int *nsplit) {
-    const int gt = decode_gt(G, D);
+void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, bool f32, int *chunk,
+                 int *nsplit) {
+    const int gt = decode_gt(G, D, f32);
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
     // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more
-    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", decode_use_mfma(D) ? 2 : 4);
+    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", decode_use_mfma(D, f32) ? 2 : 4);
     const long target = (long)compute_units * wgs_per_cu;
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
@@ -82,11 +82,51 @@ size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit) {
 // ---- element helpers ---------------------------------------------------------------------------
 
 template <typename T>
-struct Vec8;  // 8 consecutive 16-bit elements in four 32-bit registers
+struct Vec8;  // 8 consecutive elements of a row: four 32-bit registers for 16-bit types, eight for f32
+
+// shared by the 16-bit specialisations
+struct Vec8Bits16 {
+    uint4_t r;
+    __device__ __forceinline__ void zero() { r = uint4_t{0, 0, 0, 0}; }
+    __device__ __forceinline__ void load(const void *p) { r = *(const uint4_t *)p; }
+    // 8 elements `stride` apart (the query row, which may have any stride)
+    __device__ __forceinline__ void gather(const void *p, int64_t stride) {
+        const uint16_t *q = (const uint16_t *)p;
+        uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 8; e++) w[e >> 1] |= (uint32_t)q[e * stride] << ((e & 1) * 16);
+        r = uint4_t{w[0], w[1], w[2], w[3]};
+    }
+};
 
 template <>
-struct Vec8<half_t> {
-    uint4_t r;
+struct Vec8<float> {
+    float4_t a, b;
+    __device__ __forceinline__ void zero() { a = b = float4_t{0.f, 0.f, 0.f, 0.f}; }
+    __device__ __forceinline__ void load(const void *p) {
+        a = *(const float4_t *)p;
+        b = *((const float4_t *)p + 1);
+    }
+    __device__ __forceinline__ void gather(const void *p, int64_t stride) {
+        const float *q = (const float *)p;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            a[e] = q[e * stride];
+            b[e] = q[(e + 4) * stride];
+        }
+    }
+    __device__ __forceinline__ float get(int e) const { return e < 4 ? a[e] : b[e - 4]; }
+    __device__ __forceinline__ float dot(const Vec8 &o, float acc) const {
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = fmaf(a[e], o.a[e], acc);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = fmaf(b[e], o.b[e], acc);
+        return acc;
+    }
+};
+
+template <>
+struct Vec8<half_t> : Vec8Bits16 {
     __device__ __forceinline__ float dot(const Vec8 &o, float acc) const {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -103,8 +143,7 @@ struct Vec8<half_t> {
 };
 
 template <>
-struct Vec8<bf16_t> {
-    uint4_t r;
+struct Vec8<bf16_t> : Vec8Bits16 {
     __device__ __forceinline__ float get(int e) const {
         typedef uint16_t ushort8_t __attribute__((ext_vector_type(8)));
         const ushort8_t a = __builtin_bit_cast(ushort8_t, r);
@@ -169,20 +208,13 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
 #pragma unroll
     for (int hh = 0; hh < GT; hh++) {
         const int h = h0 + min(hh, nh - 1);
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1];
-        uint32_t w[4] = {0, 0, 0, 0};
-        if (active) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t x = qp[(int64_t)(c * 8 + e) * p.qs[3]];
-                w[e >> 1] |= x << ((e & 1) * 16);
-            }
-        }
-        q[hh].r = uint4_t{w[0], w[1], w[2], w[3]};
+        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1];
+        q[hh].zero();
+        if (active) q[hh].gather(qp + (int64_t)(c * 8) * p.qs[3], p.qs[3]);
     }
 
-    const uint16_t *kbase = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1] + c * 8;
-    const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1] + c * 8;
+    const T *kbase = (const T *)p.k + b * p.ks[0] + g * p.ks[1] + c * 8;
+    const T *vbase = (const T *)p.v + b * p.vs[0] + g * p.vs[1] + c * 8;
     const T *mrow = nullptr;
     if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask;
     if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const T *)p.mask + b * p.ms0;
@@ -206,11 +238,11 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
         for (int u = 0; u < U; u++) {
             key[u] = base + (u * DEC_WAVES + wave) * KPI + r;
             const bool ok = active && key[u] >= lo && key[u] < hi;
-            kk[u].r = uint4_t{0, 0, 0, 0};
-            vv[u].r = uint4_t{0, 0, 0, 0};
+            kk[u].zero();
+            vv[u].zero();
             if (ok) {
-                kk[u].r = *(const uint4_t *)(kbase + (int64_t)key[u] * p.ks[2]);
-                vv[u].r = *(const uint4_t *)(vbase + (int64_t)key[u] * p.vs[2]);
+                kk[u].load(kbase + (int64_t)key[u] * p.ks[2]);
+                vv[u].load(vbase + (int64_t)key[u] * p.vs[2]);
             }
         }
         float s[U][GT];
@@ -660,7 +692,8 @@ static void launch_vec(const AttnParams &p, dim3 grid, hipStream_t stream, int g
 
 template <typename T>
 static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
-    const int gt = decode_gt(p.G, p.D);
+    constexpr bool F32 = sizeof(T) == 4;
+    const int gt = decode_gt(p.G, p.D, F32);
     const int hb = (p.G + gt - 1) / gt;
     const long gy = (long)p.B * p.Hkv * hb;
     if (gy > 65535 || p.nsplit > 0x7fffffff) {
@@ -668,14 +701,24 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     dim3 grid((unsigned)p.nsplit, (unsigned)gy), block(64 * DEC_WAVES);
-    if (decode_use_mfma(p.D)) {
-        switch (p.D) {
-            case 32: hipLaunchKernelGGL((decode_mfma_kernel<T, 32>), grid, block, 0, stream, p); break;
-            case 64: hipLaunchKernelGGL((decode_mfma_kernel<T, 64>), grid, block, 0, stream, p); break;
-            case 96: hipLaunchKernelGGL((decode_mfma_kernel<T, 96>), grid, block, 0, stream, p); break;
-            default: hipLaunchKernelGGL((decode_mfma_kernel<T, 128>), grid, block, 0, stream, p); break;
+    if constexpr (!F32) {
+        if (decode_use_mfma(p.D, false)) {
+            switch (p.D) {
+                case 32: hipLaunchKernelGGL((decode_mfma_kernel<T, 32>), grid, block, 0, stream, p); break;
+                case 64: hipLaunchKernelGGL((decode_mfma_kernel<T, 64>), grid, block, 0, stream, p); break;
+                case 96: hipLaunchKernelGGL((decode_mfma_kernel<T, 96>), grid, block, 0, stream, p); break;
+                default: hipLaunchKernelGGL((decode_mfma_kernel<T, 128>), grid, block, 0, stream, p); break;
+            }
+            FHIP_HIP_CHECK(hipGetLastError());
+            if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
+            if (p.nsplit > 1) {
+                hipLaunchKernelGGL(decode_combine_kernel<T>, dim3((unsigned)(p.B * p.H)), dim3(64), 0, stream, p);
+                FHIP_HIP_CHECK(hipGetLastError());
+            }
+            return FHIP_OK;
         }
-    } else if (p.D <= 32) {
+    }
+    if (p.D <= 32) {
         launch_vec<T, 4>(p, grid, stream, gt);
     } else if (p.D <= 64) {
         launch_vec<T, 8>(p, grid, stream, gt);
@@ -694,8 +737,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
 int launch_decode(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
     if (dtype == FHIP_F16) return launch_decode_t<half_t>(p, stream);
     if (dtype == FHIP_BF16) return launch_decode_t<bf16_t>(p, stream);
-    set_error("decode kernel takes f16/bf16 only");
-    return FHIP_ERR_UNSUPPORTED;
+    return launch_decode_t<float>(p, stream);
 }
 
 }  // namespace fhip

@@ -58,8 +58,10 @@ int launch_decode(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 int launch_prefill_f32(const AttnParams &p, hipStream_t stream);
 
-// decode planning (host): keys per split and number of splits; `ragged`: per-batch key counts are given
-void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, int *chunk, int *nsplit);
+// decode planning (host): keys per split and number of splits; `ragged`: per-batch key counts are given;
+// `f32`: the tensors are f32 (vector variant) rather than 16-bit
+void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, bool f32, int *chunk,
+                 int *nsplit);
 size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 
 // KV cache copies

@@ -127,9 +127,11 @@ typedef struct {
 typedef enum {
     FHIP_KERNEL_AUTO = 0,
     FHIP_KERNEL_GENERIC = 1,     /* any dtype, any strides, any mask; one wavefront per query row   */
-    FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim in {64,96,128}, LDS-tiled MFMA               */
+    FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim in {64,96,128}, LDS-tiled MFMA; masks by
+                                    interval (analytic, kv_lens, or a mask tensor reduced on the device) */
     FHIP_KERNEL_PREFILL_F32 = 3, /* f32, head_dim multiple of 32 up to 128, f32 MFMA                */
-    FHIP_KERNEL_DECODE_SPLITKV = 4 /* f16/bf16, Sq == 1, split-KV streaming + LSE combine           */
+    FHIP_KERNEL_DECODE_SPLITKV = 4 /* Sq == 1, split-KV streaming + LSE combine (matrix cores for
+                                      f16/bf16, vector units for f32)                                */
 } fhip_kernel_id;
 
 

@@ -136,9 +136,10 @@ def test_kernel_selection():
     assert selected(make_args(Sq=512, Skv=512, D=64, dtype=fa.F32))[1] == fa.KERNEL_PREFILL_F32
     assert selected(make_args(Sq=1, Skv=4096, D=128))[1] == fa.KERNEL_DECODE_SPLITKV
     assert selected(make_args(Sq=1, Skv=4096, D=96, dtype=fa.BF16))[1] == fa.KERNEL_DECODE_SPLITKV
-    assert selected(make_args(Sq=1, Skv=4096, D=128, dtype=fa.F32))[1] == fa.KERNEL_PREFILL_F32
+    # f32 decode (kalosm-llama's cache is f32, attention_layer.rs:400-403) streams through the split-KV kernel too
+    assert selected(make_args(Sq=1, Skv=4096, D=128, dtype=fa.F32))[1] == fa.KERNEL_DECODE_SPLITKV
     assert selected(make_args(Sq=7, Skv=9, D=33))[1] == fa.KERNEL_GENERIC
-    # a dense additive mask (arbitrary bias in the reference's fuzz test) goes to the generic kernel
+    # a dense additive mask without the scratch its interval form needs goes to the general kernel
     a = make_args(Sq=64, Skv=64, D=128)
     a.mask_kind = fa.MaskKind.QKMask
     a.mask.ptr = FAKE

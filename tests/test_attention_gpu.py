@@ -208,7 +208,7 @@ def test_prefill_tiled(device, dtype, D, case):
         assert_parity(out_g, ref, tol, f"generic {case} D{D}")
 
 
-@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
                                      (2, 40, 333), (8, 8, 100)])
@@ -219,8 +219,36 @@ def test_decode_splitkv(device, dtype, G, D, Skv):
     assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
     out = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
     ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5)
-    tol = dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16)
     assert_parity(out, ref, tol, f"decode G{G} D{D} Skv{Skv}")
+
+
+def test_decode_f32_with_the_masks_the_reference_passes(device):
+    """kalosm-llama decodes in f32 with get_mask(1, pos, window) as a QKMask (raw/mod.rs:618-620,
+    attention_layer.rs:400-448); a padded batch would come as a BatchKeyMask."""
+    B, H, Hkv, D, Skv = 2, 8, 2, 128, 1500
+    q, k, v = _normal_qkv(18, B, H, Hkv, 1, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    qk = oracle.get_mask(1, Skv - 1, None)                       # [1, 1500] zeros
+    assert qk.shape == (1, Skv)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (fa.Tensor.from_numpy(device, qk, fa.F32), fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, qk, "qk")
+    assert_parity(out, ref, TOL_F32, "f32 decode, QKMask")
+    bk = np.zeros((B, Skv), np.float32)
+    bk[0, 1000:] = NEG_INF
+    bk[1, :200] = NEG_INF
+    out = tq.flash_attention(tk, tv, D ** -0.5, (fa.Tensor.from_numpy(device, bk, fa.F32), fa.MaskKind.BatchKeyMask)).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, bk, "batch_key")
+    assert_parity(out, ref, TOL_F32, "f32 decode, BatchKeyMask")
+    # cached K/V arrive as narrowed views of a power-of-two allocation (tensor_cache.rs:107-110)
+    kbuf = np.zeros((B, Hkv, 2048, D), np.float32)
+    vbuf = np.zeros((B, Hkv, 2048, D), np.float32)
+    kbuf[:, :, :Skv], vbuf[:, :, :Skv] = k, v
+    tkn = fa.Tensor.from_numpy(device, kbuf, fa.F32).narrow(2, 0, Skv)
+    tvn = fa.Tensor.from_numpy(device, vbuf, fa.F32).narrow(2, 0, Skv)
+    assert tq.selected_kernel(tkn, tvn, 0.1) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tkn, tvn, D ** -0.5).to_numpy()
+    assert_parity(out, oracle.flash_attention(q, k, v, D ** -0.5), TOL_F32, "f32 decode, cache views")
 
 
 def test_decode_ragged_kv_lens(device):
