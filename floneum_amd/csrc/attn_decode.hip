@@ -53,8 +53,10 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     const int gt = decode_gt(G, D, f32);
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
-    // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more
-    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", decode_use_mfma(D, f32) ? 2 : 4);
+    // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more; f32 rows carry
+    // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at
+    // batch 1 with 32768 keys)
+    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", (decode_use_mfma(D, f32) || f32) ? 2 : 4);
     const long target = (long)compute_units * wgs_per_cu;
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
