@@ -11,6 +11,12 @@
 // Products and sums are f32 throughout (no reduced-precision operand), which is what the f32
 // tolerance (relative L2 1e-5 against the reference's f32 CPU path) needs.
 //
+// Short prompts leave most of the chip idle with 128 rows per workgroup, and the f32 matrix rate makes
+// the longest wavefront's tile sequence the critical path.  The kernel therefore also comes in key-split
+// forms (template parameter S = 2, 4): the four wavefronts form S groups that own the SAME 128 / S query
+// rows, group g walks the key tiles t with t % S == g through its own LDS buffers, and the groups'
+// (m, l, O) states are merged through LDS at the end.  S times the workgroups, 1 / S of the tiles each.
+//
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199; this is the data
 // type kalosm-llama always calls with (models/kalosm-llama/src/raw/attention_layer.rs:400-448).
 #include "attn_bounds.h"
@@ -20,7 +26,6 @@
 namespace fhip {
 
 constexpr int PF32_WAVES = 4;
-constexpr int PF32_BM = 32 * PF32_WAVES;
 constexpr int PF32_BN = 32;
 constexpr float PF32_LOG2E = 1.4426950408889634f;
 
@@ -35,21 +40,29 @@ __device__ __forceinline__ float half_swap_sum32(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <int D>
+template <int D, int S>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnParams p, int nqb) {
+    constexpr int WPG = PF32_WAVES / S;   // wavefronts per key-split group
+    constexpr int BM = 32 * WPG;          // query rows per workgroup
     constexpr int KP = D * 4 + 16;  // row pitch in bytes: rows 4 banks apart -> conflict-free b128 reads
     constexpr int K_BYTES = PF32_BN * KP;
     constexpr int CPR = D / 4;      // 16-byte chunks per row
-    constexpr int NCH = PF32_BN * CPR / (64 * PF32_WAVES);
-    __shared__ __attribute__((aligned(16))) char smem[2 * K_BYTES];
+    constexpr int GT = 64 * WPG;    // threads of a group
+    constexpr int NCH = PF32_BN * CPR / GT;
+    static_assert(PF32_BN * CPR % GT == 0, "a group's threads must cover a tile evenly");
+    __shared__ __attribute__((aligned(16))) char smem[S * 2 * K_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int ln = lane & 31;
     const int h2 = lane >> 5;
+    const int grp = wave / WPG;     // key-split group
+    const int wig = wave % WPG;     // wavefront inside the group: which 32 rows
+    const int gtid = tid % GT;      // thread inside the group
+    const int gbase = grp * 2 * K_BYTES;  // the group's tile buffers
 
     const int bh_count = p.B * p.H;
     const int id = blockIdx.x;
@@ -60,10 +73,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
 
-    const int q0 = qb * PF32_BM;
-    const int qw0 = q0 + 32 * wave;
+    const int q0 = qb * BM;
+    const int qw0 = q0 + 32 * wig;
     const int query = qw0 + ln;
-    const RowBounds rb = row_bounds(p, b, q0, PF32_BM, qw0, lane);
+    const RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
     const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const bool wave_has_rows = qw0 < p.Sq;
 
@@ -90,7 +103,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     auto load_tile = [&](int j0) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int cid = tid + 64 * PF32_WAVES * i;
+            const int cid = gtid + GT * i;
             const int row = cid / CPR, col = cid % CPR;
             const int key = min(j0 + row, p.Skv - 1);
             kst[i] = *(const float4_t *)(kg + (int64_t)key * p.ks[2] + col * 4);
@@ -100,23 +113,30 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     auto store_tile = [&]() {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const int cid = tid + 64 * PF32_WAVES * i;
+            const int cid = gtid + GT * i;
             const int row = cid / CPR, col = cid % CPR;
-            *LDS32_PTR(float4_t, row * KP + col * 16) = kst[i];
-            *LDS32_PTR(float4_t, K_BYTES + row * KP + col * 16) = vst[i];
+            *LDS32_PTR(float4_t, gbase + row * KP + col * 16) = kst[i];
+            *LDS32_PTR(float4_t, gbase + K_BYTES + row * KP + col * 16) = vst[i];
         }
     };
 
+    // group g takes the tiles j_begin + (it * S + g) * 32; every group runs the same number of iterations
+    // (the barriers are workgroup-wide), a group without a tile in the last one idles through it
     const int j_begin = (lo_wg / PF32_BN) * PF32_BN;
-    if (j_begin < hi_wg) load_tile(j_begin);
+    const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PF32_BN - 1) / PF32_BN : 0;
+    const int niter = (ntiles + S - 1) / S;
+    if (grp < ntiles) load_tile(j_begin + grp * PF32_BN);
 
-    for (int j0 = j_begin; j0 < hi_wg; j0 += PF32_BN) {
+    for (int it = 0; it < niter; it++) {
+        const int t = it * S + grp;
+        const int j0 = j_begin + t * PF32_BN;
+        const bool have = t < ntiles;
         lds_barrier();  // everyone finished reading the previous tile (LDS-only barrier: the prefetch
-        store_tile();   // issued below stays in flight across the math)
+        if (have) store_tile();  // issued below stays in flight across the math)
         lds_barrier();
-        if (j0 + PF32_BN < hi_wg) load_tile(j0 + PF32_BN);
+        if (t + S < ntiles) load_tile(j0 + S * PF32_BN);
 
-        const bool tile_visible = wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;
+        const bool tile_visible = have && wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;
         if (!tile_visible) continue;
 
         // S^T: contraction step (kc, i) uses dim 8 kc + 4 h2 + i on both operands
@@ -125,7 +145,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         for (int r = 0; r < 16; r++) s[r] = 0.0f;
 #pragma unroll
         for (int kc = 0; kc < D / 8; kc++) {
-            const float4_t a = *LDS32_PTR(float4_t, ln * KP + (8 * kc + 4 * h2) * 4);
+            const float4_t a = *LDS32_PTR(float4_t, gbase + ln * KP + (8 * kc + 4 * h2) * 4);
 #pragma unroll
             for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[kc][i], s, 0, 0, 0);
         }
@@ -165,12 +185,46 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             const int krow = 8 * (r >> 2) + 4 * h2 + (r & 3);
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
-                const float a = *LDS32_PTR(float, K_BYTES + krow * KP + (32 * db + ln) * 4);
+                const float a = *LDS32_PTR(float, gbase + K_BYTES + krow * KP + (32 * db + ln) * 4);
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db], 0, 0, 0);
             }
         }
     }
 
+    if constexpr (S > 1) {
+        // merge the groups: groups 1.. park (m, l, O) in LDS, one value per lane and register, group 0
+        // folds them into its own state (log-sum-exp merge, as the split-KV combine does)
+        constexpr int NR = 16 * (D / 32) + 2;            // registers per lane
+        static_assert((S - 1) * WPG * NR * 256 <= S * 2 * K_BYTES, "merge staging exceeds the tile buffers");
+        lds_barrier();  // the tile buffers are free
+        if (grp > 0) {
+            const int slot = ((grp - 1) * WPG + wig) * NR * 256 + lane * 4;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) *LDS32_PTR(float, slot + (16 * db + r) * 256) = o[db][r];
+            *LDS32_PTR(float, slot + (NR - 2) * 256) = m;
+            *LDS32_PTR(float, slot + (NR - 1) * 256) = l;
+        }
+        lds_barrier();
+        if (grp > 0) return;
+#pragma unroll
+        for (int gsrc = 1; gsrc < S; gsrc++) {
+            const int slot = ((gsrc - 1) * WPG + wig) * NR * 256 + lane * 4;
+            const float m_other = *LDS32_PTR(float, slot + (NR - 2) * 256);
+            const float l_other = *LDS32_PTR(float, slot + (NR - 1) * 256);
+            const float m_all = fmaxf(m, m_other);
+            const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+            const float wa = __builtin_amdgcn_exp2f(m - m_safe), wb = __builtin_amdgcn_exp2f(m_other - m_safe);
+            l = l * wa + l_other * wb;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    o[db][r] = o[db][r] * wa + *LDS32_PTR(float, slot + (16 * db + r) * 256) * wb;
+            m = m_all;
+        }
+    }
     const float l_tot = half_swap_sum32(l);
     if (query < p.Sq) {
         float *op = (float *)p.out + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
@@ -184,8 +238,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     }
 }
 
-int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
-    const int nqb = (p.Sq + PF32_BM - 1) / PF32_BM;
+template <int S>
+static int launch_split(const AttnParams &p, hipStream_t stream) {
+    constexpr int BM = 32 * (PF32_WAVES / S);
+    const int nqb = (p.Sq + BM - 1) / BM;
     const long blocks = (long)nqb * p.B * p.H;
     if (blocks > 0x7fffffffL) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
@@ -193,14 +249,36 @@ int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
     switch (p.D) {
-        case 32: hipLaunchKernelGGL(prefill_f32_kernel<32>, grid, block, 0, stream, p, nqb); break;
-        case 64: hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, stream, p, nqb); break;
-        case 96: hipLaunchKernelGGL(prefill_f32_kernel<96>, grid, block, 0, stream, p, nqb); break;
-        case 128: hipLaunchKernelGGL(prefill_f32_kernel<128>, grid, block, 0, stream, p, nqb); break;
+        case 32: hipLaunchKernelGGL((prefill_f32_kernel<32, S>), grid, block, 0, stream, p, nqb); break;
+        case 64: hipLaunchKernelGGL((prefill_f32_kernel<64, S>), grid, block, 0, stream, p, nqb); break;
+        case 96:
+            if constexpr (S <= 2) hipLaunchKernelGGL((prefill_f32_kernel<96, S>), grid, block, 0, stream, p, nqb);
+            break;
+        case 128:
+            if constexpr (S <= 2) hipLaunchKernelGGL((prefill_f32_kernel<128, S>), grid, block, 0, stream, p, nqb);
+            break;
         default: set_error("prefill f32 kernel: head_dim %d not in {32, 64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
+}
+
+int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
+    // Split the keys of a query block over 2 or 4 wavefront groups while the unsplit grid is only a few
+    // workgroups per CU: the longest (last causal) query block then sets the run time, and halving it pays
+    // even when every CU has work.  Measured break-even: about 4 workgroups per CU at head_dim <= 64, 2 above
+    // (the bigger tiles leave less to gain).  A single wavefront moves a whole tile only up to head_dim 64.
+    int cus = 256, dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const long bh = (long)p.B * p.H;
+    const long wg1 = bh * ((p.Sq + 127) / 128), wg2 = bh * ((p.Sq + 63) / 64);
+    const bool small_dim = p.D <= 64;
+    int split = 1;
+    if (wg1 <= (small_dim ? 4L : 2L) * cus) split = 2;
+    if (split == 2 && small_dim && wg2 < 2L * cus) split = 4;
+    if (split == 4) return launch_split<4>(p, stream);
+    if (split == 2) return launch_split<2>(p, stream);
+    return launch_split<1>(p, stream);
 }
 
 }  // namespace fhip

@@ -208,6 +208,29 @@ def test_prefill_tiled(device, dtype, D, case):
         assert_parity(out_g, ref, tol, f"generic {case} D{D}")
 
 
+@pytest.mark.parametrize("D,B,H,Sq,Skv,analytic,form", [
+    (64, 1, 4, 200, 200, (True, 0, 0), "four groups"),
+    (64, 1, 8, 95, 700, (True, 605, 150), "four groups, window and cached keys"),
+    (32, 1, 6, 333, 333, None, "four groups, no mask"),
+    (64, 2, 32, 700, 700, (True, 0, 0), "two groups"),
+    (64, 4, 48, 900, 900, (True, 0, 300), "one group"),
+    (128, 1, 4, 300, 300, (True, 0, 0), "two groups"),
+    (96, 1, 4, 161, 417, (True, 256, 0), "two groups, cached keys"),
+    (128, 2, 40, 1000, 1000, (True, 0, 0), "one group"),
+])
+def test_prefill_f32_key_split_forms(device, D, B, H, Sq, Skv, analytic, form):
+    """The f32 kernel splits a query block's keys over 1, 2 or 4 wavefront groups depending on how many
+    workgroups the call has; each form is checked at ragged sizes (the grid sizes here select the form named)."""
+    Hkv = H // 2
+    q, k, v = _normal_qkv(12, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == fa.KERNEL_PREFILL_F32
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    mask = None if analytic is None else _analytic_mask(Sq, Skv, *analytic)
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk" if mask is not None else None)
+    assert_parity(out, ref, TOL_F32, f"f32 D{D} {form}")
+
+
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
