@@ -83,6 +83,10 @@ class CRopeTables(ctypes.Structure):
                 ("start_pos", ctypes.c_uint64), ("interleaved", ctypes.c_int32)]
 
 
+class CRmsNorm(ctypes.Structure):
+    _fields_ = [("weight", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("dtype", ctypes.c_int), ("eps", ctypes.c_float)]
+
+
 SYMBOLS = {
     "fhip_last_error": (ctypes.c_char_p, []),
     "fhip_version": (ctypes.c_char_p, []),
@@ -130,6 +134,11 @@ SYMBOLS = {
     "fhip_kv_cache_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4)]),
+    "fhip_norm_rope": (ctypes.c_int, [_P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
+                                      ctypes.c_int, ctypes.POINTER(CTensor4), ctypes.c_int]),
+    "fhip_kv_cache_norm_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRopeTables),
+                                                      ctypes.POINTER(CTensor4), ctypes.POINTER(CTensor4), ctypes.c_int,
+                                                      ctypes.POINTER(CTensor4), ctypes.POINTER(CTensor4)]),
 }
 
 _LIB = None
@@ -574,15 +583,22 @@ class KvCache:
 
         return wrap(ka), wrap(va)
 
-    def append_rope(self, rope, k, v, start_pos, interleaved=False):
+    def append_rope(self, rope, k, v, start_pos, interleaved=False, k_norm=None):
         """append(rope(k), v) in one pass: the keys are rotated (RopeCache.forward semantics) and both
-        tensors converted from their own element type to the cache's on the way into the cache."""
+        tensors converted from their own element type to the cache's on the way into the cache.  With
+        k_norm (an RmsNorm) the keys are normalised before the rotation (attention_k_norm)."""
         assert k.dtype == v.dtype
         ck, cv = k._c4(), v._c4()
         ka, va = CTensor4(), CTensor4()
         tables = rope._tables(start_pos, interleaved)
-        check(lib().fhip_kv_cache_rope_append(self.handle, self.device.stream, ctypes.byref(tables), ctypes.byref(ck),
-                                              ctypes.byref(cv), k.dtype, ctypes.byref(ka), ctypes.byref(va)))
+        if k_norm is None:
+            check(lib().fhip_kv_cache_rope_append(self.handle, self.device.stream, ctypes.byref(tables), ctypes.byref(ck),
+                                                  ctypes.byref(cv), k.dtype, ctypes.byref(ka), ctypes.byref(va)))
+        else:
+            cn = k_norm._c()
+            check(lib().fhip_kv_cache_norm_rope_append(self.handle, self.device.stream, ctypes.byref(cn),
+                                                       ctypes.byref(tables), ctypes.byref(ck), ctypes.byref(cv), k.dtype,
+                                                       ctypes.byref(ka), ctypes.byref(va)))
 
         def wrap(c):
             return Tensor(_View(self.device, c.ptr, self), self.dtype, tuple(c.shape), tuple(c.stride), c.offset)
@@ -624,13 +640,19 @@ class RopeCache:
     def _tables(self, start_pos, interleaved):
         return CRopeTables(self.cos.buffer.ptr, self.sin.buffer.ptr, self.rows, start_pos, 1 if interleaved else 0)
 
-    def apply(self, x, start_pos, interleaved=False, out_dtype=None):
-        """Tensor::rope_normal_fused / rope_fused with the tables narrowed to start_pos.. (rope.rs:139-175)."""
+    def apply(self, x, start_pos, interleaved=False, out_dtype=None, norm=None):
+        """Tensor::rope_normal_fused / rope_fused with the tables narrowed to start_pos.. (rope.rs:139-175);
+        with norm (an RmsNorm) the rows are normalised first, in the same pass."""
         out = Tensor.empty(self.device, x.shape, out_dtype if out_dtype is not None else x.dtype)
         cx, co = x._c4(), out._c4()
         tables = self._tables(start_pos, interleaved)
-        check(lib().fhip_rope(self.device.stream, ctypes.byref(tables), ctypes.byref(cx), x.dtype, ctypes.byref(co),
-                              out.dtype))
+        if norm is None:
+            check(lib().fhip_rope(self.device.stream, ctypes.byref(tables), ctypes.byref(cx), x.dtype, ctypes.byref(co),
+                                  out.dtype))
+        else:
+            cn = norm._c()
+            check(lib().fhip_norm_rope(self.device.stream, ctypes.byref(cn), ctypes.byref(tables), ctypes.byref(cx),
+                                       x.dtype, ctypes.byref(co), out.dtype))
         return out
 
     def forward(self, q, k, start_pos):
@@ -638,3 +660,27 @@ class RopeCache:
 
     def forward_interleaved(self, q, k, start_pos):
         return self.apply(q, start_pos, True), self.apply(k, start_pos, True)
+
+
+class RmsNorm:
+    """fusor::layers::RmsNorm<1, T> over the last dimension (fusor-ml/fusor/src/layers/rms_norm.rs:11-133): the
+    q / k norm of blocks that have attention_q_norm / attention_k_norm."""
+
+    def __init__(self, weight, bias=None, eps=1e-5, dtype=F32, device=None):
+        self.device = device or Device.default()
+        self.dtype = dtype
+        self.eps = float(eps)
+        self.weight = Tensor.from_numpy(self.device, np.asarray(weight, np.float32).reshape(1, -1), dtype)
+        self.bias = None if bias is None else Tensor.from_numpy(self.device, np.asarray(bias, np.float32).reshape(1, -1), dtype)
+
+    def _c(self):
+        return CRmsNorm(self.weight.buffer.ptr, self.bias.buffer.ptr if self.bias is not None else None, self.dtype,
+                        self.eps)
+
+    def forward_generic_4d(self, x, out_dtype=None):
+        """RmsNorm::forward_generic_4d (rms_norm.rs:122-133): the norm alone."""
+        out = Tensor.empty(self.device, x.shape, out_dtype if out_dtype is not None else x.dtype)
+        cx, co, cn = x._c4(), out._c4(), self._c()
+        check(lib().fhip_norm_rope(self.device.stream, ctypes.byref(cn), None, ctypes.byref(cx), x.dtype,
+                                   ctypes.byref(co), out.dtype))
+        return out

@@ -747,6 +747,7 @@ static uint64_t next_pow2(uint64_t x) {
 struct NewRows {
     fhip_dtype src_dtype;
     const fhip_rope_tables *rope;  // nullptr: plain copy
+    const fhip_rms_norm *k_norm;   // with rope: the keys are normalised first (nullptr: not)
 };
 
 // rows [first, first + count) of the new block `src` -> dst (cache dtype, strides dst_st); side 0 = keys
@@ -757,8 +758,10 @@ static int write_new_rows(const fhip_kv_cache *c, hipStream_t st, int side, cons
     const char *sp = (const char *)src->ptr + (src->offset + first * src->stride[2]) * (uint64_t)seb;
     if (!nr.rope) return launch_copy_rows(sp, src->stride, dst, dst_st, shp, seb, st);
     const int mode = side == 0 ? (nr.rope->interleaved ? 1 : 0) : 2;
+    fhip::RowNorm norm;
+    if (side == 0 && nr.k_norm) norm = {nr.k_norm->weight, nr.k_norm->bias, nr.k_norm->dtype, nr.k_norm->eps};
     return launch_rope_rows(sp, src->stride, nr.src_dtype, dst, dst_st, c->dtype, shp, nr.rope->cos, nr.rope->sin,
-                            (int64_t)(nr.rope->start_pos + first), mode, st);
+                            (int64_t)(nr.rope->start_pos + first), mode, side == 0 && nr.k_norm ? &norm : nullptr, st);
 }
 
 extern "C" {
@@ -968,6 +971,7 @@ int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k
     NewRows nr;
     nr.src_dtype = c ? c->dtype : FHIP_F32;
     nr.rope = nullptr;
+    nr.k_norm = nullptr;
     return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
 }
 
@@ -988,8 +992,16 @@ static int check_rope(const fhip_rope_tables *r, uint32_t head_dim, uint64_t row
     return FHIP_OK;
 }
 
-int fhip_rope(fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *x, fhip_dtype x_dtype, const fhip_tensor4 *out,
-              fhip_dtype out_dtype) {
+static int check_norm(const fhip_rms_norm *n) {
+    if (!n || !n->weight || !fhip::dtype_ok(n->dtype)) {
+        set_error("rms norm: NULL weight or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    return FHIP_OK;
+}
+
+static int rope_core(fhip_stream *s, const fhip_rms_norm *norm, const fhip_rope_tables *rope, const fhip_tensor4 *x,
+                     fhip_dtype x_dtype, const fhip_tensor4 *out, fhip_dtype out_dtype) {
     if (!s || !x || !out || !x->ptr || !out->ptr || !fhip::dtype_ok(x_dtype) || !fhip::dtype_ok(out_dtype)) {
         set_error("rope: NULL argument or bad dtype");
         return FHIP_ERR_INVALID_ARG;
@@ -999,17 +1011,46 @@ int fhip_rope(fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *
             set_error("rope: output shape differs from the input shape");
             return FHIP_ERR_INVALID_ARG;
         }
-    int rc = check_rope(rope, x->shape[3], x->shape[2]);
+    int rc = FHIP_OK;
+    if (rope) rc = check_rope(rope, x->shape[3], x->shape[2]);
+    else if (x->shape[3] == 0 || x->shape[3] % 2 != 0) {
+        set_error("rms norm: head_dim %u must be even", x->shape[3]);
+        rc = FHIP_ERR_INVALID_ARG;
+    }
     if (rc) return rc;
+    fhip::RowNorm rn;
+    if (norm) {
+        rc = check_norm(norm);
+        if (rc) return rc;
+        rn = {norm->weight, norm->bias, norm->dtype, norm->eps};
+    }
     FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     const char *sp = (const char *)x->ptr + x->offset * (uint64_t)fhip::elem_bytes(x_dtype);
     char *dp = (char *)out->ptr + out->offset * (uint64_t)fhip::elem_bytes(out_dtype);
-    return launch_rope_rows(sp, x->stride, x_dtype, dp, out->stride, out_dtype, x->shape, rope->cos, rope->sin,
-                            (int64_t)rope->start_pos, rope->interleaved ? 1 : 0, s->s);
+    return launch_rope_rows(sp, x->stride, x_dtype, dp, out->stride, out_dtype, x->shape, rope ? rope->cos : nullptr,
+                            rope ? rope->sin : nullptr, rope ? (int64_t)rope->start_pos : 0,
+                            rope ? (rope->interleaved ? 1 : 0) : 2, norm ? &rn : nullptr, s->s);
 }
 
-int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *k_new,
-                              const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+int fhip_rope(fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *x, fhip_dtype x_dtype, const fhip_tensor4 *out,
+              fhip_dtype out_dtype) {
+    if (!rope) {
+        set_error("rope: NULL tables");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    return rope_core(s, nullptr, rope, x, x_dtype, out, out_dtype);
+}
+
+int fhip_norm_rope(fhip_stream *s, const fhip_rms_norm *norm, const fhip_rope_tables *rope, const fhip_tensor4 *x,
+                   fhip_dtype x_dtype, const fhip_tensor4 *out, fhip_dtype out_dtype) {
+    int rc = check_norm(norm);
+    if (rc) return rc;
+    return rope_core(s, norm, rope, x, x_dtype, out, out_dtype);
+}
+
+static int rope_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *k_norm, const fhip_rope_tables *rope,
+                            const fhip_tensor4 *k_new, const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all,
+                            fhip_tensor4 *v_all) {
     if (!k_new || !fhip::dtype_ok(in_dtype)) {
         set_error("kv_cache_rope_append: NULL argument or bad dtype");
         return FHIP_ERR_INVALID_ARG;
@@ -1019,7 +1060,21 @@ int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_
     NewRows nr;
     nr.src_dtype = in_dtype;
     nr.rope = rope;
+    nr.k_norm = k_norm;
     return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
+}
+
+int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *k_new,
+                              const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    return rope_append_core(c, s, nullptr, rope, k_new, v_new, in_dtype, k_all, v_all);
+}
+
+int fhip_kv_cache_norm_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *k_norm,
+                                   const fhip_rope_tables *rope, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
+                                   fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    int rc = check_norm(k_norm);
+    if (rc) return rc;
+    return rope_append_core(c, s, k_norm, rope, k_new, v_new, in_dtype, k_all, v_all);
 }
 
 }  // extern "C"

@@ -74,8 +74,15 @@ int launch_fill_zero_rows(void *dst, const int64_t dstride[4], const uint32_t sh
 // Rotary embedding / type conversion of rows [B, heads, rows, D] from a strided source into a strided
 // destination.  mode 0: pairs (i, i + D/2), 1: pairs (2i, 2i+1), 2: conversion only.  pos0 is the row
 // of the cos/sin tables ([positions, D/2] f32) that row 0 uses.
+// norm (nullable): RMS-normalise each row first with weight / bias [D] of norm->dtype, result rounded to
+// src_dtype before the rotation.  Needs an even D.
+struct RowNorm {
+    const void *weight, *bias;
+    fhip_dtype dtype;
+    float eps;
+};
 int launch_rope_rows(const void *src, const int64_t sstride[4], fhip_dtype src_dtype, void *dst,
                      const int64_t dstride[4], fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos,
-                     const float *sin, int64_t pos0, int mode, hipStream_t stream);
+                     const float *sin, int64_t pos0, int mode, const RowNorm *norm, hipStream_t stream);
 
 }  // namespace fhip

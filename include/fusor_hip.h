@@ -262,6 +262,31 @@ int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_
                               const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all,
                               fhip_tensor4 *v_all);
 
+/* ---- q / k RMS-norm fused into the rotation ------------------------------------------------------
+ * Blocks with attention_q_norm / attention_k_norm (models/kalosm-llama/src/raw/attention_layer.rs:
+ * 229-235,251-257) normalise every [head_dim] row of q and k before the rotation:
+ * RmsNorm::forward_generic_4d (fusor-ml/fusor/src/layers/rms_norm.rs:122-133), i.e. in f32
+ *   n = x / sqrt(mean(x * x) + eps) * weight (+ bias)
+ * with the reference's operation order and its left-to-right sum (rms_norm_fused_cpu_impl,
+ * fusor-ml/fusor/src/composite/normalization.rs:351-407), rounded to x's element type (the norm
+ * returns a tensor of that type), then rotated as fhip_rope does. */
+typedef struct {
+    const void *weight; /* device, [head_dim] contiguous (RmsNorm::weight)                            */
+    const void *bias;   /* device, [head_dim] contiguous, or NULL (RmsNorm::bias)                     */
+    fhip_dtype dtype;   /* element type of weight and bias                                            */
+    float eps;
+} fhip_rms_norm;
+
+/* out = rope(rms_norm(x)); arguments as fhip_rope.  rope == NULL: the norm alone. */
+int fhip_norm_rope(fhip_stream *s, const fhip_rms_norm *norm, const fhip_rope_tables *rope, const fhip_tensor4 *x,
+                   fhip_dtype x_dtype, const fhip_tensor4 *out, fhip_dtype out_dtype);
+
+/* fhip_kv_cache_rope_append with the new keys normalised before they are rotated (the values are only
+ * converted, as before). */
+int fhip_kv_cache_norm_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *k_norm,
+                                   const fhip_rope_tables *rope, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
+                                   fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all);
+
 /* Library version string, e.g. "fusor-hip 0.1 (gfx950)". */
 const char *fhip_version(void);
 

@@ -343,10 +343,15 @@ class KvCache {
     }
     /// append(rope(k), v): the rotation of RopeCache::forward / forward_interleaved and the conversion to
     /// the cache's element type happen in the pass that writes the new rows
-    std::pair<Tensor<4>, Tensor<4>> append_rope(const fhip_rope_tables &tables, const Tensor<4> &k, const Tensor<4> &v) {
+    /// k_norm (RmsNorm::c()): the keys are RMS-normalised before the rotation (attention_k_norm)
+    std::pair<Tensor<4>, Tensor<4>> append_rope(const fhip_rope_tables &tables, const Tensor<4> &k, const Tensor<4> &v,
+                                                const fhip_rms_norm *k_norm = nullptr) {
         if (k.dtype() != v.dtype()) throw Panic("append_rope: keys and values differ in element type");
         fhip_tensor4 kn = k.c4(), vn = v.c4(), ka{}, va{};
-        check(fhip_kv_cache_rope_append(in_->c, dev_.stream(), &tables, &kn, &vn, (fhip_dtype)k.dtype(), &ka, &va));
+        if (k_norm)
+            check(fhip_kv_cache_norm_rope_append(in_->c, dev_.stream(), k_norm, &tables, &kn, &vn, (fhip_dtype)k.dtype(), &ka, &va));
+        else
+            check(fhip_kv_cache_rope_append(in_->c, dev_.stream(), &tables, &kn, &vn, (fhip_dtype)k.dtype(), &ka, &va));
         auto wrap = [&](const fhip_tensor4 &t) {
             Tensor<4> r(std::make_shared<Buffer>(dev_, t.ptr), dtype_, t.shape, t.stride, t.offset, in_);
             return r;
@@ -390,13 +395,18 @@ class RopeCache {
         t.interleaved = interleaved ? 1 : 0;
         return t;
     }
-    Tensor<4> apply(const Tensor<4> &x, uint64_t start_pos, bool interleaved, std::optional<DType> out_dtype = std::nullopt) const {
+    /// norm (RmsNorm::c()): the rows are RMS-normalised first, in the same pass (attention_q_norm)
+    Tensor<4> apply(const Tensor<4> &x, uint64_t start_pos, bool interleaved, std::optional<DType> out_dtype = std::nullopt,
+                    const fhip_rms_norm *norm = nullptr) const {
         const DType od = out_dtype.value_or(x.dtype());
         const auto &shp = x.shape();
         Tensor<4> out = Tensor<4>::empty(dev_, od, {shp[0], shp[1], shp[2], shp[3]});
         const fhip_rope_tables t = tables(start_pos, interleaved);
         const fhip_tensor4 cx = x.c4(), co = out.c4();
-        check(fhip_rope(dev_.stream(), &t, &cx, (fhip_dtype)x.dtype(), &co, (fhip_dtype)od));
+        if (norm)
+            check(fhip_norm_rope(dev_.stream(), norm, &t, &cx, (fhip_dtype)x.dtype(), &co, (fhip_dtype)od));
+        else
+            check(fhip_rope(dev_.stream(), &t, &cx, (fhip_dtype)x.dtype(), &co, (fhip_dtype)od));
         return out;
     }
     /// RopeCache::forward(q, k, start_pos) -> (q, k)   (pairs (i, i + head_dim/2))
@@ -406,6 +416,41 @@ class RopeCache {
     /// RopeCache::forward_interleaved(q, k, start_pos) -> (q, k)   (pairs (2i, 2i + 1))
     std::pair<Tensor<4>, Tensor<4>> forward_interleaved(const Tensor<4> &q, const Tensor<4> &k, uint64_t start_pos) const {
         return {apply(q, start_pos, true), apply(k, start_pos, true)};
+    }
+};
+
+/// fusor::layers::RmsNorm<1, T> over the last dimension (fusor-ml/fusor/src/layers/rms_norm.rs:11-133), as the
+/// q / k norm of attention blocks uses it; pass c() to RopeCache::apply / KvCache::append_rope to fuse it.
+class RmsNorm {
+    Tensor<2> weight_;
+    std::optional<Tensor<2>> bias_;
+    Device dev_;
+    DType dtype_;
+    float eps_;
+
+   public:
+    /// RmsNorm::new(weight, bias, eps): host values [head_dim] in f32, stored as `dtype`
+    RmsNorm(const Device &dev, DType dtype, uint32_t head_dim, const float *weight, const float *bias, float eps)
+        : weight_(Tensor<2>::from_slice(dev, dtype, {1, head_dim}, weight)), dev_(dev), dtype_(dtype), eps_(eps) {
+        if (bias) bias_ = Tensor<2>::from_slice(dev, dtype, {1, head_dim}, bias);
+    }
+    float eps() const { return eps_; }
+    fhip_rms_norm c() const {
+        fhip_rms_norm n{};
+        n.weight = weight_.c2().ptr;
+        n.bias = bias_ ? bias_->c2().ptr : nullptr;
+        n.dtype = (fhip_dtype)dtype_;
+        n.eps = eps_;
+        return n;
+    }
+    /// RmsNorm::forward_generic_4d (rms_norm.rs:122-133): the norm alone
+    Tensor<4> forward_generic_4d(const Tensor<4> &x) const {
+        const auto &shp = x.shape();
+        Tensor<4> out = Tensor<4>::empty(dev_, x.dtype(), {shp[0], shp[1], shp[2], shp[3]});
+        const fhip_rms_norm n = c();
+        const fhip_tensor4 cx = x.c4(), co = out.c4();
+        check(fhip_norm_rope(dev_.stream(), &n, nullptr, &cx, (fhip_dtype)x.dtype(), &co, (fhip_dtype)x.dtype()));
+        return out;
     }
 };
 

@@ -2,11 +2,11 @@
 
 Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this package.
 It restates fusor-ml's CPU attention composite (C, ``fusor_cpu_attention.c``), its mask builders,
-its growable KV cache and its rotary embedding (numpy, this file), and carries float64 textbook twins
-used to pin the restatements.
+its growable KV cache, its rotary embedding and its RMS norm (numpy, this file), and carries float64
+textbook twins used to pin the restatements.
 
-Parity status: everything here is pinned by the checks in tests/test_oracle.py and
-tests/test_rope_oracle.py except two bit-level details, which are PARITY UNPINNED: the summation order
+Parity status: everything here is pinned by the checks in tests/test_oracle.py,
+tests/test_rope_oracle.py and tests/test_rms_norm_oracle.py except two bit-level details, which are PARITY UNPINNED: the summation order
 of the `gemm` 0.18.2 micro-kernels inside the two matrix products (value-level parity is pinned, three
 orders of magnitude inside the 1e-5 tolerance), and the last bit of cos/sin in ``rope_tables`` (libm
 dependent; the rotation takes the tables as inputs, so no op result depends on it).
@@ -310,3 +310,29 @@ def rope_f64(x, cos, sin, start_pos=0, interleaved=False):
     else:
         out[..., :d // 2], out[..., d // 2:] = w.real, w.imag
     return out
+
+
+def rms_norm(x, weight, bias=None, eps=1e-5):
+    """RmsNorm::forward_generic_4d -> rms_norm_fused_cpu_impl (fusor-ml/fusor/src/layers/rms_norm.rs:122-133,
+    fusor-ml/fusor/src/composite/normalization.rs:351-407) over the last axis, f32, one rounding per op:
+    x*x; sum folded left to right from 0 (cpu/src/reduce.rs:752-757); / n; + eps; sqrt; x / rms; * weight; (+ bias).
+    The caller rounds the result to the tensor's element type (the cast at rms_norm.rs:132)."""
+    x = np.asarray(x, np.float32)
+    w = np.asarray(weight, np.float32)
+    n = x.shape[-1]
+    ss = np.zeros(x.shape[:-1], np.float32)
+    for i in range(n):
+        ss = (ss + (x[..., i] * x[..., i]).astype(np.float32)).astype(np.float32)
+    mean = (ss / np.float32(n)).astype(np.float32)
+    rms = np.sqrt((mean + np.float32(eps)).astype(np.float32)).astype(np.float32)
+    out = ((x / rms[..., None]).astype(np.float32) * w).astype(np.float32)
+    if bias is not None:
+        out = (out + np.asarray(bias, np.float32)).astype(np.float32)
+    return out
+
+
+def rms_norm_f64(x, weight, bias=None, eps=1e-5):
+    """The textbook definition in float64: x / sqrt(mean(x^2) + eps) * weight + bias."""
+    x = np.asarray(x, np.float64)
+    out = x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + np.float64(np.float32(eps))) * np.asarray(weight, np.float64)
+    return out if bias is None else out + np.asarray(bias, np.float64)

@@ -166,6 +166,30 @@ static void test_rope(const Device &d) {  // rope.rs:270-400 (inputs), rope.rs:4
     EXPECT(bad == 0, "%d cached values differ after append_rope", bad);
 }
 
+static void test_rms_norm(const Device &d) {  // rms_norm.rs:163-186 (values), normalization.rs:351-407 (order)
+    const float w2[2] = {2.0f, 2.0f};
+    RmsNorm norm(d, DType::F32, 2, w2, nullptr, 1e-5f);
+    auto t = t4(d, {3.0f, 4.0f, 6.0f, 8.0f}, 1, 1, 2, 2);
+    auto y = host(norm.forward_generic_4d(t));
+    const float rms1 = std::sqrt(12.5f);
+    EXPECT(std::fabs(y[0] - 3.0f / rms1 * 2.0f) < 1e-4f && std::fabs(y[1] - 4.0f / rms1 * 2.0f) < 1e-4f, "rms norm row [3, 4]: %g %g", y[0], y[1]);
+    // every step exact: squares sum to 16, mean 4, root 2; the bias is added last
+    const float w4[4] = {1.0f, 3.0f, 0.5f, -7.0f}, b4[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    RmsNorm exact(d, DType::F32, 4, w4, b4, 0.0f);
+    auto e = host(exact.forward_generic_4d(t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4)));
+    EXPECT(e[0] == 2.0f && e[1] == -2.0f && e[2] == 1.5f && e[3] == 8.0f, "exact rms norm row: %g %g %g %g", e[0], e[1], e[2], e[3]);
+    // fused into the rotation: at position 0 the rotation is the identity, so norm + rope == norm
+    const float c0[2] = {1.0f, 1.0f}, s0[2] = {0.0f, 0.0f};
+    RopeCache rope(d, 1, 2, c0, s0);
+    const fhip_rms_norm n = exact.c();
+    auto f = host(rope.apply(t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4), 0, false, std::nullopt, &n));
+    EXPECT(f[0] == 2.0f && f[1] == -2.0f && f[2] == 1.5f && f[3] == 8.0f, "norm fused into rope: %g %g %g %g", f[0], f[1], f[2], f[3]);
+    KvCache cache(d, 2, 8);
+    auto kv = cache.append_rope(rope.tables(0, false), t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4), t4(d, {5.0f, 6.0f, 7.0f, 8.0f}, 1, 1, 1, 4), &n);
+    auto kc = host(kv.first), vc = host(kv.second);
+    EXPECT(kc[0] == 2.0f && kc[3] == 8.0f && vc[0] == 5.0f && vc[3] == 8.0f, "norm fused into the cache append");
+}
+
 int main() {
     try {
         Device d(0);
@@ -177,6 +201,7 @@ int main() {
         test_mask_cache(d);
         test_kv_cache(d);
         test_rope(d);
+        test_rms_norm(d);
     } catch (const std::exception &e) {
         printf("exception: %s\n", e.what());
         return 2;

@@ -99,3 +99,86 @@ def test_kv_cache_rope_append_equals_rope_then_append(device, cache_dtype, in_dt
         assert np.array_equal(va.to_numpy().view(np.uint8), np.ascontiguousarray(rv).view(np.uint8)), f"values, step {step}"
         pos += n
     assert fused.current_seq_len() == max_len
+
+
+# ---- q / k RMS-norm fused into the rotation (attention_q_norm / attention_k_norm) ---------------------
+
+def _norm_then_rope(x, dtype, w, b, eps, rc, start, interleaved, out_dtype):
+    """What the reference computes (attention_layer.rs:229-235,272-278): the norm in f32 rounded to the
+    tensor's type, then cast -> rope -> cast."""
+    n = rounded(oracle.rms_norm(rounded(x, dtype), rounded(w, dtype), None if b is None else rounded(b, dtype), eps), dtype)
+    fn = oracle.rope_interleaved if interleaved else oracle.rope
+    return _cast_out(fn(n, rc.cos_host, rc.sin_host, start), out_dtype)
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16, fa.BF16])
+@pytest.mark.parametrize("interleaved,bias", [(False, False), (True, True)])
+@pytest.mark.parametrize("D,start", [(64, 0), (128, 37), (96, 5), (256, 2), (2, 1)])
+def test_norm_rope_bit_exact(device, dtype, interleaved, bias, D, start):
+    rc = fa.RopeCache(D, 64, 1000000.0, device)
+    rng = np.random.default_rng(D)
+    x = _x(D + start, (2, 5, 11, D)) * 3
+    w = rng.normal(1, 0.3, D).astype(np.float32)
+    b = rng.normal(0, 0.1, D).astype(np.float32) if bias else None
+    norm = fa.RmsNorm(w, b, 1e-6, dtype, device)
+    t = fa.Tensor.from_numpy(device, x, dtype)
+    out = rc.apply(t, start, interleaved, norm=norm).to_numpy()
+    ref = _norm_then_rope(x, dtype, w, b, 1e-6, rc, start, interleaved, dtype)
+    assert np.array_equal(out.view(np.uint8), ref.view(np.uint8))
+    # the norm alone (RmsNorm::forward_generic_4d)
+    alone = norm.forward_generic_4d(t).to_numpy()
+    ref_n = _cast_out(oracle.rms_norm(rounded(x, dtype), rounded(w, dtype), None if b is None else rounded(b, dtype), 1e-6), dtype)
+    assert np.array_equal(alone.view(np.uint8), ref_n.view(np.uint8))
+
+
+def test_norm_sum_order_and_reference_test_rows(device):
+    """The device sum is the reference's left-to-right fold (a row where any other order differs), and the
+    rows of the reference's own tests (rms_norm.rs:163-186) come out as expected."""
+    x = np.ones((1, 1, 2, 42), np.float32)
+    x[0, 0, 0, 0] = 4096.0
+    x[0, 0, 1, 40] = 4096.0
+    norm = fa.RmsNorm(np.ones(42, np.float32), None, 0.0, fa.F32, device)
+    out = norm.forward_generic_4d(fa.Tensor.from_numpy(device, x, fa.F32)).to_numpy()
+    assert np.array_equal(out, oracle.rms_norm(x, np.ones(42, np.float32), None, 0.0))
+    x2 = np.array([3, 4, 6, 8], np.float32).reshape(1, 1, 2, 2)
+    out2 = fa.RmsNorm(np.array([2, 2], np.float32), None, 1e-5, fa.F32, device).forward_generic_4d(
+        fa.Tensor.from_numpy(device, x2, fa.F32)).to_numpy()
+    rms1 = np.sqrt(np.float32(12.5))
+    assert abs(out2[0, 0, 0, 0] - 3.0 / rms1 * 2.0) < 1e-4 and abs(out2[0, 0, 0, 1] - 4.0 / rms1 * 2.0) < 1e-4
+
+
+def test_norm_rope_in_place_on_a_strided_view(device):
+    """out may be x itself, and x may be the transposed projection: rows are read whole before they are written."""
+    B, S, H, D = 2, 33, 6, 128
+    rc = fa.RopeCache(D, 64, 10000.0, device)
+    proj = _x(9, (B, S, H, D))
+    w = np.random.default_rng(4).normal(1, 0.2, D).astype(np.float32)
+    norm = fa.RmsNorm(w, None, 1e-6, fa.F32, device)
+    t = fa.Tensor.from_numpy(device, proj, fa.F32).transpose(1, 2)
+    import ctypes
+    cx, cn, tables = t._c4(), norm._c(), rc._tables(7, False)
+    fa.check(fa.lib().fhip_norm_rope(device.stream, ctypes.byref(cn), ctypes.byref(tables), ctypes.byref(cx), fa.F32,
+                                     ctypes.byref(cx), fa.F32))
+    ref = oracle.rope(oracle.rms_norm(proj.transpose(0, 2, 1, 3), w, None, 1e-6), rc.cos_host, rc.sin_host, 7)
+    assert np.array_equal(t.to_numpy(), ref)
+
+
+@pytest.mark.parametrize("cache_dtype,in_dtype", [(fa.F32, fa.F32), (fa.F16, fa.F32), (fa.F16, fa.F16)])
+def test_kv_cache_norm_rope_append(device, cache_dtype, in_dtype):
+    B, Hkv, D, max_len = 2, 2, 128, 24
+    rc = fa.RopeCache(D, 64, 10000.0, device)
+    w = np.random.default_rng(6).normal(1, 0.2, D).astype(np.float32)
+    norm = fa.RmsNorm(w, None, 1e-6, in_dtype, device)
+    fused = fa.KvCache(2, max_len, cache_dtype, device)
+    ref_cache = oracle.KvCache(2, max_len)
+    pos = 0
+    for step, n in enumerate([5, 1, 9, 1, 17, 2]):
+        k = _x(300 + step, (B, Hkv, n, D))
+        v = _x(400 + step, (B, Hkv, n, D))
+        tk, tv = fa.Tensor.from_numpy(device, k, in_dtype), fa.Tensor.from_numpy(device, v, in_dtype)
+        ka, va = fused.append_rope(rc, tk, tv, pos, False, k_norm=norm)
+        k_rot = _norm_then_rope(k, in_dtype, w, None, 1e-6, rc, pos, False, cache_dtype)
+        rk, rv = ref_cache.append(k_rot, _cast_out(rounded(v, in_dtype), cache_dtype))
+        assert np.array_equal(ka.to_numpy().view(np.uint8), np.ascontiguousarray(rk).view(np.uint8)), f"keys, step {step}"
+        assert np.array_equal(va.to_numpy().view(np.uint8), np.ascontiguousarray(rv).view(np.uint8)), f"values, step {step}"
+        pos += n
