@@ -33,7 +33,7 @@ MEASURED_TRAFFIC_BYTES = {"C2": 270.2e6, "C3": 214.6e6}
 
 
 def configs():
-    # name -> description of the synthetic workload (BASELINE.json `configs`, in order)
+    # name -> description of the synthetic workload (the benchmark configurations, in order)
     return {
         "C1": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True),
         "C2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),

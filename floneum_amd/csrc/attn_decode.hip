@@ -30,16 +30,9 @@ constexpr int DEC_WAVES = 4;
 constexpr int DEC_UNROLL = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 
-static int env_int(const char *name, int dflt) {
-    const char *s = getenv(name);
-    if (!s || !*s) return dflt;
-    int v = atoi(s);
-    return v > 0 ? v : dflt;
-}
-
 // the matrix-core variant takes 16-bit tensors; f32 tensors run on the vector variant
 static bool decode_use_mfma(int D, bool f32) {
-    return !f32 && (D == 32 || D == 64 || D == 96 || D == 128) && env_int("FHIP_DECODE_VARIANT", 1) == 1;
+    return !f32 && (D == 32 || D == 64 || D == 96 || D == 128);
 }
 
 // query heads handled by one workgroup
@@ -56,12 +49,12 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more; f32 rows carry
     // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at
     // batch 1 with 32768 keys)
-    const int wgs_per_cu = env_int("FHIP_DECODE_WGS_PER_CU", (decode_use_mfma(D, f32) || f32) ? 2 : 4);
+    const int wgs_per_cu = (decode_use_mfma(D, f32) || f32) ? 2 : 4;
     const long target = (long)compute_units * wgs_per_cu;
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
-    const int max_chunk = env_int("FHIP_DECODE_MAX_CHUNK", ragged && units >= target ? 512 : 1024);
-    const int min_chunk = env_int("FHIP_DECODE_MIN_CHUNK", 256);
+    const int max_chunk = ragged && units >= target ? 512 : 1024;
+    const int min_chunk = 256;
     long ns = (target + units - 1) / units;
     const long ns_max = (Skv + min_chunk - 1) / min_chunk;
     const long ns_min = (Skv + max_chunk - 1) / max_chunk;
