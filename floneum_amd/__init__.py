@@ -363,6 +363,15 @@ class Tensor:
         shp[dim] = length
         return Tensor(self.buffer, self.dtype, shp, self.strides, self.offset + start * self.strides[dim])
 
+    def broadcast_to(self, shape):
+        """Layout::broadcast_to (fusor-ml/types/src/layout.rs): dimensions of size 1 repeat with stride 0."""
+        assert len(shape) == len(self.shape)
+        st = []
+        for have, want, stride in zip(self.shape, shape, self.strides):
+            assert have == want or have == 1, f"cannot broadcast {self.shape} to {tuple(shape)}"
+            st.append(stride if have == want else 0)
+        return Tensor(self.buffer, self.dtype, shape, st, self.offset)
+
     def is_contiguous(self):
         return self.strides == _contig_strides(self.shape)
 

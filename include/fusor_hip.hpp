@@ -177,6 +177,17 @@ class Tensor {
         t.offset_ += (uint64_t)start * (uint64_t)stride_[dim];
         return t;
     }
+    /// Layout::broadcast_to: dimensions of size 1 repeat with stride 0, no copy
+    Tensor broadcast_to(const uint32_t (&shape)[R]) const {
+        Tensor t = *this;
+        for (int i = 0; i < R; i++) {
+            if (shape_[i] == shape[i]) continue;
+            if (shape_[i] != 1) throw Panic("broadcast_to: only dimensions of size 1 repeat");
+            t.shape_[i] = shape[i];
+            t.stride_[i] = 0;
+        }
+        return t;
+    }
     /// as_slice().await: contiguous readback of this view (synchronises the stream)
     void to_host(void *host) const {
         if (!is_contiguous()) throw Panic("to_host needs a contiguous view");

@@ -355,3 +355,23 @@ def test_output_written_as_batch_seq_heads_dim(device, dtype, Sq):
         else:
             tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
             assert_parity(got.astype(np.float32), plain.astype(np.float32), tol, "general kernel, transposed output")
+
+
+@pytest.mark.parametrize("dtype,Sq", [(fa.F16, 300), (fa.F32, 200), (fa.F16, 1)])
+def test_broadcast_views_of_one_kv_head(device, dtype, Sq):
+    """The reference expands K/V over the query heads with reshape + broadcast_to (stride 0) before its matmuls
+    (fusor flash_attention.rs:104-138).  The op takes such a view directly: one stored KV head repeated for every
+    query head gives the same result as the grouped call."""
+    B, H, D, Skv = 2, 8, 64, 333
+    q, k, v = _normal_qkv(31, B, H, 1, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    kb, vb = tk.broadcast_to((B, H, Skv, D)), tv.broadcast_to((B, H, Skv, D))
+    assert kb.strides[1] == 0 and kb.shape == (B, H, Skv, D)
+    out_b = tq.flash_attention(kb, vb, D ** -0.5).to_numpy()
+    out_g = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, None, None)
+    tol = TOL_F32 if dtype == fa.F32 else TOL_16
+    assert_parity(out_b, ref, tol, "broadcast kv heads")
+    assert_parity(out_g, ref, tol, "one kv head, grouped")
+    if Sq > 1:  # the tiled kernels walk the keys in the same order either way (the decode split differs)
+        assert np.array_equal(out_b.view(np.uint8), out_g.view(np.uint8))
