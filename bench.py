@@ -304,6 +304,19 @@ def run_config(name, steps, warmup, with_cpu=True):
                            ragged_lens=c.get("ragged"), kv_sets_rotated=n_sets,
                            algorithmic_flops=flops, algorithmic_bytes=byts),
                dtype=c["dtype"], frac_of_roofline=value / roof["peak"], spot_check_max_abs_err=err)
+    if lens is not None:
+        # what the ragged lengths cost: the same call with every sequence at the mean length (same buffers,
+        # the same bytes to within rounding), so any difference in GB/s is load imbalance between workgroups
+        eq = np.full(c["B"], int(round(float(lens.mean()))), np.int32)
+        eq_t = fa.IntTensor(dev, eq)
+        _, eq_byts = algorithmic(c, eq)
+        eq_blocks, _ = prepare(fa, dev, c, sets, eq_t)
+        eq_wall_ms, _, _, _ = time_config(fa, dev, c, eq_blocks, max(5, steps // 2), min(warmup, 5))
+        eq_value = eq_byts / (eq_wall_ms * 1e-3) / 1e9
+        res["imbalance"] = dict(lens_min=int(lens.min()), lens_mean=float(lens.mean()), lens_max=int(lens.max()),
+                                equal_lengths_value=eq_value, unit=unit, ragged_over_equal=value / eq_value,
+                                note="same call with every sequence at the mean length; 1.0 = the ragged batch "
+                                     "streams as fast as an even one")
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(oracle, c, host, lens, flops, byts)
     return res
@@ -352,6 +365,8 @@ def main():
             "spot_check_max_abs_err": main_res["spot_check_max_abs_err"]}
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
+    if "imbalance" in main_res:
+        line["imbalance"] = main_res["imbalance"]
     if not a.no_extra and a.config == "C2":
         # the other half of the metric: C3 prefill on the matrix cores
         # the shader clock needs some tens of milliseconds of matrix load to settle: warm the prefill

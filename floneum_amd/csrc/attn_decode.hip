@@ -175,7 +175,10 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
     const int D = p.D;
     const bool active = c * 8 < D;
 
-    const int split = blockIdx.x;
+    // Workgroups go to the 8 XCDs round-robin in launch order (x fastest), and with ragged lengths only the
+    // first splits of a row of the grid have keys: taken as they come, XCD 0 would get up to one more busy
+    // workgroup per (batch, head) than XCD 7.  Rotating the split by the row spreads them evenly.
+    const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);
     const int HB = (p.G + GT - 1) / GT;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
@@ -413,7 +416,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
     const int q4 = lane >> 4; // key group
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
-    const int split = blockIdx.x;
+    const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
     const int HB = (p.G + DM_HEADS - 1) / DM_HEADS;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
