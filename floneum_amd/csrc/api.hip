@@ -59,11 +59,6 @@ static int validate(const fhip_attn_args *a) {
     }
     const uint32_t *qs = a->q.shape, *ks = a->k.shape, *vs = a->v.shape, *os = a->out.shape;
     for (int i = 0; i < 4; i++) {
-        if (qs[i] == 0 || ks[i] == 0 || vs[i] == 0) {
-            set_error("empty tensors are not supported (q %u,%u,%u,%u k %u,%u,%u,%u)", qs[0], qs[1], qs[2],
-                      qs[3], ks[0], ks[1], ks[2], ks[3]);
-            return FHIP_ERR_INVALID_ARG;
-        }
         if (qs[i] > 0x7fffffffu || ks[i] > 0x7fffffffu) {
             set_error("dimension larger than 2^31-1");
             return FHIP_ERR_INVALID_ARG;
@@ -72,7 +67,8 @@ static int validate(const fhip_attn_args *a) {
     const uint32_t B = qs[0], H = qs[1], Sq = qs[2], D = qs[3];
     const uint32_t Hkv = ks[1], Skv = ks[2];
     // reference: assert!(num_heads.is_multiple_of(num_kv_heads), ...) flash_attention.rs:94-99
-    if (H % Hkv != 0) {
+    // (u32::is_multiple_of(0) holds for 0 only)
+    if (Hkv == 0 ? H != 0 : H % Hkv != 0) {
         set_error("Number of Q heads (%u) must be divisible by number of K/V heads (%u)", H, Hkv);
         return FHIP_ERR_INVALID_ARG;
     }
@@ -93,11 +89,13 @@ static int validate(const fhip_attn_args *a) {
                       os[2], os[3], B, H, Sq, D);
             return FHIP_ERR_INVALID_ARG;
         }
-    if (!a->q.ptr || !a->k.ptr || !a->v.ptr || !a->out.ptr) {
+    // a tensor without elements needs no memory
+    const bool q_empty = B == 0 || H == 0 || Sq == 0 || D == 0, kv_empty = B == 0 || Hkv == 0 || Skv == 0 || D == 0;
+    if ((!q_empty && (!a->q.ptr || !a->out.ptr)) || (!kv_empty && (!a->k.ptr || !a->v.ptr))) {
         set_error("q, k, v and out need device pointers");
         return FHIP_ERR_INVALID_ARG;
     }
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < 4 && !q_empty; i++)
         if (os[i] > 1 && a->out.stride[i] == 0) {
             set_error("output stride %d is 0 (overlapping writes)", i);
             return FHIP_ERR_INVALID_ARG;
@@ -153,6 +151,15 @@ static int validate(const fhip_attn_args *a) {
     }
     return FHIP_OK;
 }
+
+// Calls whose result is fixed by the shapes alone.  No output element: nothing to do.  No key (Skv == 0)
+// but output elements: the reference's composite multiplies a [Sq, 0] matrix of probabilities with a
+// [0, D] matrix of values, which is all zeros (fusor flash_attention.rs:141-199: the softmax of an empty
+// row is empty, no 0/0 is ever formed).
+static bool output_is_empty(const fhip_attn_args *a) {
+    return a->q.shape[0] == 0 || a->q.shape[1] == 0 || a->q.shape[2] == 0 || a->q.shape[3] == 0;
+}
+static bool no_keys(const fhip_attn_args *a) { return a->k.shape[2] == 0; }
 
 static bool aligned16(const void *p, uint64_t off_elems, int eb) {
     return (((uintptr_t)p + off_elems * (uint64_t)eb) & 15u) == 0;
@@ -218,6 +225,10 @@ static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
 // (the size query); otherwise a masked call without enough scratch takes the general kernel.
 static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_workspace = false) {
     const int f = a->force_kernel;
+    if (output_is_empty(a) || no_keys(a)) {  // answered without an attention kernel
+        *id = FHIP_KERNEL_GENERIC;
+        return FHIP_OK;
+    }
     const bool mask_ok = mask_scratch_ok(a, assume_workspace);
     if (f != FHIP_KERNEL_AUTO) {
         bool ok = false;
@@ -549,6 +560,7 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     int32_t id;
     rc = select_kernel(args, &id, true);
     if (rc) return rc;
+    if (output_is_empty(args) || no_keys(args)) return FHIP_OK;
     if (id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) *bytes = mask_scratch_bytes(args);
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
         int chunk, nsplit;
@@ -570,9 +582,18 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     int32_t id;
     rc = select_kernel(args, &id);
     if (rc) return rc;
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    if (output_is_empty(args) || no_keys(args)) {
+        if (!output_is_empty(args)) {
+            char *out = (char *)args->out.ptr + args->out.offset * (uint64_t)elem_bytes(args->out_dtype);
+            rc = launch_fill_zero_rows(out, args->out.stride, args->out.shape, elem_bytes(args->out_dtype), s->s);
+            if (rc) return rc;
+        }
+        if (args->main_kernel_done) FHIP_HIP_CHECK(hipEventRecord(args->main_kernel_done->e, s->s));
+        return FHIP_OK;
+    }
     AttnParams p;
     fill_params(args, &p);
-    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
     if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
         // dense mask: reduce it to one visible interval per row on the device; the tiled kernel runs

@@ -194,7 +194,10 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
 /* out = softmax(q k^T * scale + mask) v with GQA head mapping kv_head = head / (H / Hkv).
  * Replaces fusor_core::Tensor::flash_attention (core/src/composite/flash_attention.rs:28-52) and,
  * for FHIP_MASK_BATCH_KEY, the composite fallback fusor takes on GPU (fusor
- * flash_attention.rs:61-72).  Asynchronous on `s`. */
+ * flash_attention.rs:61-72).  Asynchronous on `s`.
+ * Rows whose keys are all masked come out NaN (0/0, as in the reference).  Tensors without elements
+ * are valid: with no output element nothing runs; with no key (Skv == 0) the output is all zeros, which
+ * is what the reference's [Sq, 0] x [0, D] product gives (fusor flash_attention.rs:141-199). */
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
 
 /* ---- masks: host builders, bit-exact with the reference ---------------------------------------

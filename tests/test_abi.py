@@ -117,12 +117,24 @@ def test_validate_other_errors():
     assert status(a)[0] == fa.ERR_INVALID_ARG
     a = make_args(D=1024)
     assert status(a)[0] == fa.ERR_UNSUPPORTED
-    a = make_args(Skv=8)
-    a.k.shape[2] = 0
-    a.v.shape[2] = 0
-    assert status(a)[0] == fa.ERR_INVALID_ARG
     assert fa.lib().fhip_flash_attention_validate(None) == fa.ERR_INVALID_ARG
     assert fa.lib().fhip_flash_attention(None, ctypes.byref(make_args())) == fa.ERR_INVALID_ARG
+
+
+def test_validate_accepts_tensors_without_elements():
+    # no keys, no queries, no batch: valid calls (the result is all zeros, or has no element); no memory needed
+    for kw in (dict(Skv=0), dict(Sq=0), dict(B=0), dict(H=0, Hkv=0)):
+        a = make_args(**kw)
+        assert status(a)[0] == fa.OK, kw
+        need = ctypes.c_size_t(99)
+        assert fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
+        assert need.value == 0
+    a = make_args(Sq=0)
+    a.q.ptr = a.out.ptr = None
+    assert status(a)[0] == fa.OK
+    # u32::is_multiple_of(0) holds for 0 only (fusor flash_attention.rs:94-99)
+    rc, msg = status(make_args(H=4, Hkv=0))
+    assert rc == fa.ERR_INVALID_ARG and "divisible" in msg
 
 
 def selected(a):

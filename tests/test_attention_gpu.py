@@ -375,3 +375,29 @@ def test_broadcast_views_of_one_kv_head(device, dtype, Sq):
     assert_parity(out_g, ref, tol, "one kv head, grouped")
     if Sq > 1:  # the tiled kernels walk the keys in the same order either way (the decode split differs)
         assert np.array_equal(out_b.view(np.uint8), out_g.view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_tensors_without_elements(device, dtype):
+    """No output element: nothing is computed.  No key: the reference's composite multiplies [Sq, 0] probabilities
+    with [0, D] values, which is all zeros, not NaN (fusor flash_attention.rs:141-199; a row whose keys are all
+    MASKED is the NaN case)."""
+    D = 64
+    for B, H, Hkv, Sq, Skv in ((0, 4, 2, 5, 7), (2, 0, 0, 5, 7), (2, 4, 2, 0, 7)):
+        tq = fa.Tensor.from_numpy(device, np.zeros((B, H, Sq, D), np.float32), dtype)
+        tk = fa.Tensor.from_numpy(device, np.zeros((B, Hkv, Skv, D), np.float32), dtype)
+        out = tq.flash_attention(tk, tk, 0.125).to_numpy()
+        assert out.shape == (B, H, Sq, D) and out.size == 0
+    q = _normal_qkv(41, 2, 4, 2, 5, 1, D)[0]
+    tq = fa.Tensor.from_numpy(device, q, dtype)
+    tk = fa.Tensor.from_numpy(device, np.zeros((2, 2, 0, D), np.float32), dtype)
+    out_t = fa.Tensor.from_numpy(device, np.full((2, 4, 5, D), 7.0, np.float32), dtype)  # must be overwritten
+    args = tq._attn_args(tk, tk, 0.125, None, None, None, None, fa.KERNEL_AUTO, out_t)
+    import ctypes
+    fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    out = out_t.to_numpy()
+    assert out.shape == (2, 4, 5, D) and not out.any()
+    # heads that cannot be grouped still panic, as u32::is_multiple_of does for a zero divisor
+    with pytest.raises(AssertionError, match="divisible"):
+        tq.flash_attention(fa.Tensor.from_numpy(device, np.zeros((2, 0, 3, D), np.float32), dtype),
+                           fa.Tensor.from_numpy(device, np.zeros((2, 0, 3, D), np.float32), dtype), 0.125)
