@@ -70,6 +70,36 @@ def test_padding_batch_key_mask(device, dtype, D):
                       f"un-padded sequence {b}")
 
 
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 64), (fa.F32, 128), (fa.F16, 128)])
+def test_block_diagonal_mask_of_the_vision_blocks(device, dtype, D):
+    """Qwen-VL's vision blocks mask with a block-diagonal [S, S] tensor built from cu_seqlens
+    (models/kalosm-llama/src/raw/vision/qwen_vision_block.rs:211-226): every row sees one contiguous run of
+    keys, so the interval form applies and the tiled kernel runs; the result equals running each block alone."""
+    cu_seqlens = [0, 70, 71, 300, 513]
+    S = cu_seqlens[-1]
+    mask = np.full((S, S), NEG_INF, np.float32)
+    for last, nxt in zip(cu_seqlens[:-1], cu_seqlens[1:]):
+        mask[last:nxt, last:nxt] = 0.0
+    q, k, v = _normal_qkv(27, 1, 4, 4, S, S, D)
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    want = fa.KERNEL_PREFILL_F32 if dtype == fa.F32 else fa.KERNEL_PREFILL_MFMA
+    ws, ws_bytes = device.workspace(1 << 20)
+    out_t = fa.Tensor.empty(device, (1, 4, S, D), dtype)
+    args = tq._attn_args(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask), None, None, None, fa.KERNEL_AUTO, out_t)
+    args.workspace, args.workspace_bytes = ws, ws_bytes
+    kid = ctypes.c_int32()
+    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), device.compute_units, ctypes.byref(kid)))
+    assert kid.value == want
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "qk")
+    assert_parity(out, ref, _tol(dtype), "block-diagonal mask")
+    for last, nxt in zip(cu_seqlens[:-1], cu_seqlens[1:]):
+        tqb, tkb, tvb = _tensors(device, dtype, q[:, :, last:nxt], k[:, :, last:nxt], v[:, :, last:nxt])
+        alone = tqb.flash_attention(tkb, tvb, D ** -0.5).to_numpy()
+        assert_parity(out[:, :, last:nxt], alone, dict(max_abs=2e-6 if dtype == fa.F32 else 2e-3, rel_l2=1e-5 if dtype == fa.F32 else 1e-3),
+                      f"block {last}:{nxt} alone")
+
+
 @pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.BF16, 64), (fa.F32, 64)])
 @pytest.mark.parametrize("shape", ["bias", "two_runs", "nan", "positive_inf"])
 def test_masks_that_are_not_intervals_fall_back(device, dtype, D, shape):
