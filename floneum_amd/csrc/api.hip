@@ -235,7 +235,7 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
         switch (f) {
             case FHIP_KERNEL_GENERIC: ok = true; break;
             case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a) && mask_ok; break;
-            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a) && mask_ok; break;
+            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a); break;  // its mask-adding form needs no scratch
             case FHIP_KERNEL_DECODE_SPLITKV: ok = decode_eligible(a); break;
             default: set_error("unknown force_kernel %d", f); return FHIP_ERR_INVALID_ARG;
         }
@@ -251,7 +251,7 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
         *id = FHIP_KERNEL_DECODE_SPLITKV;
     else if (prefill_mfma_eligible(a) && mask_ok)
         *id = FHIP_KERNEL_PREFILL_MFMA;
-    else if (prefill_f32_eligible(a) && mask_ok)
+    else if (prefill_f32_eligible(a))
         *id = FHIP_KERNEL_PREFILL_F32;
     else
         *id = FHIP_KERNEL_GENERIC;
@@ -595,9 +595,16 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     AttnParams p;
     fill_params(args, &p);
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    if (id == FHIP_KERNEL_PREFILL_F32 && args->mask_kind != FHIP_MASK_NONE && !mask_scratch_ok(args, false)) {
+        // no scratch for the interval form: the f32 kernel adds the mask tensor element by element
+        rc = launch_prefill_f32(p, s->s);
+        if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+        return rc;
+    }
     if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
-        // dense mask: reduce it to one visible interval per row on the device; the tiled kernel runs
-        // if every row is of that form, the general kernel (queued right behind it) if not
+        // dense mask: reduce it to one visible interval per row on the device; the tiled kernel skips the
+        // masked tiles if every row is of that form.  If not, the kernel queued right behind it takes the
+        // call: the f32 kernel's mask-adding form, or the general kernel for 16-bit tensors.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
         rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
@@ -610,7 +617,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
         AttnParams pg = p;
         pg.only_if_bad = bad;
-        return launch_generic(pg, args->dtype, s->s);
+        return id == FHIP_KERNEL_PREFILL_F32 ? launch_prefill_f32(pg, s->s) : launch_generic(pg, args->dtype, s->s);
     }
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;

@@ -40,7 +40,10 @@ __device__ __forceinline__ float half_swap_sum32(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <int D, int S>
+// BIAS: the additive mask tensor is applied as it is, element by element (p.mask, no interval form): finite
+// biases, several visible runs per row, NaN or +inf entries.  Score = (q.k * scale) + mask as in the reference
+// (fusor flash_attention.rs:145,177), every key tile is visited.
+template <int D, int S, bool BIAS>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnParams p, int nqb) {
     constexpr int WPG = PF32_WAVES / S;   // wavefronts per key-split group
     constexpr int BM = 32 * WPG;          // query rows per workgroup
@@ -53,7 +56,11 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     __shared__ __attribute__((aligned(16))) char smem[S * 2 * K_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
-    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
+    if constexpr (BIAS) {
+        if (p.only_if_bad && *p.only_if_bad == 0) return;  // the interval form of the mask has served the call
+    } else {
+        if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the BIAS form takes the call
+    }
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
@@ -97,7 +104,12 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 #pragma unroll
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
     float m = -INFINITY, l = 0.0f;
-    const float scale2 = p.scale * PF32_LOG2E;
+    // scores reach the softmax in the base-2 domain: raw dot products times scale * log2(e); with BIAS they are
+    // scaled, biased, and then only multiplied by log2(e)
+    const float scale2 = BIAS ? PF32_LOG2E : p.scale * PF32_LOG2E;
+    const float *mrow = nullptr;
+    if constexpr (BIAS)
+        mrow = (const float *)p.mask + (int64_t)(p.mask_kind == FHIP_MASK_QK ? min(query, p.Sq - 1) : b) * p.ms0;
 
     float4_t kst[NCH], vst[NCH];
     auto load_tile = [&](int j0) {
@@ -139,6 +151,15 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         const bool tile_visible = have && wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;
         if (!tile_visible) continue;
 
+        float bias[BIAS ? 16 : 1];
+        if constexpr (BIAS) {  // requested before the matrix work that hides their latency
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                bias[r] = key < p.Skv ? mrow[(int64_t)key * p.ms1] : 0.0f;
+            }
+        }
+
         // S^T: contraction step (kc, i) uses dim 8 kc + 4 h2 + i on both operands
         float16_t s;
 #pragma unroll
@@ -157,6 +178,11 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
                 const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
                 s[r] = (key >= rb.klo && key < rb.khi) ? s[r] : -INFINITY;
             }
+        }
+
+        if constexpr (BIAS) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[r] = s[r] * p.scale + bias[r];
         }
 
         float mx = s[0];
@@ -238,7 +264,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     }
 }
 
-template <int S>
+template <int S, bool BIAS>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
     constexpr int BM = 32 * (PF32_WAVES / S);
     const int nqb = (p.Sq + BM - 1) / BM;
@@ -249,13 +275,13 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
     switch (p.D) {
-        case 32: hipLaunchKernelGGL((prefill_f32_kernel<32, S>), grid, block, 0, stream, p, nqb); break;
-        case 64: hipLaunchKernelGGL((prefill_f32_kernel<64, S>), grid, block, 0, stream, p, nqb); break;
+        case 32: hipLaunchKernelGGL((prefill_f32_kernel<32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
+        case 64: hipLaunchKernelGGL((prefill_f32_kernel<64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 96:
-            if constexpr (S <= 2) hipLaunchKernelGGL((prefill_f32_kernel<96, S>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<96, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         case 128:
-            if constexpr (S <= 2) hipLaunchKernelGGL((prefill_f32_kernel<128, S>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<128, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         default: set_error("prefill f32 kernel: head_dim %d not in {32, 64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
@@ -276,9 +302,17 @@ int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
     int split = 1;
     if (wg1 <= (small_dim ? 4L : 2L) * cus) split = 2;
     if (split == 2 && small_dim && wg2 < 2L * cus) split = 4;
-    if (split == 4) return launch_split<4>(p, stream);
-    if (split == 2) return launch_split<2>(p, stream);
-    return launch_split<1>(p, stream);
+    // a mask tensor without its interval form is added element by element (the 16 bias registers leave no
+    // room for the key-split form at head_dim 96 / 128)
+    if (p.mask && !p.iv) {
+        if (!small_dim) split = 1;
+        if (split == 4) return launch_split<4, true>(p, stream);
+        if (split == 2) return launch_split<2, true>(p, stream);
+        return launch_split<1, true>(p, stream);
+    }
+    if (split == 4) return launch_split<4, false>(p, stream);
+    if (split == 2) return launch_split<2, false>(p, stream);
+    return launch_split<1, false>(p, stream);
 }
 
 }  // namespace fhip

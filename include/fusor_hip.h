@@ -183,8 +183,9 @@ int fhip_flash_attention_validate(const fhip_attn_args *args);
 
 /* Which kernel fhip_flash_attention will run for these arguments (host-only).  For a prefill call
  * with a mask tensor and a sufficient workspace in `args` this names the tiled kernel, which runs if
- * the mask turns out to be made of intervals (decided on the device); without the workspace it
- * names the general kernel. */
+ * the mask turns out to be made of intervals (decided on the device) and otherwise hands over, inside
+ * the same call, to the kernel that adds the mask values one by one (the f32 tiled kernel's own
+ * mask-adding form, the general kernel for 16-bit tensors); without the workspace it names that kernel. */
 int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id);
 
 /* Bytes of device workspace the call needs (0 for the single-pass kernels).  `compute_units`

@@ -103,8 +103,9 @@ def test_block_diagonal_mask_of_the_vision_blocks(device, dtype, D):
 @pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.BF16, 64), (fa.F32, 64)])
 @pytest.mark.parametrize("shape", ["bias", "two_runs", "nan", "positive_inf"])
 def test_masks_that_are_not_intervals_fall_back(device, dtype, D, shape):
-    """Finite biases, several visible runs, NaN or +inf entries: the general kernel adds the values as the
-    reference does (fusor flash_attention.rs:161-176)."""
+    """Finite biases, several visible runs, NaN or +inf entries: the mask values are added as the reference adds
+    them (fusor flash_attention.rs:161-176), by the f32 kernel's mask-adding form or, for 16-bit tensors, the
+    general kernel."""
     B, H, Hkv, Sq, Skv = 1, 2, 1, 140, 200
     q, k, v = _normal_qkv(23, B, H, Hkv, Sq, Skv, D)
     rng = np.random.default_rng(5)
@@ -176,3 +177,47 @@ def test_without_workspace_the_general_kernel_runs(device):
     fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
     ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), D ** -0.5, mask, "qk")
     assert_parity(out_t.to_numpy(), ref, TOL_16, "no workspace")
+
+
+
+@pytest.mark.parametrize("D,B,H,S", [(64, 3, 4, 200), (128, 2, 4, 333), (64, 8, 12, 512), (96, 1, 2, 100)])
+@pytest.mark.parametrize("workspace", [True, False])
+def test_padding_mask_with_a_large_finite_value(device, D, B, H, S, workspace):
+    """rbert masks padded keys with -10000.0 instead of -inf (models/rbert/src/raw/qwen/attention.rs:91-113,
+    BatchKeyMask, f32).  That is a finite bias, so no interval form exists; the f32 tiled kernel adds it element by
+    element, with or without scratch memory."""
+    q, k, v = _normal_qkv(28, B, H, H, S, S, D)
+    mask = np.zeros((B, S), np.float32)
+    for b in range(B):
+        mask[b, S - 1 - 13 * b:] = -10000.0
+    tq, tk, tv, tm = _tensors(device, fa.F32, q, k, v, mask)
+    out_t = fa.Tensor.empty(device, (B, H, S, D), fa.F32)
+    args = tq._attn_args(tk, tv, D ** -0.5, (tm, fa.MaskKind.BatchKeyMask), None, None, None, fa.KERNEL_AUTO, out_t)
+    if workspace:
+        need = ctypes.c_size_t()
+        fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+        ws, ws_bytes = device.workspace(max(need.value, 16))
+        args.workspace, args.workspace_bytes = ws, ws_bytes
+    kid = ctypes.c_int32()
+    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), device.compute_units, ctypes.byref(kid)))
+    assert kid.value == fa.KERNEL_PREFILL_F32
+    fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "batch_key")
+    assert_parity(out_t.to_numpy(), ref, TOL_F32, "-10000 padding mask")
+
+
+@pytest.mark.parametrize("D,S", [(64, 150), (128, 300), (32, 77)])
+def test_additive_bias_matrix_on_the_f32_tiled_kernel(device, D, S):
+    """A [Sq, Skv] tensor of finite biases (with a masked band and one fully masked row) through the tiled kernel."""
+    q, k, v = _normal_qkv(29, 2, 4, 2, S, S + 40, D)
+    rng = np.random.default_rng(8)
+    mask = rng.normal(0, 2, (S, S + 40)).astype(np.float32)
+    mask[:, 20:50] = NEG_INF
+    mask[5, :] = NEG_INF
+    tq, tk, tv, tm = _tensors(device, fa.F32, q, k, v, mask)
+    assert tq.selected_kernel(tk, tv, 0.1, (tm, fa.MaskKind.QKMask)) == fa.KERNEL_PREFILL_F32
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk")
+    keep = [r for r in range(S) if r != 5]
+    assert np.isnan(out[:, :, 5]).all() and np.isnan(ref[:, :, 5]).all()
+    assert_parity(out[:, :, keep], ref[:, :, keep], TOL_F32, "bias matrix")
