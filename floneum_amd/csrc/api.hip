@@ -177,7 +177,7 @@ static bool rows_vectorizable(const fhip_tensor4 &t, int eb) {
 static bool decode_eligible(const fhip_attn_args *a) {
     const uint32_t D = a->q.shape[3];
     if (a->q.shape[2] != 1) return false;
-    if (D % 8 != 0 || D < 8 || D > 128) return false;
+    if (D % 8 != 0 || D < 8 || D > 256) return false;
     const int eb = a->dtype == FHIP_F32 ? 4 : 2;
     if (!rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;
     if (a->k.stride[2] < 0 || a->v.stride[2] < 0) return false;

@@ -10,7 +10,7 @@
 //     O^T[dim][head] += V^T . P^T with V^T read by the transposing LDS load.  The softmax state of
 //     head j lives in the lanes with lane % 16 == j, so scores, probabilities and the output
 //     accumulator never change lanes.
-//   decode_vec_kernel (any head_dim multiple of 8 up to 128): LPK lanes x 8 elements per row, dot
+//   decode_vec_kernel (any head_dim multiple of 8 up to 256): LPK lanes x 8 elements per row, dot
 //     products on v_dot2, DPP reductions; every group of LPK lanes keeps its own softmax state.
 // Both keep (m, l, acc) in the log2 domain, merge lanes -> wavefront -> workgroup at the end and
 // write one partial (acc[D], m, l) per (batch, head, split).
@@ -153,7 +153,8 @@ struct Vec8<bf16_t> : Vec8Bits16 {
 
 template <int LPK>
 __device__ __forceinline__ float lpk_sum(float x) {
-    if constexpr (LPK == 16) return group_sum16(x);
+    if constexpr (LPK == 32) return group_sum32(x);
+    else if constexpr (LPK == 16) return group_sum16(x);
     else if constexpr (LPK == 8) return group_sum8(x);
     else return group_sum4(x);
 }
@@ -634,46 +635,49 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
         ns = max(1, min(ns, (len + p.chunk - 1) / p.chunk));  // split 0 is always written
     }
     const float *ws = (const float *)p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
-    const int d0 = threadIdx.x, d1 = threadIdx.x + 64;
-    float M = -INFINITY, L = 0.0f, A0 = 0.0f, A1 = 0.0f;
-    for (int s0 = 0; s0 < ns; s0 += 8) {
-        float ms[8], ls[8], a0[8], a1[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const bool ok = s0 + u < ns;
-            const float *src = ws + (int64_t)(ok ? s0 + u : s0) * (D + 2);
-            ms[u] = ok ? src[D] : -INFINITY;
-            ls[u] = ok ? src[D + 1] : 0.0f;
-            a0[u] = (ok && d0 < D) ? src[d0] : 0.0f;
-            a1[u] = (ok && d1 < D) ? src[d1] : 0.0f;
-        }
-        float Mn = M;
-#pragma unroll
-        for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
-        const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
-        const float c = __builtin_amdgcn_exp2f(M - Ms);
-        L *= c;
-        A0 *= c;
-        A1 *= c;
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
-            L += w * ls[u];
-            A0 += w * a0[u];
-            A1 += w * a1[u];
-        }
-        M = Mn;
-    }
     const int64_t ob = b * p.os[0] + h * p.os[1];
-    if (d0 < D) {
-        const float val = A0 / L;
-        if (p.out_f32) ((float *)p.out)[ob + d0 * p.os[3]] = val;
-        else ((T *)p.out)[ob + d0 * p.os[3]] = from_float<T>(val);
-    }
-    if (d1 < D) {
-        const float val = A1 / L;
-        if (p.out_f32) ((float *)p.out)[ob + d1 * p.os[3]] = val;
-        else ((T *)p.out)[ob + d1 * p.os[3]] = from_float<T>(val);
+    // 128 dims per round (one round up to head_dim 128, two at 256)
+    for (int dbase = 0; dbase < D; dbase += 128) {
+        const int d0 = dbase + threadIdx.x, d1 = dbase + threadIdx.x + 64;
+        float M = -INFINITY, L = 0.0f, A0 = 0.0f, A1 = 0.0f;
+        for (int s0 = 0; s0 < ns; s0 += 8) {
+            float ms[8], ls[8], a0[8], a1[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const bool ok = s0 + u < ns;
+                const float *src = ws + (int64_t)(ok ? s0 + u : s0) * (D + 2);
+                ms[u] = ok ? src[D] : -INFINITY;
+                ls[u] = ok ? src[D + 1] : 0.0f;
+                a0[u] = (ok && d0 < D) ? src[d0] : 0.0f;
+                a1[u] = (ok && d1 < D) ? src[d1] : 0.0f;
+            }
+            float Mn = M;
+#pragma unroll
+            for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
+            const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+            const float c = __builtin_amdgcn_exp2f(M - Ms);
+            L *= c;
+            A0 *= c;
+            A1 *= c;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
+                L += w * ls[u];
+                A0 += w * a0[u];
+                A1 += w * a1[u];
+            }
+            M = Mn;
+        }
+        if (d0 < D) {
+            const float val = A0 / L;
+            if (p.out_f32) ((float *)p.out)[ob + d0 * p.os[3]] = val;
+            else ((T *)p.out)[ob + d0 * p.os[3]] = from_float<T>(val);
+        }
+        if (d1 < D) {
+            const float val = A1 / L;
+            if (p.out_f32) ((float *)p.out)[ob + d1 * p.os[3]] = val;
+            else ((T *)p.out)[ob + d1 * p.os[3]] = from_float<T>(val);
+        }
     }
 }
 
@@ -720,8 +724,10 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         launch_vec<T, 4>(p, grid, stream, gt);
     } else if (p.D <= 64) {
         launch_vec<T, 8>(p, grid, stream, gt);
-    } else {
+    } else if (p.D <= 128) {
         launch_vec<T, 16>(p, grid, stream, gt);
+    } else {
+        launch_vec<T, 32>(p, grid, stream, gt);
     }
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));

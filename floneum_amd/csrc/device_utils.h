@@ -91,7 +91,7 @@ constexpr int DPP_QUAD_XOR2 = 0x4E;    // quad_perm [2,3,0,1]
 constexpr int DPP_ROW_HALF_MIRROR = 0x141;
 constexpr int DPP_ROW_MIRROR = 0x140;
 
-// sum over each aligned group of 4 / 8 / 16 lanes, result in every lane of the group
+// sum over each aligned group of 4 / 8 / 16 / 32 lanes, result in every lane of the group
 __device__ __forceinline__ float group_sum4(float x) {
     x += dpp_mov<DPP_QUAD_XOR1>(x);
     x += dpp_mov<DPP_QUAD_XOR2>(x);
@@ -105,6 +105,11 @@ __device__ __forceinline__ float group_sum8(float x) {
 __device__ __forceinline__ float group_sum16(float x) {
     x = group_sum8(x);
     x += dpp_mov<DPP_ROW_MIRROR>(x);
+    return x;
+}
+__device__ __forceinline__ float group_sum32(float x) {
+    x = group_sum16(x);
+    x += __shfl_xor(x, 16, 64);
     return x;
 }
 

@@ -234,7 +234,8 @@ def test_prefill_f32_key_split_forms(device, D, B, H, Sq, Skv, analytic, form):
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
-                                     (2, 40, 333), (8, 8, 100)])
+                                     (2, 40, 333), (8, 8, 100), (2, 256, 1500), (4, 192, 700), (1, 160, 300),
+                                     (8, 256, 260)])
 def test_decode_splitkv(device, dtype, G, D, Skv):
     B, Hkv = 3, 2
     q, k, v = _normal_qkv(12, B, Hkv * G, Hkv, 1, Skv, D, 0.5)
