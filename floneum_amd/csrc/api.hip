@@ -204,7 +204,7 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
 static bool prefill_f32_eligible(const fhip_attn_args *a) {
     if (a->dtype != FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
-    if (!(D == 32 || D == 64 || D == 96 || D == 128)) return false;
+    if (D % 4 != 0 || D > 128) return false;  // rows are padded with zeros to the next multiple of 32 on the way into LDS
     if (!(a->scale > 0.0f)) return false;
     if (!rows_vectorizable(a->q, 4) || !rows_vectorizable(a->k, 4) || !rows_vectorizable(a->v, 4)) return false;
     return true;

@@ -93,7 +93,8 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         const int qrow = min(query, p.Sq - 1);
         const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
-        for (int kc = 0; kc < D / 8; kc++) qreg[kc] = *(const float4_t *)(qp + 8 * kc + 4 * h2);
+        for (int kc = 0; kc < D / 8; kc++)
+            qreg[kc] = 8 * kc + 4 * h2 < p.D ? *(const float4_t *)(qp + 8 * kc + 4 * h2) : float4_t{0.f, 0.f, 0.f, 0.f};
     }
     const float *kg = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
     const float *vg = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
@@ -118,8 +119,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             const int cid = gtid + GT * i;
             const int row = cid / CPR, col = cid % CPR;
             const int key = min(j0 + row, p.Skv - 1);
-            kst[i] = *(const float4_t *)(kg + (int64_t)key * p.ks[2] + col * 4);
-            vst[i] = *(const float4_t *)(vg + (int64_t)key * p.vs[2] + col * 4);
+            const bool in_row = col * 4 < p.D;  // a head_dim below D is padded with zeros
+            kst[i] = in_row ? *(const float4_t *)(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            vst[i] = in_row ? *(const float4_t *)(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     };
     auto store_tile = [&]() {
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                op[dim * p.os[3]] = o[db][r] / l_tot;  // no visible key: 0/0 = NaN like the reference
+                if (dim < p.D) op[dim * p.os[3]] = o[db][r] / l_tot;  // no visible key: 0/0 = NaN like the reference
             }
     }
 }
@@ -274,7 +276,7 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
-    switch (p.D) {
+    switch ((p.D + 31) / 32 * 32) {  // the kernel's D is head_dim rounded up to a multiple of 32
         case 32: hipLaunchKernelGGL((prefill_f32_kernel<32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 64: hipLaunchKernelGGL((prefill_f32_kernel<64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 96:
@@ -283,7 +285,7 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
         case 128:
             if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<128, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
-        default: set_error("prefill f32 kernel: head_dim %d not in {32, 64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
+        default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;

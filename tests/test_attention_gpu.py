@@ -231,6 +231,29 @@ def test_prefill_f32_key_split_forms(device, D, B, H, Sq, Skv, analytic, form):
     assert_parity(out, ref, TOL_F32, f"f32 D{D} {form}")
 
 
+@pytest.mark.parametrize("D", [80, 48, 4, 100, 124, 20])
+@pytest.mark.parametrize("case", ["causal", "full_ragged", "bias"])
+def test_prefill_f32_head_dims_between_the_tile_widths(device, D, case):
+    """The f32 kernel pads head_dim to the next multiple of 32 with zeros on the way into LDS: Qwen-VL's vision
+    blocks have head_dim 80 (models/kalosm-llama/src/raw/vision), other widths are covered for the same price."""
+    B, H, Hkv = 2, 4, 2
+    Sq, Skv = (150, 150) if case == "causal" else (70, 333)
+    q, k, v = _normal_qkv(13, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    mask, kind, analytic, mt = None, None, None, None
+    if case == "causal":
+        analytic = (True, 0, 0)
+        mask, kind = _analytic_mask(Sq, Skv, True, 0, 0), "qk"
+    elif case == "bias":
+        mask, kind = np.random.default_rng(3).normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
+        mask[:, 100:140] = NEG_INF
+        mt = (fa.Tensor.from_numpy(device, mask, fa.F32), fa.MaskKind.QKMask)
+    assert tq.selected_kernel(tk, tv, 0.1, mt, analytic=analytic) == fa.KERNEL_PREFILL_F32
+    out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, kind)
+    assert_parity(out, ref, TOL_F32, f"f32 head_dim {D} {case}")
+
+
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
