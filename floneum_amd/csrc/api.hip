@@ -204,7 +204,7 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
 static bool prefill_f32_eligible(const fhip_attn_args *a) {
     if (a->dtype != FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
-    if (D % 4 != 0 || D > 128) return false;  // rows are padded with zeros to the next multiple of 32 on the way into LDS
+    if (D % 4 != 0 || D > 256) return false;  // rows are padded with zeros to the tile width on the way into LDS
     if (!(a->scale > 0.0f)) return false;
     if (!rows_vectorizable(a->q, 4) || !rows_vectorizable(a->k, 4) || !rows_vectorizable(a->v, 4)) return false;
     return true;
@@ -221,6 +221,9 @@ static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
     return a->workspace && ((uintptr_t)a->workspace & 15) == 0 && a->workspace_bytes >= mask_scratch_bytes(a);
 }
 
+// The f32 tiled kernel can add a mask tensor element by element (no scratch, no interval form) up to head_dim 128.
+static bool f32_adds_masks(const fhip_attn_args *a) { return a->q.shape[3] <= 128; }
+
 // assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
 // (the size query); otherwise a masked call without enough scratch takes the general kernel.
 static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_workspace = false) {
@@ -235,7 +238,7 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
         switch (f) {
             case FHIP_KERNEL_GENERIC: ok = true; break;
             case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a) && mask_ok; break;
-            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a); break;  // its mask-adding form needs no scratch
+            case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a) && (mask_ok || f32_adds_masks(a)); break;
             case FHIP_KERNEL_DECODE_SPLITKV: ok = decode_eligible(a); break;
             default: set_error("unknown force_kernel %d", f); return FHIP_ERR_INVALID_ARG;
         }
@@ -251,7 +254,7 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
         *id = FHIP_KERNEL_DECODE_SPLITKV;
     else if (prefill_mfma_eligible(a) && mask_ok)
         *id = FHIP_KERNEL_PREFILL_MFMA;
-    else if (prefill_f32_eligible(a))
+    else if (prefill_f32_eligible(a) && (mask_ok || f32_adds_masks(a)))
         *id = FHIP_KERNEL_PREFILL_F32;
     else
         *id = FHIP_KERNEL_GENERIC;
@@ -617,7 +620,8 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
         AttnParams pg = p;
         pg.only_if_bad = bad;
-        return id == FHIP_KERNEL_PREFILL_F32 ? launch_prefill_f32(pg, s->s) : launch_generic(pg, args->dtype, s->s);
+        return id == FHIP_KERNEL_PREFILL_F32 && f32_adds_masks(args) ? launch_prefill_f32(pg, s->s)
+                                                                    : launch_generic(pg, args->dtype, s->s);
     }
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;

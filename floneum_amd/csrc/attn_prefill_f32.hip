@@ -266,6 +266,203 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     }
 }
 
+// ---- head_dim 129 .. 256 (Gemma-3's key length is 256) -------------------------------------------------------
+// A wavefront cannot hold 256 dims of Q and O for 32 rows, so two wavefronts share the 32 rows: wavefront
+// `hf` of the pair owns dims [128 hf, 128 hf + 128) of Q, K, V and O.  Per key tile each computes its half of
+// the contraction S^T = K Q^T, the halves are exchanged through LDS (in the K tile's space, which is free by
+// then) and added, both run the same softmax on the same sums, and each accumulates its half of O^T.
+// Workgroup = 2 pairs = 64 query rows; K, V tiles of 32 keys x 256 dims (zero-padded above head_dim).
+constexpr int PFW_DP = 256, PFW_DH = 128;
+
+__global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(AttnParams p, int nqb) {
+    constexpr int BM = 64;
+    constexpr int KP = PFW_DP * 4 + 16;
+    constexpr int K_BYTES = PF32_BN * KP;
+    constexpr int CPR = PFW_DP / 4;
+    constexpr int NCH = PF32_BN * CPR / (64 * PF32_WAVES);
+    static_assert(PF32_WAVES * 16 * 256 <= K_BYTES, "the score exchange must fit the K tile's space");
+    __shared__ __attribute__((aligned(16))) char smem[2 * K_BYTES];
+    auto lds_base = (__attribute__((address_space(3))) char *)smem;
+
+    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int ln = lane & 31;
+    const int h2 = lane >> 5;
+    const int pr = wave >> 1;  // which 32 rows
+    const int hf = wave & 1;   // which half of the dims
+    const int d0 = PFW_DH * hf;
+
+    const int bh_count = p.B * p.H;
+    const int id = blockIdx.x;
+    const int qb = nqb - 1 - id / bh_count;
+    int rem = id % bh_count;
+    const int b = rem / p.H;
+    int h = rem % p.H;
+    if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
+    const int g = h / p.G;
+
+    const int q0 = qb * BM;
+    const int qw0 = q0 + 32 * pr;
+    const int query = qw0 + ln;
+    const RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
+    const bool wave_has_rows = qw0 < p.Sq;
+
+    float4_t qreg[PFW_DH / 8];
+    {
+        const int qrow = min(query, p.Sq - 1);
+        const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
+#pragma unroll
+        for (int kc = 0; kc < PFW_DH / 8; kc++) {
+            const int dim = d0 + 8 * kc + 4 * h2;
+            qreg[kc] = dim < p.D ? *(const float4_t *)(qp + dim) : float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    const float *kg = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
+    const float *vg = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
+
+    float16_t o[PFW_DH / 32];
+#pragma unroll
+    for (int db = 0; db < PFW_DH / 32; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    const float scale2 = p.scale * PF32_LOG2E;
+
+    // K and V take turns in one set of staging registers: V(j) is in flight while K(j) is multiplied, K(j+1)
+    // while V(j) is
+    float4_t st[NCH];
+    auto load_rows = [&](const float *base, const int64_t row_stride, int j0) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int cid = tid + 64 * PF32_WAVES * i;
+            const int row = cid / CPR, col = cid % CPR;
+            const int key = min(j0 + row, p.Skv - 1);
+            st[i] = col * 4 < p.D ? *(const float4_t *)(base + (int64_t)key * row_stride + col * 4)
+                                  : float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    auto store_rows = [&](int lds_off) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int cid = tid + 64 * PF32_WAVES * i;
+            const int row = cid / CPR, col = cid % CPR;
+            *LDS32_PTR(float4_t, lds_off + row * KP + col * 16) = st[i];
+        }
+    };
+
+    const int j_begin = (lo_wg / PF32_BN) * PF32_BN;
+    if (j_begin < hi_wg) load_rows(kg, p.ks[2], j_begin);
+
+    // every wavefront passes the same four barriers per tile, whether or not its rows see the tile
+    for (int j0 = j_begin; j0 < hi_wg; j0 += PF32_BN) {
+        store_rows(0);                    // K(j); its space is free since the last barrier of the previous tile
+        load_rows(vg, p.vs[2], j0);       // V(j), needed after the softmax
+        lds_barrier();
+        const bool tile_visible = wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;  // the same for both halves
+
+        // this half of S^T: contraction step (kc, i) uses dim d0 + 8 kc + 4 h2 + i on both operands
+        float16_t s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        if (tile_visible) {
+#pragma unroll
+            for (int kc = 0; kc < PFW_DH / 8; kc++) {
+                const float4_t a = *LDS32_PTR(float4_t, ln * KP + (d0 + 8 * kc + 4 * h2) * 4);
+#pragma unroll
+                for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], qreg[kc][i], s, 0, 0, 0);
+            }
+        }
+        lds_barrier();  // the K tile has been read: its space takes the exchange
+        if (tile_visible) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) *LDS32_PTR(float, wave * 4096 + r * 256 + lane * 4) = s[r];
+        }
+        lds_barrier();
+        if (tile_visible) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float other = *LDS32_PTR(float, (wave ^ 1) * 4096 + r * 256 + lane * 4);
+                s[r] = hf == 0 ? s[r] + other : other + s[r];  // low + high half on both wavefronts: identical sums
+            }
+        }
+        store_rows(K_BYTES);              // V(j); every wavefront is past P.V of the previous tile
+        if (j0 + PF32_BN < hi_wg) load_rows(kg, p.ks[2], j0 + PF32_BN);  // K(j+1)
+        lds_barrier();                    // V(j) visible, the exchange has been read
+        if (!tile_visible) continue;
+
+        // element r is key j0 + 8 (r / 4) + 4 h2 + r % 4 for query `query`
+        if (!(j0 >= rb.full_lo_w && j0 + PF32_BN <= rb.full_hi_w)) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                s[r] = (key >= rb.klo && key < rb.khi) ? s[r] : -INFINITY;
+            }
+        }
+
+        float mx = s[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[r]);
+        mx = half_swap_max32(mx);
+        const float m_new = fmaxf(m, mx * scale2);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
+        m = m_new;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale2, -m_safe));
+            psum += s[r];
+        }
+        l = l * corr + psum;
+#pragma unroll
+        for (int db = 0; db < PFW_DH / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] *= corr;
+
+        // this half of O^T += V^T . P^T
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int krow = 8 * (r >> 2) + 4 * h2 + (r & 3);
+#pragma unroll
+            for (int db = 0; db < PFW_DH / 32; db++) {
+                const float a = *LDS32_PTR(float, K_BYTES + krow * KP + (d0 + 32 * db + ln) * 4);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db], 0, 0, 0);
+            }
+        }
+    }
+
+    const float l_tot = half_swap_sum32(l);
+    if (query < p.Sq) {
+        float *op = (float *)p.out + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
+#pragma unroll
+        for (int db = 0; db < PFW_DH / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int dim = d0 + 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                if (dim < p.D) op[dim * p.os[3]] = o[db][r] / l_tot;  // no visible key: 0/0 = NaN like the reference
+            }
+    }
+}
+
+static int launch_wide(const AttnParams &p, hipStream_t stream) {
+    if (p.mask && !p.iv) {
+        set_error("prefill f32: a mask tensor without its interval form is not supported above head_dim 128");
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    const int nqb = (p.Sq + 63) / 64;
+    const long blocks = (long)nqb * p.B * p.H;
+    if (blocks > 0x7fffffffL) {
+        set_error("prefill f32: too many workgroups (%ld)", blocks);
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(prefill_f32_wide_kernel, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), 0, stream, p, nqb);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
 template <int S, bool BIAS>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
     constexpr int BM = 32 * (PF32_WAVES / S);
@@ -292,6 +489,7 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
 }
 
 int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
+    if (p.D > 128) return launch_wide(p, stream);
     // Split the keys of a query block over 2 or 4 wavefront groups while the unsplit grid is only a few
     // workgroups per CU: the longest (last causal) query block then sets the run time, and halving it pays
     // even when every CU has work.  Measured break-even: about 4 workgroups per CU at head_dim <= 64, 2 above

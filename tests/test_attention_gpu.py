@@ -254,6 +254,36 @@ def test_prefill_f32_head_dims_between_the_tile_widths(device, D, case):
     assert_parity(out, ref, TOL_F32, f"f32 head_dim {D} {case}")
 
 
+@pytest.mark.parametrize("D", [256, 192, 132, 160])
+@pytest.mark.parametrize("case", ["causal", "full_ragged", "window_offset", "mask_tensor", "bias_tensor"])
+def test_prefill_f32_wide_heads(device, D, case):
+    """head_dim 129..256 (Gemma-3's key length is 256): two wavefronts share 32 query rows, each owning half of
+    the dims; the halves of every score are exchanged and added before the softmax."""
+    B, H, Hkv = 2, 4, 2
+    Sq, Skv = {"causal": (150, 150), "full_ragged": (70, 333), "window_offset": (97, 400), "mask_tensor": (130, 130),
+               "bias_tensor": (64, 100)}[case]
+    q, k, v = _normal_qkv(14, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    mask, kind, analytic, mt, want = None, None, None, None, fa.KERNEL_PREFILL_F32
+    if case == "causal":
+        analytic = (True, 0, 0)
+    elif case == "window_offset":
+        analytic = (True, Skv - Sq, 120)
+    elif case == "mask_tensor":
+        mask = oracle.get_mask(Sq, 0, 50)
+        mt = (fa.Tensor.from_numpy(device, mask, fa.F32), fa.MaskKind.QKMask)
+    elif case == "bias_tensor":  # no interval form and no mask-adding form this wide: the general kernel
+        mask = np.random.default_rng(3).normal(0, 1, (Sq, Skv)).astype(np.float32)
+        mt = (fa.Tensor.from_numpy(device, mask, fa.F32), fa.MaskKind.QKMask)
+    if analytic is not None:
+        mask = _analytic_mask(Sq, Skv, *analytic)
+    out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, None if mask is None else "qk")
+    assert_parity(out, ref, TOL_F32, f"f32 head_dim {D} {case}")
+    if mt is None:
+        assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == want
+
+
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
