@@ -134,6 +134,8 @@ SYMBOLS = {
     "fhip_kv_cache_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4)]),
+    "fhip_mask_get_mask_device": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int32,
+                                                 ctypes.c_uint64, _P]),
     "fhip_norm_rope": (ctypes.c_int, [_P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
                                       ctypes.c_int, ctypes.POINTER(CTensor4), ctypes.c_int]),
     "fhip_kv_cache_norm_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRopeTables),
@@ -542,6 +544,20 @@ class MaskCache:
             t = Tensor.from_numpy(device, host, self.dtype) if device is not None else None
             return AttentionMask(t, host, analytic)
         return AttentionMask(base._mask, base.host, analytic)
+
+    def get_mask_on_device(self, seq_len, seqlen_offset, sliding_window_size, device):
+        """The same tensor written by a kernel: no host loop over seq_len^2 elements, no upload."""
+        L = lib()
+        has_w = sliding_window_size is not None
+        w = int(sliding_window_size) if has_w else 0
+        rows, cols = ctypes.c_uint32(), ctypes.c_uint64()
+        check(L.fhip_mask_get_mask_shape(seq_len, seqlen_offset, int(has_w), w, ctypes.byref(rows), ctypes.byref(cols)))
+        t = Tensor.empty(device, (rows.value, cols.value), self.dtype)
+        check(L.fhip_mask_get_mask_device(device.stream, self.dtype, seq_len, seqlen_offset, int(has_w), w,
+                                          ctypes.c_void_p(t.buffer.ptr)))
+        am = CAnalyticMask()
+        rc = L.fhip_mask_get_analytic(seq_len, seqlen_offset, int(has_w), w, ctypes.byref(am))
+        return AttentionMask(t, None, am if rc == OK else None)
 
 
 # ---- KV cache -----------------------------------------------------------------------------------------

@@ -715,6 +715,17 @@ int fhip_mask_get_mask(fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offse
     return FHIP_OK;
 }
 
+int fhip_mask_get_mask_device(fhip_stream *s, fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
+                              uint64_t window, void *out_device) {
+    if (!s || !dtype_ok(dtype) || (seq_len && !out_device)) {
+        set_error("mask_get_mask_device: NULL stream, bad dtype or NULL out");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const uint64_t off = mask_offset(seq_len, seqlen_offset, has_window, window);
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return launch_mask_build(out_device, dtype, seq_len, off + seq_len, off, has_window ? 1 : 0, window, s->s);
+}
+
 int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window, uint64_t window,
                            fhip_analytic_mask *out) {
     if (!out) {

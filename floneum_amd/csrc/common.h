@@ -42,6 +42,10 @@ size_t mask_intervals_bytes(int rows);
 // fills iv[rows] and *bad (zeroed first) from the mask described by p.mask / p.ms0 / p.ms1 / p.mask_kind
 int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32_t *bad, hipStream_t stream);
 
+// writes get_mask's [rows, cols] tensor (0 / -inf bit patterns of `dtype`) into device memory; off = cols - rows
+int launch_mask_build(void *out, fhip_dtype dtype, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
+                      uint64_t window, hipStream_t stream);
+
 // thread-local error text
 void set_error(const char *fmt, ...);
 int hip_fail(hipError_t e, const char *what);

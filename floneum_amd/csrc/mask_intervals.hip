@@ -6,8 +6,12 @@
 // has, per row, ONE run of zeros.  This kernel checks that per row and writes the run as {lo, hi}; the
 // tiled attention kernels then mask by interval and never read the [rows, kv_seq_len] tensor again.  A
 // row that is anything else (finite biases, several runs, NaN) is counted in *bad and the call falls
-// back to the general kernel, which adds the mask values as the reference does
+// back to a kernel that adds the mask values as the reference does
 // (fusor-ml/fusor/src/composite/flash_attention.rs:161-176).
+//
+// The other direction lives here too: mask_build_kernel writes the tensor MaskCache::get_mask would build
+// (mask_cache.rs:36-116) straight into device memory, for callers that want the tensor without the O(seq^2)
+// host loop and the upload.
 #include "common.h"
 #include "device_utils.h"
 
@@ -98,6 +102,39 @@ int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32
     else
         hipLaunchKernelGGL(mask_intervals_kernel<2>, grid, block, 0, stream, (const char *)p.mask, p.ms0, p.ms1, rows, cols,
                            dtype == FHIP_F16 ? 0xFC00u : 0xFF80u, vec_ok, iv, bad);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+// element (i, j) of get_mask(seq_len, seqlen_offset, window): columns below `off` are visible cached keys, the
+// rest is the causal (j - off > i) or sliding-window (i < j - off or j - off + window <= i) base mask
+template <typename W>
+__global__ __launch_bounds__(256) void mask_build_kernel(W *out, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
+                                                         uint64_t window, W ninf) {
+    const uint64_t total = (uint64_t)rows * cols;
+    for (uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256) {
+        const uint64_t i = idx / cols, c = idx % cols;
+        bool masked = false;
+        if (c >= off) {
+            const uint64_t j = c - off;
+            masked = has_window ? (i < j || j + window <= i) : (j > i);
+        }
+        out[idx] = masked ? ninf : (W)0;
+    }
+}
+
+int launch_mask_build(void *out, fhip_dtype dtype, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
+                      uint64_t window, hipStream_t stream) {
+    const uint64_t total = (uint64_t)rows * cols;
+    if (total == 0) return FHIP_OK;
+    const uint64_t blocks = (total + 255) / 256;
+    const dim3 grid((unsigned)(blocks < 65536 * 4 ? blocks : 65536 * 4)), block(256);
+    if (dtype == FHIP_F32)
+        hipLaunchKernelGGL(mask_build_kernel<uint32_t>, grid, block, 0, stream, (uint32_t *)out, rows, cols, off, has_window,
+                           window, 0xFF800000u);
+    else
+        hipLaunchKernelGGL(mask_build_kernel<uint16_t>, grid, block, 0, stream, (uint16_t *)out, rows, cols, off, has_window,
+                           window, (uint16_t)(dtype == FHIP_F16 ? 0xFC00u : 0xFF80u));
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
 }

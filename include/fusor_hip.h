@@ -215,6 +215,11 @@ int fhip_mask_get_mask_shape(uint32_t seq_len, uint64_t seqlen_offset, int32_t h
                              uint64_t window, uint32_t *rows, uint64_t *cols);
 int fhip_mask_get_mask(fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset,
                        int32_t has_window, uint64_t window, void *out);
+/* The same tensor written by a kernel into device memory ([rows, cols] of fhip_mask_get_mask_shape, row-major):
+ * no O(seq_len^2) host loop, no upload.  seqlen_offset = 0 without a window gives AttentionMask::causal,
+ * with one MaskCache::create_sliding_window_mask.  Asynchronous on `s`. */
+int fhip_mask_get_mask_device(fhip_stream *s, fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset,
+                              int32_t has_window, uint64_t window, void *out_device);
 /* The analytic descriptor equal to get_mask(seq_len, seqlen_offset, window) (no tensor built). */
 int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
                            uint64_t window, fhip_analytic_mask *out);

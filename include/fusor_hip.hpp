@@ -297,21 +297,21 @@ class MaskCache {
         fhip_analytic_mask am{};
         const bool have_am = fhip_mask_get_analytic(seq_len, seqlen_offset, has_w, w, &am) == FHIP_OK;
         const auto key = std::make_pair(seq_len, has_w ? (int64_t)w : (int64_t)-1);
+        // the tensors are written by a kernel (bit for bit what the reference's host loops build)
         auto it = masks_.find(key);
         if (it == masks_.end()) {
-            std::vector<char> host((size_t)seq_len * seq_len * dtype_bytes(dtype_));
-            if (has_w) check(fhip_mask_sliding_window((fhip_dtype)dtype_, seq_len, w, host.data()));
-            else check(fhip_mask_causal((fhip_dtype)dtype_, seq_len, host.data()));
             const uint32_t shape[2] = {seq_len, seq_len};
-            it = masks_.emplace(key, AttentionMask(Tensor<2>::from_slice(dev, dtype_, shape, host.data()))).first;
+            Tensor<2> base = Tensor<2>::empty(dev, dtype_, shape);
+            check(fhip_mask_get_mask_device(dev.stream(), (fhip_dtype)dtype_, seq_len, 0, has_w, w, base.c2().ptr));
+            it = masks_.emplace(key, AttentionMask(base)).first;
         }
         std::optional<fhip_analytic_mask> oam;
         if (have_am) oam = am;
         if (cols > seq_len) {  // left padding with zeros (mask_cache.rs:73-85)
-            std::vector<char> host((size_t)rows * cols * dtype_bytes(dtype_));
-            check(fhip_mask_get_mask((fhip_dtype)dtype_, seq_len, seqlen_offset, has_w, w, host.data()));
             const uint32_t shape[2] = {rows, (uint32_t)cols};
-            return AttentionMask(Tensor<2>::from_slice(dev, dtype_, shape, host.data()), oam);
+            Tensor<2> full = Tensor<2>::empty(dev, dtype_, shape);
+            check(fhip_mask_get_mask_device(dev.stream(), (fhip_dtype)dtype_, seq_len, seqlen_offset, has_w, w, full.c2().ptr));
+            return AttentionMask(full, oam);
         }
         return AttentionMask(it->second.mask(), oam);
     }

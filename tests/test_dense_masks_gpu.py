@@ -221,3 +221,18 @@ def test_additive_bias_matrix_on_the_f32_tiled_kernel(device, D, S):
     keep = [r for r in range(S) if r != 5]
     assert np.isnan(out[:, :, 5]).all() and np.isnan(ref[:, :, 5]).all()
     assert_parity(out[:, :, keep], ref[:, :, keep], TOL_F32, "bias matrix")
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16, fa.BF16])
+def test_masks_built_on_the_device_equal_the_host_builders(device, dtype):
+    """fhip_mask_get_mask_device writes, bit for bit, what MaskCache::get_mask builds on the host
+    (mask_cache.rs:36-116), for the reference's own cases (mask_cache.rs:120-175) and a sweep."""
+    cases = [(3, 0, None), (4, 0, 2), (2, 3, None), (1, 4095, None), (5, 2, 3), (5, 2, 9), (7, 100, 4), (64, 1000, 64),
+             (130, 270, None), (300, 0, 100), (1, 0, 1), (9, 5, 0)]
+    mc = fa.MaskCache(dtype)
+    for seq, off, w in cases:
+        on_dev = mc.get_mask_on_device(seq, off, w, device).mask().to_numpy()
+        host = oracle.get_mask(seq, off, w)
+        assert on_dev.shape == host.shape, (seq, off, w)
+        want = fa.Tensor.from_numpy(device, host, dtype).to_numpy()
+        assert np.array_equal(on_dev.view(np.uint8), want.view(np.uint8)), (seq, off, w)
