@@ -134,6 +134,10 @@ SYMBOLS = {
     "fhip_kv_cache_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4)]),
+    "fhip_stream_begin_capture": (ctypes.c_int, [_P]),
+    "fhip_stream_end_capture": (ctypes.c_int, [_P, _PP]),
+    "fhip_graph_launch": (ctypes.c_int, [_P, _P]),
+    "fhip_graph_destroy": (ctypes.c_int, [_P]),
     "fhip_mask_get_mask_device": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int32,
                                                  ctypes.c_uint64, _P]),
     "fhip_norm_rope": (ctypes.c_int, [_P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
@@ -236,6 +240,10 @@ class Device:
     def synchronize(self):
         check(lib().fhip_stream_synchronize(self.stream))
 
+    def capture(self):
+        """Context manager: library calls made inside are recorded into a Graph instead of running."""
+        return _Capture(self)
+
     def workspace(self, nbytes):
         """A grow-only scratch buffer owned by the device object (the caller of the C ABI owns the
         workspace; this is the Python caller's)."""
@@ -246,6 +254,41 @@ class Device:
             self._workspace = self.malloc(nbytes)
             self._workspace_bytes = nbytes
         return self._workspace, self._workspace_bytes
+
+
+class Graph:
+    """A recorded sequence of library calls (fhip_graph): launch() replays it with one submission."""
+
+    def __init__(self, device, handle):
+        self.device, self.handle = device, handle
+
+    def launch(self):
+        check(lib().fhip_graph_launch(self.handle, self.device.stream))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().fhip_graph_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class _Capture:
+    def __init__(self, device):
+        self.device, self.graph = device, None
+
+    def __enter__(self):
+        check(lib().fhip_stream_begin_capture(self.device.stream))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        h = ctypes.c_void_p()
+        rc = lib().fhip_stream_end_capture(self.device.stream, ctypes.byref(h))
+        if exc_type is None:
+            check(rc)
+            self.graph = Graph(self.device, h)
+        return False
 
 
 class Buffer:

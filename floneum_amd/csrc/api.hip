@@ -21,6 +21,11 @@ struct fhip_event {
     fhip_device *dev;
     hipEvent_t e;
 };
+struct fhip_graph {
+    fhip_device *dev;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
 
 namespace fhip {
 
@@ -478,6 +483,69 @@ int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes) {
     }
     if (!bytes) return FHIP_OK;
     FHIP_HIP_CHECK(hipMemsetAsync(dst, value, bytes, s->s));
+    return FHIP_OK;
+}
+
+// ---- stream capture: a sequence of calls recorded once and replayed with one launch --------------------
+
+int fhip_stream_begin_capture(fhip_stream *s) {
+    if (!s) {
+        set_error("stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    FHIP_HIP_CHECK(hipStreamBeginCapture(s->s, hipStreamCaptureModeThreadLocal));
+    return FHIP_OK;
+}
+
+int fhip_stream_end_capture(fhip_stream *s, fhip_graph **out) {
+    if (!s || !out) {
+        set_error("stream/out is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *out = nullptr;
+    hipGraph_t g = nullptr;
+    FHIP_HIP_CHECK(hipStreamEndCapture(s->s, &g));
+    if (!g) {
+        set_error("the capture produced no graph (a call in it failed)");
+        return FHIP_ERR_HIP;
+    }
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return hip_fail(e, "hipGraphInstantiate");
+    }
+    fhip_graph *gr = new (std::nothrow) fhip_graph();
+    if (!gr) {
+        (void)hipGraphExecDestroy(ex);
+        (void)hipGraphDestroy(g);
+        set_error("out of host memory");
+        return FHIP_ERR_HIP;
+    }
+    gr->dev = s->dev;
+    gr->graph = g;
+    gr->exec = ex;
+    *out = gr;
+    return FHIP_OK;
+}
+
+int fhip_graph_launch(fhip_graph *g, fhip_stream *s) {
+    if (!g || !s) {
+        set_error("graph/stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    FHIP_HIP_CHECK(hipGraphLaunch(g->exec, s->s));
+    return FHIP_OK;
+}
+
+int fhip_graph_destroy(fhip_graph *g) {
+    if (!g) return FHIP_OK;
+    hipError_t e1 = hipGraphExecDestroy(g->exec), e2 = hipGraphDestroy(g->graph);
+    delete g;
+    if (e1 != hipSuccess) return hip_fail(e1, "hipGraphExecDestroy");
+    if (e2 != hipSuccess) return hip_fail(e2, "hipGraphDestroy");
     return FHIP_OK;
 }
 

@@ -54,13 +54,16 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
     const int max_chunk = ragged && units >= target ? 512 : 1024;
-    const int min_chunk = 256;
+    // few (batch, kv head) units, e.g. batch 1: down to one workgroup step of 128 keys per split, because a
+    // workgroup's steps run one after the other and each costs a memory latency.  Up to 256 keys the matrix-core
+    // variant is quicker unsplit than with a second launch to merge two splits (measured 6.6 vs 8.6 us).
+    const int min_chunk = 128;
     long ns = (target + units - 1) / units;
     const long ns_max = (Skv + min_chunk - 1) / min_chunk;
     const long ns_min = (Skv + max_chunk - 1) / max_chunk;
     if (ns > ns_max) ns = ns_max;
     if (ns < ns_min) ns = ns_min;
-    if (ns < 1) ns = 1;
+    if (ns < 1 || (Skv <= 256 && decode_use_mfma(D, f32))) ns = 1;
     long c = (Skv + ns - 1) / ns;
     c = (c + 127) / 128 * 128;  // a workgroup step covers 128 keys
     *chunk = (int)c;
@@ -209,7 +212,11 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
         const int h = h0 + min(hh, nh - 1);
         const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1];
         q[hh].zero();
-        if (active) q[hh].gather(qp + (int64_t)(c * 8) * p.qs[3], p.qs[3]);
+        if (active) {
+            // one 16 / 32-byte load when the row is contiguous and aligned, element by element otherwise
+            if (p.qs[3] == 1 && (((uintptr_t)(qp + c * 8)) & 15) == 0) q[hh].load(qp + c * 8);
+            else q[hh].gather(qp + (int64_t)(c * 8) * p.qs[3], p.qs[3]);
+        }
     }
 
     const T *kbase = (const T *)p.k + b * p.ks[0] + g * p.ks[1] + c * 8;
@@ -622,9 +629,10 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
 }
 
 // ---- pass 2 -------------------------------------------------------------------------------------
-// One 64-lane wavefront per (batch, head); up to 8 partials are fetched in one round of loads.
+// One 64-lane wavefront per (batch, head); up to U partials are fetched in one round of loads (a round costs
+// one memory latency, so calls with many splits take the wide form).
 
-template <typename T>
+template <typename T, int U>
 __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
     const int bh = blockIdx.x;
     const int h = bh % p.H, b = bh / p.H;
@@ -640,10 +648,10 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
     for (int dbase = 0; dbase < D; dbase += 128) {
         const int d0 = dbase + threadIdx.x, d1 = dbase + threadIdx.x + 64;
         float M = -INFINITY, L = 0.0f, A0 = 0.0f, A1 = 0.0f;
-        for (int s0 = 0; s0 < ns; s0 += 8) {
-            float ms[8], ls[8], a0[8], a1[8];
+        for (int s0 = 0; s0 < ns; s0 += U) {
+            float ms[U], ls[U], a0[U], a1[U];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < U; u++) {
                 const bool ok = s0 + u < ns;
                 const float *src = ws + (int64_t)(ok ? s0 + u : s0) * (D + 2);
                 ms[u] = ok ? src[D] : -INFINITY;
@@ -653,14 +661,14 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
             }
             float Mn = M;
 #pragma unroll
-            for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
+            for (int u = 0; u < U; u++) Mn = fmaxf(Mn, ms[u]);
             const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
             const float c = __builtin_amdgcn_exp2f(M - Ms);
             L *= c;
             A0 *= c;
             A1 *= c;
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < U; u++) {
                 const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
                 L += w * ls[u];
                 A0 += w * a0[u];
@@ -679,6 +687,13 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
             else ((T *)p.out)[ob + d1 * p.os[3]] = from_float<T>(val);
         }
     }
+}
+
+template <typename T>
+static void launch_combine(const AttnParams &p, hipStream_t stream) {
+    const dim3 grid((unsigned)(p.B * p.H)), block(64);
+    if (p.nsplit <= 8) hipLaunchKernelGGL((decode_combine_kernel<T, 8>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((decode_combine_kernel<T, 32>), grid, block, 0, stream, p);
 }
 
 template <typename T, int LPK>
@@ -714,7 +729,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
             FHIP_HIP_CHECK(hipGetLastError());
             if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
             if (p.nsplit > 1) {
-                hipLaunchKernelGGL(decode_combine_kernel<T>, dim3((unsigned)(p.B * p.H)), dim3(64), 0, stream, p);
+                launch_combine<T>(p, stream);
                 FHIP_HIP_CHECK(hipGetLastError());
             }
             return FHIP_OK;
@@ -732,7 +747,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
     if (p.nsplit > 1) {
-        hipLaunchKernelGGL(decode_combine_kernel<T>, dim3((unsigned)(p.B * p.H)), dim3(64), 0, stream, p);
+        launch_combine<T>(p, stream);
         FHIP_HIP_CHECK(hipGetLastError());
     }
     return FHIP_OK;

@@ -168,6 +168,20 @@ int fhip_memcpy_d2h(fhip_stream *s, void *dst, const void *src, size_t bytes); /
 int fhip_memcpy_d2d(fhip_stream *s, void *dst, const void *src, size_t bytes);
 int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes);
 
+/* Stream capture.  A decode step is a handful of short launches (rope, cache write, attention, merge), so a
+ * serving loop is bound by launch cost; everything this library queues between begin and end is recorded
+ * into one graph instead of running, and fhip_graph_launch replays it with a single submission.  All entry
+ * points that take a stream can be captured EXCEPT those that may allocate or synchronise: fhip_malloc /
+ * fhip_free, fhip_memcpy_d2h, fhip_stream_synchronize, fhip_kv_cache_append* when the cache has to grow.
+ * Pointers and shapes are frozen at capture time; what may change between replays is the CONTENT of device
+ * memory, e.g. the int32 kv_lens a ragged decode call reads, the new rows, the cache itself.
+ * (The reference has no counterpart: WGPU command buffers are rebuilt every step.) */
+typedef struct fhip_graph fhip_graph;
+int fhip_stream_begin_capture(fhip_stream *s);
+int fhip_stream_end_capture(fhip_stream *s, fhip_graph **out);
+int fhip_graph_launch(fhip_graph *g, fhip_stream *s);
+int fhip_graph_destroy(fhip_graph *g);
+
 /* HIP events on a library stream (timing in benchmarks; the reference has no GPU timers). */
 int fhip_event_create(fhip_device *dev, fhip_event **out);
 int fhip_event_destroy(fhip_event *e);

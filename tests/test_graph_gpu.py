@@ -1,0 +1,101 @@
+"""GPU tests of stream capture: library calls recorded into a graph and replayed.
+
+A serving loop is bound by launch cost (a batch-1 decode step is a few launches of ~10 us), so the calls of a
+step are meant to be recorded once and replayed.  What changes between replays is the content of device
+memory only: the query rows, the int32 key counts a ragged decode call reads, the cache.  Every replay is
+checked against the same calls made eagerly on the same state, with eager work and synchronisation between
+the replays.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import floneum_amd as fa
+import oracle
+from conftest import TOL_16, TOL_F32, assert_parity
+from test_attention_gpu import _normal_qkv, rounded
+
+pytestmark = pytest.mark.gpu
+
+
+def _upload(device, t, host):
+    host = np.ascontiguousarray(host)
+    fa.check(fa.lib().fhip_memcpy_h2d(device.stream, ctypes.c_void_p(t.buffer.ptr), host.ctypes.data_as(ctypes.c_void_p),
+                                      host.nbytes))
+
+
+def _bound_args(device, q, k, v, scale, out, **kw):
+    args = q._attn_args(k, v, scale, kw.get("mask"), kw.get("analytic"), kw.get("kv_lens"), None, fa.KERNEL_AUTO, out)
+    need = ctypes.c_size_t()
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+    if need.value:
+        ws = fa.Buffer(device, need.value)
+        args.workspace, args.workspace_bytes = ws.ptr, need.value
+        args._keep.append(ws)
+    return args
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_decode_step_replayed_with_growing_key_counts(device, dtype):
+    """rope(q) + ragged split-KV decode over a fixed cache buffer, recorded once; the key counts and the query change
+    between replays."""
+    B, H, Hkv, D, Smax = 3, 8, 2, 128, 700
+    _, k, v = _normal_qkv(51, B, H, Hkv, 1, Smax, D, 0.5)
+    tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (k, v))
+    rc = fa.RopeCache(D, 1024, 10000.0, device)
+    q_in = fa.Tensor.empty(device, (B, H, 1, D), fa.F32)
+    q_rot = fa.Tensor.empty(device, (B, H, 1, D), dtype)
+    out = fa.Tensor.empty(device, (B, H, 1, D), dtype)
+    lens_t = fa.IntTensor(device, np.array([1, 1, 1], np.int32))
+    args = _bound_args(device, q_rot, tk, tv, D ** -0.5, out, kv_lens=lens_t)
+    tables = rc._tables(5, False)
+    cq, cr = q_in._c4(), q_rot._c4()
+
+    def step():
+        fa.check(fa.lib().fhip_rope(device.stream, ctypes.byref(tables), ctypes.byref(cq), fa.F32, ctypes.byref(cr), dtype))
+        fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+
+    with device.capture() as cap:
+        step()
+    graph = cap.graph
+    tol = TOL_F32 if dtype == fa.F32 else TOL_16
+    for it, lens in enumerate(([5, 700, 333], [6, 1, 334], [700, 700, 700], [129, 64, 2])):
+        q = _normal_qkv(60 + it, B, H, Hkv, 1, 1, D, 0.5)[0]
+        _upload(device, q_in, q)
+        _upload(device, lens_t, np.array(lens, np.int32))
+        graph.launch()
+        replayed = out.to_numpy()
+        step()                                    # the same calls, eagerly, on the same state
+        eager = out.to_numpy()
+        assert np.array_equal(replayed.view(np.uint8), eager.view(np.uint8)), f"replay {it}"
+        q_r = rounded(oracle.rope(q, rc.cos_host, rc.sin_host, 5), dtype)
+        for b in range(B):
+            ref = oracle.flash_attention(q_r[b:b + 1], rounded(k[b:b + 1, :, :lens[b]], dtype),
+                                         rounded(v[b:b + 1, :, :lens[b]], dtype), D ** -0.5)
+            assert_parity(replayed[b:b + 1], ref, tol, f"replay {it} sequence {b}")
+
+
+def test_masked_prefill_replayed(device):
+    """A prefill call with a mask tensor is three launches (interval scan, tiled kernel, the kernel for masks that are
+    not intervals) and a kernel that clears the scan's counter: all of it is recorded, and the mask content may
+    change between replays, including from the interval form to a bias."""
+    B, H, Hkv, S, D = 1, 4, 2, 200, 64
+    q, k, v = _normal_qkv(52, B, H, Hkv, S, S, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    tm = fa.Tensor.empty(device, (S, S), fa.F32)
+    out = fa.Tensor.empty(device, (B, H, S, D), fa.F32)
+    args = _bound_args(device, tq, tk, tv, D ** -0.5, out, mask=(tm, fa.MaskKind.QKMask))
+    _upload(device, tm, oracle.get_mask(S, 0))
+    with device.capture() as cap:
+        fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    rng = np.random.default_rng(1)
+    bias = rng.normal(0, 1, (S, S)).astype(np.float32)
+    bias[:, 150:] = float("-inf")
+    for it, mask in enumerate((oracle.get_mask(S, 0), bias, oracle.get_mask(S, 0, 40), bias * 2)):
+        _upload(device, tm, mask)
+        cap.graph.launch()
+        got = out.to_numpy()
+        ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk")
+        assert_parity(got, ref, TOL_F32, f"replay {it}")
+        _ = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()   # unrelated eager work between the replays
