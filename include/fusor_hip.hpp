@@ -49,6 +49,22 @@ inline size_t dtype_bytes(DType d) { return d == DType::F32 ? 4 : 2; }
 enum class MaskKind { QKMask = FHIP_MASK_QK, BatchKeyMask = FHIP_MASK_BATCH_KEY };
 
 /// One GPU plus one stream.  Cheap to copy (shared handle), like fusor's Device.
+/// A recorded sequence of library calls (fhip_graph); launch() replays it with one submission.
+class Graph {
+    struct Inner {
+        fhip_graph *g = nullptr;
+        ~Inner() {
+            if (g) fhip_graph_destroy(g);
+        }
+    };
+    std::shared_ptr<Inner> in_;
+    fhip_stream *stream_;
+
+   public:
+    Graph(fhip_graph *g, fhip_stream *s) : in_(std::make_shared<Inner>()), stream_(s) { in_->g = g; }
+    void launch() const { check(fhip_graph_launch(in_->g, stream_)); }
+};
+
 class Device {
     struct Inner {
         fhip_device *dev = nullptr;
@@ -89,6 +105,23 @@ class Device {
         return in_->workspace;
     }
     size_t workspace_bytes() const { return in_->workspace_bytes; }
+    /// Records the library calls `body` makes on this device's stream instead of running them.  The body must not
+    /// allocate or read back (pre-allocate outputs and workspace; no as_slice / to_host inside).
+    template <typename F>
+    Graph capture(F &&body) const {
+        check(fhip_stream_begin_capture(in_->stream));
+        try {
+            body();
+        } catch (...) {
+            fhip_graph *dropped = nullptr;
+            (void)fhip_stream_end_capture(in_->stream, &dropped);
+            if (dropped) fhip_graph_destroy(dropped);
+            throw;
+        }
+        fhip_graph *g = nullptr;
+        check(fhip_stream_end_capture(in_->stream, &g));
+        return Graph(g, in_->stream);
+    }
 };
 
 /// Owning device allocation, freed with the last tensor that views it.

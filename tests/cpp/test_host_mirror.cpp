@@ -190,6 +190,28 @@ static void test_rms_norm(const Device &d) {  // rms_norm.rs:163-186 (values), n
     EXPECT(kc[0] == 2.0f && kc[3] == 8.0f && vc[0] == 5.0f && vc[3] == 8.0f, "norm fused into the cache append");
 }
 
+static void test_capture(const Device &d) {  // a recorded rope call replays on new contents of the same buffers
+    const float c0[4] = {1.0f, 1.0f, 0.0f, 0.0f}, s0[4] = {0.0f, 0.0f, 1.0f, 1.0f};  // position 0: identity, 1: +90 degrees
+    RopeCache rope(d, 2, 2, c0, s0);
+    auto x = t4(d, {1.0f, 2.0f, 3.0f, 4.0f, 1.0f, 2.0f, 3.0f, 4.0f}, 1, 1, 2, 4);
+    const uint32_t shape[4] = {1, 1, 2, 4};
+    auto y = Tensor<4>::empty(d, DType::F32, shape);
+    const fhip_rope_tables t = rope.tables(0, false);
+    const fhip_tensor4 cx = x.c4(), cy = y.c4();
+    Graph g = d.capture([&] { check(fhip_rope(d.stream(), &t, &cx, FHIP_F32, &cy, FHIP_F32)); });
+    g.launch();
+    auto h = host(y);
+    // row 0 unchanged; row 1: pairs (0,2), (1,3) turned by 90 degrees: (1,3) -> (-3,1), (2,4) -> (-4,2)
+    EXPECT(h[0] == 1.0f && h[3] == 4.0f && h[4] == -3.0f && h[5] == -4.0f && h[6] == 1.0f && h[7] == 2.0f,
+           "captured rope: %g %g %g %g | %g %g %g %g", h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]);
+    const float nx[8] = {5.0f, 6.0f, 7.0f, 8.0f, 5.0f, 6.0f, 7.0f, 8.0f};
+    check(fhip_memcpy_h2d(d.stream(), cx.ptr, nx, sizeof(nx)));
+    g.launch();
+    h = host(y);
+    EXPECT(h[0] == 5.0f && h[4] == -7.0f && h[5] == -8.0f && h[6] == 5.0f && h[7] == 6.0f, "replay on new contents: %g %g %g %g",
+           h[4], h[5], h[6], h[7]);
+}
+
 int main() {
     try {
         Device d(0);
@@ -202,6 +224,7 @@ int main() {
         test_kv_cache(d);
         test_rope(d);
         test_rms_norm(d);
+        test_capture(d);
     } catch (const std::exception &e) {
         printf("exception: %s\n", e.what());
         return 2;
