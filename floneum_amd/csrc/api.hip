@@ -206,12 +206,14 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     return true;
 }
 
+// The tiled kernel that computes in f32 on the f32 matrix cores.  It is THE prefill kernel for f32 tensors and the
+// second choice for 16-bit ones (rows widened on load): head dims and mask tensors their own kernel does not take.
 static bool prefill_f32_eligible(const fhip_attn_args *a) {
-    if (a->dtype != FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
     if (D % 4 != 0 || D > 256) return false;  // rows are padded with zeros to the tile width on the way into LDS
     if (!(a->scale > 0.0f)) return false;
-    if (!rows_vectorizable(a->q, 4) || !rows_vectorizable(a->k, 4) || !rows_vectorizable(a->v, 4)) return false;
+    const int eb = elem_bytes(a->dtype);
+    if (!rows_vectorizable(a->q, eb) || !rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;
     return true;
 }
 
@@ -668,14 +670,14 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
     if (id == FHIP_KERNEL_PREFILL_F32 && args->mask_kind != FHIP_MASK_NONE && !mask_scratch_ok(args, false)) {
         // no scratch for the interval form: the f32 kernel adds the mask tensor element by element
-        rc = launch_prefill_f32(p, s->s);
+        rc = launch_prefill_f32(p, args->dtype, s->s);
         if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
         return rc;
     }
     if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
         // dense mask: reduce it to one visible interval per row on the device; the tiled kernel skips the
         // masked tiles if every row is of that form.  If not, the kernel queued right behind it takes the
-        // call: the f32 kernel's mask-adding form, or the general kernel for 16-bit tensors.
+        // call: the f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
         rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
@@ -683,18 +685,18 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         AttnParams pt = p;
         pt.iv = iv;
         pt.iv_bad = bad;
-        rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, s->s);
+        rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, args->dtype, s->s);
         if (rc) return rc;
         if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
         AttnParams pg = p;
         pg.only_if_bad = bad;
-        return id == FHIP_KERNEL_PREFILL_F32 && f32_adds_masks(args) ? launch_prefill_f32(pg, s->s)
-                                                                    : launch_generic(pg, args->dtype, s->s);
+        return prefill_f32_eligible(args) && f32_adds_masks(args) ? launch_prefill_f32(pg, args->dtype, s->s)
+                                                                  : launch_generic(pg, args->dtype, s->s);
     }
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
-        case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, s->s); break;
+        case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
             decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr, args->dtype == FHIP_F32, &p.chunk, &p.nsplit);
             const size_t need = decode_workspace_bytes(p.B, p.H, p.Hkv, p.D, p.nsplit);

@@ -29,6 +29,24 @@ constexpr int PF32_WAVES = 4;
 constexpr int PF32_BN = 32;
 constexpr float PF32_LOG2E = 1.4426950408889634f;
 
+// four consecutive elements of a row as f32 (16-bit storage types are widened exactly)
+__device__ __forceinline__ float4_t load4(const float *p) { return *(const float4_t *)p; }
+__device__ __forceinline__ float4_t load4(const half_t *p) {
+    const half4_t h = *(const half4_t *)p;
+    return float4_t{(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
+}
+__device__ __forceinline__ float4_t load4(const bf16_t *p) {
+    const uint2_t u = *(const uint2_t *)p;
+    return float4_t{__uint_as_float(u[0] << 16), __uint_as_float(u[0] & 0xffff0000u), __uint_as_float(u[1] << 16),
+                    __uint_as_float(u[1] & 0xffff0000u)};
+}
+// one output element: the tensors' type, or f32 when the call asks for an f32 result of 16-bit inputs
+template <typename T>
+__device__ __forceinline__ void store_out(const AttnParams &p, int64_t idx, float v) {
+    if (sizeof(T) == 4 || p.out_f32) ((float *)p.out)[idx] = v;
+    else ((T *)p.out)[idx] = from_float<T>(v);
+}
+
 #define LDS32_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
 
 __device__ __forceinline__ float half_swap_max32(float x) {
@@ -43,7 +61,7 @@ __device__ __forceinline__ float half_swap_sum32(float x) {
 // BIAS: the additive mask tensor is applied as it is, element by element (p.mask, no interval form): finite
 // biases, several visible runs per row, NaN or +inf entries.  Score = (q.k * scale) + mask as in the reference
 // (fusor flash_attention.rs:145,177), every key tile is visited.
-template <int D, int S, bool BIAS>
+template <typename T, int D, int S, bool BIAS>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnParams p, int nqb) {
     constexpr int WPG = PF32_WAVES / S;   // wavefronts per key-split group
     constexpr int BM = 32 * WPG;          // query rows per workgroup
@@ -91,13 +109,13 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     float4_t qreg[D / 8];
     {
         const int qrow = min(query, p.Sq - 1);
-        const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
+        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
         for (int kc = 0; kc < D / 8; kc++)
-            qreg[kc] = 8 * kc + 4 * h2 < p.D ? *(const float4_t *)(qp + 8 * kc + 4 * h2) : float4_t{0.f, 0.f, 0.f, 0.f};
+            qreg[kc] = 8 * kc + 4 * h2 < p.D ? load4(qp + 8 * kc + 4 * h2) : float4_t{0.f, 0.f, 0.f, 0.f};
     }
-    const float *kg = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
-    const float *vg = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
+    const T *kg = (const T *)p.k + b * p.ks[0] + g * p.ks[1];
+    const T *vg = (const T *)p.v + b * p.vs[0] + g * p.vs[1];
 
     float16_t o[D / 32];
 #pragma unroll
@@ -108,9 +126,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     // scores reach the softmax in the base-2 domain: raw dot products times scale * log2(e); with BIAS they are
     // scaled, biased, and then only multiplied by log2(e)
     const float scale2 = BIAS ? PF32_LOG2E : p.scale * PF32_LOG2E;
-    const float *mrow = nullptr;
+    const T *mrow = nullptr;
     if constexpr (BIAS)
-        mrow = (const float *)p.mask + (int64_t)(p.mask_kind == FHIP_MASK_QK ? min(query, p.Sq - 1) : b) * p.ms0;
+        mrow = (const T *)p.mask + (int64_t)(p.mask_kind == FHIP_MASK_QK ? min(query, p.Sq - 1) : b) * p.ms0;
 
     float4_t kst[NCH], vst[NCH];
     auto load_tile = [&](int j0) {
@@ -120,8 +138,8 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             const int row = cid / CPR, col = cid % CPR;
             const int key = min(j0 + row, p.Skv - 1);
             const bool in_row = col * 4 < p.D;  // a head_dim below D is padded with zeros
-            kst[i] = in_row ? *(const float4_t *)(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
-            vst[i] = in_row ? *(const float4_t *)(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            kst[i] = in_row ? load4(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            vst[i] = in_row ? load4(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     };
     auto store_tile = [&]() {
@@ -158,7 +176,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                bias[r] = key < p.Skv ? mrow[(int64_t)key * p.ms1] : 0.0f;
+                bias[r] = key < p.Skv ? to_float(mrow[(int64_t)key * p.ms1]) : 0.0f;
             }
         }
 
@@ -255,13 +273,13 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     }
     const float l_tot = half_swap_sum32(l);
     if (query < p.Sq) {
-        float *op = (float *)p.out + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
+        const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                if (dim < p.D) op[dim * p.os[3]] = o[db][r] / l_tot;  // no visible key: 0/0 = NaN like the reference
+                if (dim < p.D) store_out<T>(p, ob + dim * p.os[3], o[db][r] / l_tot);  // no visible key: 0/0 = NaN like the reference
             }
     }
 }
@@ -274,6 +292,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 // Workgroup = 2 pairs = 64 query rows; K, V tiles of 32 keys x 256 dims (zero-padded above head_dim).
 constexpr int PFW_DP = 256, PFW_DH = 128;
 
+template <typename T>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(AttnParams p, int nqb) {
     constexpr int BM = 64;
     constexpr int KP = PFW_DP * 4 + 16;
@@ -313,15 +332,15 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     float4_t qreg[PFW_DH / 8];
     {
         const int qrow = min(query, p.Sq - 1);
-        const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
+        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
 #pragma unroll
         for (int kc = 0; kc < PFW_DH / 8; kc++) {
             const int dim = d0 + 8 * kc + 4 * h2;
-            qreg[kc] = dim < p.D ? *(const float4_t *)(qp + dim) : float4_t{0.f, 0.f, 0.f, 0.f};
+            qreg[kc] = dim < p.D ? load4(qp + dim) : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     }
-    const float *kg = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
-    const float *vg = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
+    const T *kg = (const T *)p.k + b * p.ks[0] + g * p.ks[1];
+    const T *vg = (const T *)p.v + b * p.vs[0] + g * p.vs[1];
 
     float16_t o[PFW_DH / 32];
 #pragma unroll
@@ -334,14 +353,13 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     // K and V take turns in one set of staging registers: V(j) is in flight while K(j) is multiplied, K(j+1)
     // while V(j) is
     float4_t st[NCH];
-    auto load_rows = [&](const float *base, const int64_t row_stride, int j0) {
+    auto load_rows = [&](const T *base, const int64_t row_stride, int j0) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int cid = tid + 64 * PF32_WAVES * i;
             const int row = cid / CPR, col = cid % CPR;
             const int key = min(j0 + row, p.Skv - 1);
-            st[i] = col * 4 < p.D ? *(const float4_t *)(base + (int64_t)key * row_stride + col * 4)
-                                  : float4_t{0.f, 0.f, 0.f, 0.f};
+            st[i] = col * 4 < p.D ? load4(base + (int64_t)key * row_stride + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     };
     auto store_rows = [&](int lds_off) {
@@ -436,17 +454,18 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
 
     const float l_tot = half_swap_sum32(l);
     if (query < p.Sq) {
-        float *op = (float *)p.out + b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
+        const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
         for (int db = 0; db < PFW_DH / 32; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int dim = d0 + 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                if (dim < p.D) op[dim * p.os[3]] = o[db][r] / l_tot;  // no visible key: 0/0 = NaN like the reference
+                if (dim < p.D) store_out<T>(p, ob + dim * p.os[3], o[db][r] / l_tot);  // no visible key: 0/0 = NaN like the reference
             }
     }
 }
 
+template <typename T>
 static int launch_wide(const AttnParams &p, hipStream_t stream) {
     if (p.mask && !p.iv) {
         set_error("prefill f32: a mask tensor without its interval form is not supported above head_dim 128");
@@ -458,12 +477,12 @@ static int launch_wide(const AttnParams &p, hipStream_t stream) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(prefill_f32_wide_kernel, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), 0, stream, p, nqb);
+    hipLaunchKernelGGL(prefill_f32_wide_kernel<T>, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), 0, stream, p, nqb);
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
 }
 
-template <int S, bool BIAS>
+template <typename T, int S, bool BIAS>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
     constexpr int BM = 32 * (PF32_WAVES / S);
     const int nqb = (p.Sq + BM - 1) / BM;
@@ -474,13 +493,13 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
     switch ((p.D + 31) / 32 * 32) {  // the kernel's D is head_dim rounded up to a multiple of 32
-        case 32: hipLaunchKernelGGL((prefill_f32_kernel<32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
-        case 64: hipLaunchKernelGGL((prefill_f32_kernel<64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
+        case 32: hipLaunchKernelGGL((prefill_f32_kernel<T, 32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
+        case 64: hipLaunchKernelGGL((prefill_f32_kernel<T, 64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 96:
-            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<96, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         case 128:
-            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<128, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
@@ -488,8 +507,10 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
     return FHIP_OK;
 }
 
-int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
-    if (p.D > 128) return launch_wide(p, stream);
+// 16-bit tensors are served by the unsplit forms only (their own matrix-core kernel takes the common shapes)
+template <typename T>
+static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
+    if (p.D > 128) return launch_wide<T>(p, stream);
     // Split the keys of a query block over 2 or 4 wavefront groups while the unsplit grid is only a few
     // workgroups per CU: the longest (last causal) query block then sets the run time, and halving it pays
     // even when every CU has work.  Measured break-even: about 4 workgroups per CU at head_dim <= 64, 2 above
@@ -502,17 +523,28 @@ int launch_prefill_f32(const AttnParams &p, hipStream_t stream) {
     int split = 1;
     if (wg1 <= (small_dim ? 4L : 2L) * cus) split = 2;
     if (split == 2 && small_dim && wg2 < 2L * cus) split = 4;
+    if (sizeof(T) != 4) split = 1;
     // a mask tensor without its interval form is added element by element (the 16 bias registers leave no
     // room for the key-split form at head_dim 96 / 128)
     if (p.mask && !p.iv) {
         if (!small_dim) split = 1;
-        if (split == 4) return launch_split<4, true>(p, stream);
-        if (split == 2) return launch_split<2, true>(p, stream);
-        return launch_split<1, true>(p, stream);
+        if constexpr (sizeof(T) == 4) {
+            if (split == 4) return launch_split<T, 4, true>(p, stream);
+            if (split == 2) return launch_split<T, 2, true>(p, stream);
+        }
+        return launch_split<T, 1, true>(p, stream);
     }
-    if (split == 4) return launch_split<4, false>(p, stream);
-    if (split == 2) return launch_split<2, false>(p, stream);
-    return launch_split<1, false>(p, stream);
+    if constexpr (sizeof(T) == 4) {
+        if (split == 4) return launch_split<T, 4, false>(p, stream);
+        if (split == 2) return launch_split<T, 2, false>(p, stream);
+    }
+    return launch_split<T, 1, false>(p, stream);
+}
+
+int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
+    if (dtype == FHIP_F16) return launch_prefill_f32_t<half_t>(p, stream);
+    if (dtype == FHIP_BF16) return launch_prefill_f32_t<bf16_t>(p, stream);
+    return launch_prefill_f32_t<float>(p, stream);
 }
 
 }  // namespace fhip

@@ -60,7 +60,8 @@ int hip_fail(hipError_t e, const char *what);
 int launch_generic(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 int launch_decode(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
-int launch_prefill_f32(const AttnParams &p, hipStream_t stream);
+// f32 arithmetic on the f32 matrix cores; `dtype` is the tensors' storage type (16-bit rows are widened on load)
+int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 
 // decode planning (host): keys per split and number of splits; `ragged`: per-batch key counts are given;
 // `f32`: the tensors are f32 (vector variant) rather than 16-bit

@@ -129,9 +129,12 @@ typedef enum {
     FHIP_KERNEL_GENERIC = 1,     /* any dtype, any strides, any mask; one wavefront per query row   */
     FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim in {64,96,128}, LDS-tiled MFMA; masks by
                                     interval (analytic, kv_lens, or a mask tensor reduced on the device) */
-    FHIP_KERNEL_PREFILL_F32 = 3, /* f32, head_dim multiple of 32 up to 128, f32 MFMA                */
-    FHIP_KERNEL_DECODE_SPLITKV = 4 /* Sq == 1, split-KV streaming + LSE combine (matrix cores for
-                                      f16/bf16, vector units for f32)                                */
+    FHIP_KERNEL_PREFILL_F32 = 3, /* f32 arithmetic on the f32 MFMA, LDS-tiled: f32 tensors, and 16-bit tensors
+                                    (widened on load) the kernel above does not take; head_dim multiple of
+                                    4 up to 256; masks by interval or, up to head_dim 128, added as they are */
+    FHIP_KERNEL_DECODE_SPLITKV = 4 /* Sq == 1, head_dim multiple of 8 up to 256: split-KV streaming + LSE
+                                      combine (matrix cores for f16/bf16 at head_dim 32/64/96/128, vector
+                                      units otherwise)                                                 */
 } fhip_kernel_id;
 
 
@@ -198,8 +201,9 @@ int fhip_flash_attention_validate(const fhip_attn_args *args);
 /* Which kernel fhip_flash_attention will run for these arguments (host-only).  For a prefill call
  * with a mask tensor and a sufficient workspace in `args` this names the tiled kernel, which runs if
  * the mask turns out to be made of intervals (decided on the device) and otherwise hands over, inside
- * the same call, to the kernel that adds the mask values one by one (the f32 tiled kernel's own
- * mask-adding form, the general kernel for 16-bit tensors); without the workspace it names that kernel. */
+ * the same call, to the kernel that adds the mask values one by one (the mask-adding form of the
+ * f32-arithmetic tiled kernel up to head_dim 128, the general kernel above); without the workspace it
+ * names that kernel. */
 int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id);
 
 /* Bytes of device workspace the call needs (0 for the single-pass kernels).  `compute_units`

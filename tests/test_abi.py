@@ -151,13 +151,24 @@ def test_kernel_selection():
     # f32 decode (kalosm-llama's cache is f32, attention_layer.rs:400-403) streams through the split-KV kernel too
     assert selected(make_args(Sq=1, Skv=4096, D=128, dtype=fa.F32))[1] == fa.KERNEL_DECODE_SPLITKV
     assert selected(make_args(Sq=7, Skv=9, D=33))[1] == fa.KERNEL_GENERIC
-    # a dense additive mask without the scratch its interval form needs goes to the general kernel
+    # a dense additive mask without the scratch its interval form needs: the f32-arithmetic tiled kernel adds the mask
+    # element by element (16-bit rows are widened on load), up to head_dim 128; beyond that the general kernel
     a = make_args(Sq=64, Skv=64, D=128)
     a.mask_kind = fa.MaskKind.QKMask
     a.mask.ptr = FAKE
     a.mask.shape[:] = [64, 64]
     a.mask.stride[:] = [64, 1]
+    assert selected(a)[1] == fa.KERNEL_PREFILL_F32
+    a = make_args(Sq=64, Skv=64, D=256)
+    a.mask_kind = fa.MaskKind.QKMask
+    a.mask.ptr = FAKE
+    a.mask.shape[:] = [64, 64]
+    a.mask.stride[:] = [64, 1]
     assert selected(a)[1] == fa.KERNEL_GENERIC
+    # 16-bit head dims their own matrix-core kernel does not take run on the f32-arithmetic kernel
+    assert selected(make_args(Sq=64, Skv=64, D=80))[1] == fa.KERNEL_PREFILL_F32
+    assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_F32
+    assert selected(make_args(Sq=64, Skv=64, D=264))[1] == fa.KERNEL_GENERIC
     # innermost stride != 1 or a misaligned base pointer -> generic
     a = make_args(Sq=64, Skv=64, D=128)
     a.k.stride[:] = [2 * 64 * 128, 1, 128 * 2, 64]

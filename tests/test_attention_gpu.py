@@ -284,6 +284,47 @@ def test_prefill_f32_wide_heads(device, D, case):
         assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == want
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("D,case", [(80, "causal"), (256, "causal"), (192, "window_offset"), (32, "full_ragged"), (40, "causal"),
+                                    (128, "bias"), (64, "bias"), (96, "bias_batch_key")])
+def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
+    """Head dims and mask tensors the 16-bit matrix-core kernel does not take run on the tiled kernel that computes
+    in f32: rows are widened on their way into LDS, the result is rounded to the tensors' type."""
+    B, H, Hkv = 2, 4, 2
+    Sq, Skv = {"causal": (150, 150), "window_offset": (97, 400), "full_ragged": (70, 333), "bias": (90, 200),
+               "bias_batch_key": (90, 200)}[case]
+    q, k, v = _normal_qkv(15, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    mask, kind, analytic, mt = None, None, None, None
+    if case == "causal":
+        analytic = (True, 0, 0)
+    elif case == "window_offset":
+        analytic = (True, Skv - Sq, 120)
+    elif case == "bias":
+        mask, kind = np.random.default_rng(3).normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
+        mask[:, 100:140] = NEG_INF
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "bias_batch_key":
+        mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+        mask[0, 150:] = -10000.0
+        mask[1, :20] = -10000.0
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.BatchKeyMask)
+    if analytic is not None:
+        mask, kind = _analytic_mask(Sq, Skv, *analytic), "qk"
+    if mt is None:
+        assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == fa.KERNEL_PREFILL_F32
+    out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 None if mask is None else rounded(mask, dtype), kind)
+    tol = dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16
+    assert_parity(out, ref, tol, f"16-bit on the f32 kernel, D{D} {case}")
+    # and with an f32 result the only rounding left is the inputs'
+    if mt is None:
+        out32 = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out_dtype=fa.F32).to_numpy()
+        assert out32.dtype == np.float32
+        assert_parity(out32, ref, TOL_F32, f"f32 result, D{D} {case}")
+
+
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),

@@ -104,8 +104,8 @@ def test_block_diagonal_mask_of_the_vision_blocks(device, dtype, D):
 @pytest.mark.parametrize("shape", ["bias", "two_runs", "nan", "positive_inf"])
 def test_masks_that_are_not_intervals_fall_back(device, dtype, D, shape):
     """Finite biases, several visible runs, NaN or +inf entries: the mask values are added as the reference adds
-    them (fusor flash_attention.rs:161-176), by the f32 kernel's mask-adding form or, for 16-bit tensors, the
-    general kernel."""
+    them (fusor flash_attention.rs:161-176), by the mask-adding form of the f32-arithmetic tiled kernel (which widens
+    16-bit rows on load)."""
     B, H, Hkv, Sq, Skv = 1, 2, 1, 140, 200
     q, k, v = _normal_qkv(23, B, H, Hkv, Sq, Skv, D)
     rng = np.random.default_rng(5)
@@ -165,13 +165,14 @@ def test_strided_and_broadcast_mask_views(device):
     assert_parity(out, ref, TOL_16, "transposed mask view")
 
 
-def test_without_workspace_the_general_kernel_runs(device):
-    """The C ABI never allocates: a masked call that brings no scratch is served by the general kernel."""
+def test_without_workspace_the_mask_is_added_element_by_element(device):
+    """The C ABI never allocates: a masked call that brings no scratch is served by the f32-arithmetic tiled kernel,
+    which adds the mask as it is (16-bit rows are widened on load)."""
     D, S = 64, 100
     q, k, v = _normal_qkv(26, 1, 2, 1, S, S, D)
     mask = oracle.get_mask(S, 0)
     tq, tk, tv, tm = _tensors(device, fa.F16, q, k, v, mask)
-    assert tq.selected_kernel(tk, tv, 0.1, (tm, fa.MaskKind.QKMask)) == fa.KERNEL_GENERIC
+    assert tq.selected_kernel(tk, tv, 0.1, (tm, fa.MaskKind.QKMask)) == fa.KERNEL_PREFILL_F32
     out_t = fa.Tensor.empty(device, (1, 2, S, D), fa.F16)
     args = tq._attn_args(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask), None, None, None, fa.KERNEL_AUTO, out_t)
     fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
