@@ -47,6 +47,15 @@ __device__ __forceinline__ void store_out(const AttnParams &p, int64_t idx, floa
     else ((T *)p.out)[idx] = from_float<T>(v);
 }
 
+// odd rounds of `cus` workgroups are numbered backwards (see AttnParams::snake_cus)
+__device__ __forceinline__ int snake_order(int id, int total, int cus) {
+    if (cus <= 0) return id;
+    const int r = id / cus, j = id % cus;
+    if ((r & 1) == 0) return id;
+    const int len = min(cus, total - r * cus);
+    return r * cus + (len - 1 - j);
+}
+
 #define LDS32_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
 
 __device__ __forceinline__ float half_swap_max32(float x) {
@@ -90,7 +99,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int gbase = grp * 2 * K_BYTES;  // the group's tile buffers
 
     const int bh_count = p.B * p.H;
-    const int id = blockIdx.x;
+    const int id = snake_order(blockIdx.x, gridDim.x, p.snake_cus);
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
     const int b = rem / p.H;
@@ -314,7 +323,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     const int d0 = PFW_DH * hf;
 
     const int bh_count = p.B * p.H;
-    const int id = blockIdx.x;
+    const int id = snake_order(blockIdx.x, gridDim.x, p.snake_cus);
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
     const int b = rem / p.H;
@@ -526,19 +535,25 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
     if (sizeof(T) != 4) split = 1;
     // a mask tensor without its interval form is added element by element (the 16 bias registers leave no
     // room for the key-split form at head_dim 96 / 128)
-    if (p.mask && !p.iv) {
-        if (!small_dim) split = 1;
+    const bool add_mask = p.mask && !p.iv;
+    if (add_mask && !small_dim) split = 1;
+    AttnParams ps = p;
+    {
+        const long blocks = bh * ((p.Sq + 128 / split - 1) / (128 / split));
+        ps.snake_cus = (blocks > cus && blocks <= 2L * cus) ? cus : 0;
+    }
+    if (add_mask) {
         if constexpr (sizeof(T) == 4) {
-            if (split == 4) return launch_split<T, 4, true>(p, stream);
-            if (split == 2) return launch_split<T, 2, true>(p, stream);
+            if (split == 4) return launch_split<T, 4, true>(ps, stream);
+            if (split == 2) return launch_split<T, 2, true>(ps, stream);
         }
-        return launch_split<T, 1, true>(p, stream);
+        return launch_split<T, 1, true>(ps, stream);
     }
     if constexpr (sizeof(T) == 4) {
-        if (split == 4) return launch_split<T, 4, false>(p, stream);
-        if (split == 2) return launch_split<T, 2, false>(p, stream);
+        if (split == 4) return launch_split<T, 4, false>(ps, stream);
+        if (split == 2) return launch_split<T, 2, false>(ps, stream);
     }
-    return launch_split<T, 1, false>(p, stream);
+    return launch_split<T, 1, false>(ps, stream);
 }
 
 int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {

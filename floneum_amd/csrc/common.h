@@ -35,6 +35,10 @@ struct AttnParams {
     const int2 *iv;
     const int32_t *iv_bad;
     const int32_t *only_if_bad;
+    // Tiled f32 prefill only.  Workgroups are numbered longest first.  When the whole grid is resident at once
+    // (two workgroups per CU) nothing is rebalanced at run time, so the second half of the numbers is walked
+    // backwards: a CU's two workgroups are then a long and a short one.  0: off; else the number of CUs.
+    int32_t snake_cus;
 };
 
 // bytes of device scratch the interval form of a dense mask needs
