@@ -496,3 +496,28 @@ def test_tensors_without_elements(device, dtype):
     with pytest.raises(AssertionError, match="divisible"):
         tq.flash_attention(fa.Tensor.from_numpy(device, np.zeros((2, 0, 3, D), np.float32), dtype),
                            fa.Tensor.from_numpy(device, np.zeros((2, 0, 3, D), np.float32), dtype), 0.125)
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 128), (fa.F32, 64)])
+def test_decode_over_a_very_long_cache(device, dtype, D):
+    """Half a million keys for one sequence: hundreds of splits, 64-bit row offsets, several rounds in the merge."""
+    Skv = 500_003
+    q, k, v = _normal_qkv(16, 1, 2, 1, 1, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
+    # Half a million f32 terms summed left to right (the reference's fold) carry more rounding error than the 1e-5
+    # the benchmark sizes are held to, so the referee here is the float64 definition: the device result must be at
+    # least as close to it as the f32 restatement is, and within the usual bound
+    qr, kr, vr = rounded(q, dtype), rounded(k, dtype), rounded(v, dtype)
+    exact = oracle.flash_attention_f64(qr, kr, vr, D ** -0.5)
+    restated = oracle.flash_attention(qr, kr, vr, D ** -0.5)
+    from conftest import rel_l2
+    err_dev, err_restated = rel_l2(out, exact), rel_l2(restated, exact)
+    bound = 1e-5 if dtype == fa.F32 else 1e-3
+    assert err_dev <= max(bound, 1.5 * err_restated), (err_dev, err_restated)
+    assert not np.isnan(out).any()
+    # the last position only (a sliding window of one key) must return that key's value row
+    out1 = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, Skv - 1, 1)).to_numpy()
+    want = rounded(v, dtype)[:, :1, Skv - 1:Skv].repeat(2, axis=1)
+    assert_parity(out1, want, dict(max_abs=1e-6, rel_l2=1e-6) if dtype == fa.F32 else TOL_16, "window of one key at the end")
