@@ -231,6 +231,15 @@ static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
 // The f32 tiled kernel can add a mask tensor element by element (no scratch, no interval form) up to head_dim 128.
 static bool f32_adds_masks(const fhip_attn_args *a) { return a->q.shape[3] <= 128; }
 
+// Key split of a call the f32-arithmetic tiled kernel serves (few query rows on a long cache), and where its
+// partial results go in the workspace: behind the mask scratch, 256-byte aligned.
+static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
+    const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
+    prefill_f32_plan((int)a->q.shape[0], (int)a->q.shape[1], (int)a->q.shape[2], (int)a->k.shape[2], (int)a->q.shape[3],
+                     causal_square, cus > 0 ? cus : 256, nsplit, chunk);
+}
+static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratch_bytes(a) + 255) & ~(size_t)255; }
+
 // assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
 // (the size query); otherwise a masked call without enough scratch takes the general kernel.
 static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_workspace = false) {
@@ -635,6 +644,13 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     if (rc) return rc;
     if (output_is_empty(args) || no_keys(args)) return FHIP_OK;
     if (id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) *bytes = mask_scratch_bytes(args);
+    if (id == FHIP_KERNEL_PREFILL_F32) {
+        int ns, chunk;
+        f32_split_plan(args, compute_units, &ns, &chunk);
+        const size_t part = prefill_f32_workspace_bytes((int)args->q.shape[0], (int)args->q.shape[1], (int)args->q.shape[2],
+                                                        (int)args->q.shape[3], ns);
+        if (part) *bytes = f32_partials_offset(args) + part;
+    }
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
         int chunk, nsplit;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
@@ -668,6 +684,18 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     AttnParams p;
     fill_params(args, &p);
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    if (id == FHIP_KERNEL_PREFILL_F32) {
+        // few query rows on a long cache: split the keys over workgroups if the caller brought the scratch for it
+        int ns, chunk;
+        f32_split_plan(args, s->dev->prop.multiProcessorCount, &ns, &chunk);
+        const size_t off = f32_partials_offset(args);
+        const size_t part = prefill_f32_workspace_bytes(p.B, p.H, p.Sq, p.D, ns);
+        if (part && args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes >= off + part) {
+            p.pf_nsplit = ns;
+            p.pf_chunk = chunk;
+            p.partials = (float *)((char *)args->workspace + off);
+        }
+    }
     if (id == FHIP_KERNEL_PREFILL_F32 && args->mask_kind != FHIP_MASK_NONE && !mask_scratch_ok(args, false)) {
         // no scratch for the interval form: the f32 kernel adds the mask tensor element by element
         rc = launch_prefill_f32(p, args->dtype, s->s);

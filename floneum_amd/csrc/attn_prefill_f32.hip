@@ -99,7 +99,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int gbase = grp * 2 * K_BYTES;  // the group's tile buffers
 
     const int bh_count = p.B * p.H;
-    const int id = snake_order(blockIdx.x, gridDim.x, p.snake_cus);
+    const int nks = max(p.pf_nsplit, 1);
+    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
+    const int id = snake_order(blockIdx.x / nks, gridDim.x / nks, p.snake_cus);
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
     const int b = rem / p.H;
@@ -110,7 +112,14 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int q0 = qb * BM;
     const int qw0 = q0 + 32 * wig;
     const int query = qw0 + ln;
-    const RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    if (nks > 1) {  // this workgroup's share of the keys
+        const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
+        rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
+        rb.lo_w = max(rb.lo_w, c_lo), rb.hi_w = min(rb.hi_w, c_hi);
+        rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
+        rb.klo = max(rb.klo, c_lo), rb.khi = min(rb.khi, c_hi);
+    }
     const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const bool wave_has_rows = qw0 < p.Sq;
 
@@ -281,6 +290,24 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         }
     }
     const float l_tot = half_swap_sum32(l);
+    if (nks > 1) {
+        // park this share's state; the merge kernel normalises
+        if (query < p.Sq) {
+            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * (p.D + 2);
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                    if (dim < p.D) ws[dim] = o[db][r];
+                }
+            if (h2 == 0) {
+                ws[p.D] = m;
+                ws[p.D + 1] = l_tot;
+            }
+        }
+        return;
+    }
     if (query < p.Sq) {
         const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
@@ -291,6 +318,36 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
                 if (dim < p.D) store_out<T>(p, ob + dim * p.os[3], o[db][r] / l_tot);  // no visible key: 0/0 = NaN like the reference
             }
     }
+}
+
+// Merge of the key shares: one wavefront per (batch, head, query row), log-sum-exp over the shares (the state is
+// in the base-2 domain), then the division the single-pass form does in its epilogue.
+template <typename T>
+__global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    if (row >= rows) return;
+    // the same hand-over between the interval form and the mask-adding form as in the main kernel
+    if ((p.iv_bad && *p.iv_bad != 0) || (p.only_if_bad && *p.only_if_bad == 0)) return;
+    const int query = (int)(row % p.Sq);
+    const int h = (int)((row / p.Sq) % p.H), b = (int)(row / p.Sq / p.H);
+    const int D = p.D, ns = p.pf_nsplit;
+    const float *ws = p.partials + row * ns * (D + 2);
+    float M = -INFINITY;
+    for (int sp = 0; sp < ns; sp++) M = fmaxf(M, ws[sp * (D + 2) + D]);
+    const float Ms = (M == -INFINITY) ? 0.0f : M;
+    float L = 0.0f, A0 = 0.0f, A1 = 0.0f;
+    for (int sp = 0; sp < ns; sp++) {
+        const float *src = ws + sp * (D + 2);
+        const float w = __builtin_amdgcn_exp2f(src[D] - Ms);
+        L += w * src[D + 1];
+        if (lane < D) A0 += w * src[lane];
+        if (lane + 64 < D) A1 += w * src[lane + 64];
+    }
+    const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
+    if (lane < D) store_out<T>(p, ob + lane * p.os[3], A0 / L);  // no visible key: 0/0 = NaN like the reference
+    if (lane + 64 < D) store_out<T>(p, ob + (lane + 64) * p.os[3], A1 / L);
 }
 
 // ---- head_dim 129 .. 256 (Gemma-3's key length is 256) -------------------------------------------------------
@@ -495,7 +552,7 @@ template <typename T, int S, bool BIAS>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
     constexpr int BM = 32 * (PF32_WAVES / S);
     const int nqb = (p.Sq + BM - 1) / BM;
-    const long blocks = (long)nqb * p.B * p.H;
+    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -513,7 +570,36 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
+    if (p.pf_nsplit > 1) {
+        const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+        hipLaunchKernelGGL(prefill_f32_merge_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+        FHIP_HIP_CHECK(hipGetLastError());
+    }
     return FHIP_OK;
+}
+
+// Few query rows on a long cache (a new chat turn, a prompt fed in pieces): the grid of query blocks alone leaves
+// most CUs idle, so the keys are split over workgroups as well, down to 512 keys per share, until there are about
+// two workgroups per CU.  Square causal calls are left alone (their shares would be uneven, and they fill the
+// chip from 1024 rows on).
+void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+    *nsplit = 1;
+    *chunk = Skv;
+    if (D > 128 || causal_square) return;
+    const long wgs = (long)B * H * ((Sq + 31) / 32);  // at the finest query blocking the kernel has
+    const long want = (2L * compute_units + wgs - 1) / wgs;
+    const long most = Skv / 512;
+    long ns = want < most ? want : most;
+    if (ns < 2) return;
+    long c = (Skv + ns - 1) / ns;
+    c = (c + 31) / 32 * 32;
+    *chunk = (int)c;
+    *nsplit = (int)((Skv + c - 1) / c);
+}
+
+size_t prefill_f32_workspace_bytes(int B, int H, int Sq, int D, int nsplit) {
+    if (nsplit <= 1) return 0;
+    return (size_t)B * H * Sq * nsplit * (size_t)(D + 2) * sizeof(float);
 }
 
 // 16-bit tensors are served by the unsplit forms only (their own matrix-core kernel takes the common shapes)
@@ -526,7 +612,7 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
     // (the bigger tiles leave less to gain).  A single wavefront moves a whole tile only up to head_dim 64.
     int cus = 256, dev = 0;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    const long bh = (long)p.B * p.H;
+    const long bh = (long)p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     const long wg1 = bh * ((p.Sq + 127) / 128), wg2 = bh * ((p.Sq + 63) / 64);
     const bool small_dim = p.D <= 64;
     int split = 1;

@@ -39,7 +39,15 @@ struct AttnParams {
     // (two workgroups per CU) nothing is rebalanced at run time, so the second half of the numbers is walked
     // backwards: a CU's two workgroups are then a long and a short one.  0: off; else the number of CUs.
     int32_t snake_cus;
+    // Tiled f32 prefill only: keys split over pf_nsplit workgroups per query block (few query rows on a long
+    // cache would otherwise occupy a fraction of the chip).  Split s takes keys [s * pf_chunk, (s + 1) * pf_chunk)
+    // and parks (O unnormalised, m, l) per row in `partials` [B, H, Sq, pf_nsplit, D + 2]; a merge kernel follows.
+    int32_t pf_nsplit, pf_chunk;
 };
+
+// the key split of a tiled f32 prefill call (1 = none) and the scratch it needs
+void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk);
+size_t prefill_f32_workspace_bytes(int B, int H, int Sq, int D, int nsplit);
 
 // bytes of device scratch the interval form of a dense mask needs
 size_t mask_intervals_bytes(int rows);

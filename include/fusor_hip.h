@@ -113,9 +113,10 @@ typedef struct {
                         results.  A prefill call with a mask TENSOR uses it to reduce the mask to one
                         visible interval per row on the device (every mask fusor builds, and every
                         padding mask, has that form) and then runs the tiled kernel; a mask that is
-                        not of that form, or a call that brings no workspace, is served by the general
-                        kernel, which adds the mask values like the reference.  Same results either
-                        way.                                                                          */
+                        not of that form, or a call that brings no workspace, is served by a kernel
+                        that adds the mask values like the reference.  A prefill call of few query rows
+                        on a long cache uses it to split the keys over workgroups; without it the call
+                        runs unsplit.  Same results either way.                                       */
     size_t workspace_bytes;
     int32_t force_kernel; /* 0 = choose; otherwise a fhip_kernel_id (testing / benchmarking)       */
     /* Optional profiling hook: when non-NULL the event is recorded on the stream right after the

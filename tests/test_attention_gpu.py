@@ -5,6 +5,8 @@ fusor-ml/fusor/src/composite/flash_attention.rs:207-359 and the fuzz tests of
 fusor-ml/core/src/composite/flash_attention.rs:559-1060 (same shape ranges, seeded here), then the
 benchmark configurations at reduced and full size.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -521,3 +523,46 @@ def test_decode_over_a_very_long_cache(device, dtype, D):
     out1 = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, Skv - 1, 1)).to_numpy()
     want = rounded(v, dtype)[:, :1, Skv - 1:Skv].repeat(2, axis=1)
     assert_parity(out1, want, dict(max_abs=1e-6, rel_l2=1e-6) if dtype == fa.F32 else TOL_16, "window of one key at the end")
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 128), (fa.F32, 64), (fa.F32, 80), (fa.F16, 80), (fa.BF16, 40)])
+@pytest.mark.parametrize("case", ["causal_offset", "window", "mask_tensor", "bias_tensor", "kv_lens", "full"])
+def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
+    """A new chat turn on a long cached context: few query blocks, thousands of keys.  The f32-arithmetic tiled
+    kernel then splits the keys over workgroups and merges the shares; the result must not depend on it."""
+    B, H, Hkv, Sq, Skv = 1, 4, 2, 100, 5000
+    q, k, v = _normal_qkv(17, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    mask, kind, analytic, mt, lens_t = None, None, None, None, None
+    if case == "causal_offset":
+        analytic = (True, Skv - Sq, 0)
+    elif case == "window":
+        analytic = (True, Skv - Sq, 1500)
+    elif case == "mask_tensor":
+        mask, kind = oracle.get_mask(Sq, Skv - Sq), "qk"
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "bias_tensor":
+        mask, kind = np.random.default_rng(4).normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
+        mask[:, 700:2100] = NEG_INF
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "kv_lens":
+        lens_t = fa.IntTensor(device, np.array([3333], np.int32))
+        mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+        mask[0, 3333:] = NEG_INF
+    if analytic is not None:
+        mask, kind = _analytic_mask(Sq, Skv, *analytic), "qk"
+    # with the workspace the library asks for (the keys are split) ...
+    need = ctypes.c_size_t()
+    args = tq._attn_args(tk, tv, D ** -0.5, mt, analytic, lens_t, None, fa.KERNEL_AUTO, None)
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+    assert need.value > B * H * Sq * 2 * (D + 2) * 4, "the size query must ask for room for at least two shares"
+    out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic, kv_lens=lens_t).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 None if mask is None else rounded(mask, dtype), kind)
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+    assert_parity(out, ref, tol, f"split keys, {case} D{D}")
+    # ... and without any workspace (one workgroup walks all keys of its query block)
+    out_t = fa.Tensor.empty(device, (B, H, Sq, D), dtype)
+    args = tq._attn_args(tk, tv, D ** -0.5, mt, analytic, lens_t, None, fa.KERNEL_AUTO, out_t)
+    fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    assert_parity(out_t.to_numpy(), ref, tol, f"unsplit, {case} D{D}")
