@@ -239,6 +239,11 @@ static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *c
                      causal_square, cus > 0 ? cus : 256, nsplit, chunk);
 }
 static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratch_bytes(a) + 255) & ~(size_t)255; }
+static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
+    const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
+    prefill_mfma_plan((int)a->q.shape[0], (int)a->q.shape[1], (int)a->q.shape[2], (int)a->k.shape[2], causal_square,
+                      cus > 0 ? cus : 256, nsplit, chunk);
+}
 
 // assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
 // (the size query); otherwise a masked call without enough scratch takes the general kernel.
@@ -651,6 +656,13 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
                                                         (int)args->q.shape[3], ns);
         if (part) *bytes = f32_partials_offset(args) + part;
     }
+    if (id == FHIP_KERNEL_PREFILL_MFMA) {
+        int ns, chunk;
+        mfma_split_plan(args, compute_units, &ns, &chunk);
+        const size_t part = prefill_mfma_workspace_bytes((int)args->q.shape[0], (int)args->q.shape[1], (int)args->q.shape[2],
+                                                         (int)args->q.shape[3], ns);
+        if (part) *bytes = f32_partials_offset(args) + part;
+    }
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
         int chunk, nsplit;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
@@ -693,6 +705,19 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         if (part && args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes >= off + part) {
             p.pf_nsplit = ns;
             p.pf_chunk = chunk;
+            p.pf_pitch = p.D + 2;
+            p.partials = (float *)((char *)args->workspace + off);
+        }
+    }
+    if (id == FHIP_KERNEL_PREFILL_MFMA) {
+        int ns, chunk;
+        mfma_split_plan(args, s->dev->prop.multiProcessorCount, &ns, &chunk);
+        const size_t off = f32_partials_offset(args);
+        const size_t part = prefill_mfma_workspace_bytes(p.B, p.H, p.Sq, p.D, ns);
+        if (part && args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes >= off + part) {
+            p.pf_nsplit = ns;
+            p.pf_chunk = chunk;
+            p.pf_pitch = p.D + 4;  // rows of the partials are written in 16-byte pieces
             p.partials = (float *)((char *)args->workspace + off);
         }
     }
@@ -718,6 +743,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
         AttnParams pg = p;
         pg.only_if_bad = bad;
+        if (id == FHIP_KERNEL_PREFILL_MFMA) pg.pf_nsplit = 0;  // the split was planned for the other kernel's blocks
         return prefill_f32_eligible(args) && f32_adds_masks(args) ? launch_prefill_f32(pg, args->dtype, s->s)
                                                                   : launch_generic(pg, args->dtype, s->s);
     }

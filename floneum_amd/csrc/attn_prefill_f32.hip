@@ -293,7 +293,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     if (nks > 1) {
         // park this share's state; the merge kernel normalises
         if (query < p.Sq) {
-            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * (p.D + 2);
+            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * p.pf_pitch;
 #pragma unroll
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
@@ -332,14 +332,14 @@ __global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
     if ((p.iv_bad && *p.iv_bad != 0) || (p.only_if_bad && *p.only_if_bad == 0)) return;
     const int query = (int)(row % p.Sq);
     const int h = (int)((row / p.Sq) % p.H), b = (int)(row / p.Sq / p.H);
-    const int D = p.D, ns = p.pf_nsplit;
-    const float *ws = p.partials + row * ns * (D + 2);
+    const int D = p.D, ns = p.pf_nsplit, pitch = p.pf_pitch;
+    const float *ws = p.partials + row * ns * pitch;
     float M = -INFINITY;
-    for (int sp = 0; sp < ns; sp++) M = fmaxf(M, ws[sp * (D + 2) + D]);
+    for (int sp = 0; sp < ns; sp++) M = fmaxf(M, ws[sp * pitch + D]);
     const float Ms = (M == -INFINITY) ? 0.0f : M;
     float L = 0.0f, A0 = 0.0f, A1 = 0.0f;
     for (int sp = 0; sp < ns; sp++) {
-        const float *src = ws + sp * (D + 2);
+        const float *src = ws + sp * pitch;
         const float w = __builtin_amdgcn_exp2f(src[D] - Ms);
         L += w * src[D + 1];
         if (lane < D) A0 += w * src[lane];
@@ -548,6 +548,20 @@ static int launch_wide(const AttnParams &p, hipStream_t stream) {
     return FHIP_OK;
 }
 
+template <typename T>
+static int launch_merge_t(const AttnParams &p, hipStream_t stream) {
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    hipLaunchKernelGGL(prefill_f32_merge_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+int launch_prefill_merge(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
+    if (dtype == FHIP_F16) return launch_merge_t<half_t>(p, stream);
+    if (dtype == FHIP_BF16) return launch_merge_t<bf16_t>(p, stream);
+    return launch_merge_t<float>(p, stream);
+}
+
 template <typename T, int S, bool BIAS>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
     constexpr int BM = 32 * (PF32_WAVES / S);
@@ -570,11 +584,7 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
-    if (p.pf_nsplit > 1) {
-        const int64_t rows = (int64_t)p.B * p.H * p.Sq;
-        hipLaunchKernelGGL(prefill_f32_merge_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
-        FHIP_HIP_CHECK(hipGetLastError());
-    }
+    if (p.pf_nsplit > 1) return launch_merge_t<T>(p, stream);
     return FHIP_OK;
 }
 
@@ -587,6 +597,7 @@ void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, 
     *chunk = Skv;
     if (D > 128 || causal_square) return;
     const long wgs = (long)B * H * ((Sq + 31) / 32);  // at the finest query blocking the kernel has
+    if (wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy (two workgroups per CU)
     const long want = (2L * compute_units + wgs - 1) / wgs;
     const long most = Skv / 512;
     long ns = want < most ? want : most;

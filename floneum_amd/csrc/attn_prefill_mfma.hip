@@ -134,7 +134,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // workgroup -> (query block, batch, head): long query blocks first, and heads laid out so
     // the workgroups that land on one XCD (id % 8) share a KV head whenever H is a multiple of 8
     const int bh_count = p.B * p.H;
-    const int id = blockIdx.x;
+    const int nks = max(p.pf_nsplit, 1);
+    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
+    const int id = blockIdx.x / nks;
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
     const int b = rem / p.H;
@@ -145,7 +147,14 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int q0 = qb * PF_BM;
     const int qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
-    const RowBounds rb = row_bounds(p, b, q0, PF_BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, PF_BM, qw0, lane);
+    if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
+        const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
+        rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
+        rb.lo_w = max(rb.lo_w, c_lo), rb.hi_w = min(rb.hi_w, c_hi);
+        rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
+        rb.klo = max(rb.klo, c_lo), rb.khi = min(rb.khi, c_hi);
+    }
     const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const int full_lo_w = rb.full_lo_w, full_hi_w = rb.full_hi_w, klo = rb.klo, khi = rb.khi;
     const int qrow = min(query, p.Sq - 1);
@@ -497,20 +506,32 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     lds_barrier();
     // ---- epilogue: out[query][dim] = O^T[dim][query] / l ----------------------------------------------
     const float l_tot = half_swap_sum(l);
-    const float inv = 1.0f / l_tot;
-    const bool dead = (l_tot == 0.0f);  // no visible key: the reference gives NaN (0/0)
-    if (out_vec) {
+    // With the keys split over workgroups the "output" is this share's row in the partials: O unnormalised
+    // as f32 in 16-byte pieces, then (m, l); the merge kernel normalises.
+    const bool parked = nks > 1;
+    const float inv = parked ? 1.0f : 1.0f / l_tot;
+    const bool dead = !parked && (l_tot == 0.0f);  // no visible key: the reference gives NaN (0/0)
+    const bool out_f32 = parked || p.out_f32;
+    const int64_t os0 = parked ? (int64_t)p.H * p.Sq * nks * p.pf_pitch : p.os[0];
+    const int64_t os1 = parked ? (int64_t)p.Sq * nks * p.pf_pitch : p.os[1];
+    const int64_t os2 = parked ? (int64_t)nks * p.pf_pitch : p.os[2];
+    char *const og = parked ? (char *)(p.partials + (int64_t)ksplit * p.pf_pitch) : (char *)p.out;
+    if (parked && query < p.Sq && h2 == 0) {
+        float *ws = (float *)og + b * os0 + h * os1 + (int64_t)query * os2;
+        ws[D] = m;
+        ws[D + 1] = l_tot;
+    }
+    if (out_vec || parked) {
         // transpose through a wavefront-private slice of the LDS so that every global store is a
         // 16-byte piece of a contiguous row; 32 rows per round for 2-byte outputs, 16 for f32
-        const int esz = p.out_f32 ? 4 : 2;
+        const int esz = out_f32 ? 4 : 2;
         const int pitch = D * esz + 16;                      // rows stay 16-byte aligned, 4 banks apart
         constexpr int SLICE = 32 * (D * 2 + 16);             // bytes per wavefront
         static_assert(PF_WAVES * SLICE <= NS * STAGE, "epilogue staging exceeds the tile buffers");
         auto wbase = lds_base + wave * SLICE;
-        const int rounds = p.out_f32 ? 2 : 1;
+        const int rounds = out_f32 ? 2 : 1;
         const int rows_per_round = 32 / rounds;
         const int cpr = D * esz / 16;
-        char *og = (char *)p.out;
         for (int rd = 0; rd < rounds; rd++) {
             const int row_lo_ = rd * rows_per_round;
             if (ln >= row_lo_ && ln < row_lo_ + rows_per_round) {
@@ -522,7 +543,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
                         for (int e = 0; e < 4; e++) v4[e] = dead ? __builtin_nanf("") : o[db][4 * rq + e] * inv;
                         const int dim = 32 * db + 8 * rq + 4 * h2;
-                        if (p.out_f32) {
+                        if (out_f32) {
                             *(__attribute__((address_space(3))) float4_t *)(wbase + (ln - row_lo_) * pitch + dim * 4) =
                                 float4_t{v4[0], v4[1], v4[2], v4[3]};
                         } else {
@@ -537,7 +558,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                 const int qr = qw0 + row_lo_ + row;
                 if (qr < p.Sq) {
                     const uint4_t val = *(__attribute__((address_space(3))) uint4_t *)(wbase + row * pitch + col * 16);
-                    const int64_t eidx = b * p.os[0] + h * p.os[1] + (int64_t)qr * p.os[2];
+                    const int64_t eidx = b * os0 + h * os1 + (int64_t)qr * os2;
                     *(uint4_t *)(og + eidx * esz + col * 16) = val;
                 }
             }
@@ -560,7 +581,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 template <typename T>
 static int launch_t(const AttnParams &p, hipStream_t stream) {
     const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
-    const long blocks = (long)nqb * p.B * p.H;
+    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -578,7 +599,32 @@ static int launch_t(const AttnParams &p, hipStream_t stream) {
         default: set_error("prefill MFMA kernel: head_dim %d not in {64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
+    if (p.pf_nsplit > 1) return launch_prefill_merge(p, sizeof(T) == 2 && std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     return FHIP_OK;
+}
+
+// Few query rows on a long cache: 256-row query blocks alone leave most CUs idle, so the keys are split over
+// workgroups too, down to 1024 keys per share, until there are about two workgroups per CU.
+void prefill_mfma_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+    *nsplit = 1;
+    *chunk = Skv;
+    if (causal_square) return;
+    const long wgs = (long)B * H * ((Sq + PF_BM - 1) / PF_BM);
+    if (2 * wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy: parking and
+                                          // merging partial results would cost more than it gains (measured)
+    const long want = (2L * compute_units + wgs - 1) / wgs;
+    const long most = Skv / 1024;
+    long ns = want < most ? want : most;
+    if (ns < 2) return;
+    long c = (Skv + ns - 1) / ns;
+    c = (c + PF_BN - 1) / PF_BN * PF_BN;
+    *chunk = (int)c;
+    *nsplit = (int)((Skv + c - 1) / c);
+}
+
+size_t prefill_mfma_workspace_bytes(int B, int H, int Sq, int D, int nsplit) {
+    if (nsplit <= 1) return 0;
+    return (size_t)B * H * Sq * nsplit * (size_t)(D + 4) * sizeof(float);
 }
 
 int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {

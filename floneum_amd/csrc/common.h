@@ -39,15 +39,21 @@ struct AttnParams {
     // (two workgroups per CU) nothing is rebalanced at run time, so the second half of the numbers is walked
     // backwards: a CU's two workgroups are then a long and a short one.  0: off; else the number of CUs.
     int32_t snake_cus;
-    // Tiled f32 prefill only: keys split over pf_nsplit workgroups per query block (few query rows on a long
+    // Tiled prefill kernels: keys split over pf_nsplit workgroups per query block (few query rows on a long
     // cache would otherwise occupy a fraction of the chip).  Split s takes keys [s * pf_chunk, (s + 1) * pf_chunk)
-    // and parks (O unnormalised, m, l) per row in `partials` [B, H, Sq, pf_nsplit, D + 2]; a merge kernel follows.
+    // and parks (O unnormalised, m, l) per row in `partials` [B, H, Sq, pf_nsplit, pf_pitch]; a merge kernel follows.
     int32_t pf_nsplit, pf_chunk;
+    int32_t pf_pitch;  // floats per (row, share) in `partials`: D + 2, or D + 4 where rows are written in 16-byte pieces
 };
 
 // the key split of a tiled f32 prefill call (1 = none) and the scratch it needs
 void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk);
 size_t prefill_f32_workspace_bytes(int B, int H, int Sq, int D, int nsplit);
+// the same for the 16-bit matrix-core prefill kernel (256-row query blocks, one workgroup per CU)
+void prefill_mfma_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk);
+size_t prefill_mfma_workspace_bytes(int B, int H, int Sq, int D, int nsplit);
+// merges the key shares parked in p.partials (p.pf_nsplit, p.pf_pitch) into p.out
+int launch_prefill_merge(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 
 // bytes of device scratch the interval form of a dense mask needs
 size_t mask_intervals_bytes(int rows);

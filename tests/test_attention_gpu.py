@@ -525,11 +525,12 @@ def test_decode_over_a_very_long_cache(device, dtype, D):
     assert_parity(out1, want, dict(max_abs=1e-6, rel_l2=1e-6) if dtype == fa.F32 else TOL_16, "window of one key at the end")
 
 
-@pytest.mark.parametrize("dtype,D", [(fa.F32, 128), (fa.F32, 64), (fa.F32, 80), (fa.F16, 80), (fa.BF16, 40)])
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 128), (fa.F32, 64), (fa.F32, 80), (fa.F16, 80), (fa.BF16, 40), (fa.F16, 128),
+                                     (fa.BF16, 64), (fa.F16, 96)])
 @pytest.mark.parametrize("case", ["causal_offset", "window", "mask_tensor", "bias_tensor", "kv_lens", "full"])
 def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
-    """A new chat turn on a long cached context: few query blocks, thousands of keys.  The f32-arithmetic tiled
-    kernel then splits the keys over workgroups and merges the shares; the result must not depend on it."""
+    """A new chat turn on a long cached context: few query blocks, thousands of keys.  Both tiled prefill kernels
+    then split the keys over workgroups and merge the shares; the result must not depend on it."""
     B, H, Hkv, Sq, Skv = 1, 4, 2, 100, 5000
     q, k, v = _normal_qkv(17, B, H, Hkv, Sq, Skv, D)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
