@@ -337,17 +337,19 @@ __global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
     float M = -INFINITY;
     for (int sp = 0; sp < ns; sp++) M = fmaxf(M, ws[sp * pitch + D]);
     const float Ms = (M == -INFINITY) ? 0.0f : M;
-    float L = 0.0f, A0 = 0.0f, A1 = 0.0f;
+    float L = 0.0f, A[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // dims lane, lane + 64, lane + 128, lane + 192
     for (int sp = 0; sp < ns; sp++) {
         const float *src = ws + sp * pitch;
         const float w = __builtin_amdgcn_exp2f(src[D] - Ms);
         L += w * src[D + 1];
-        if (lane < D) A0 += w * src[lane];
-        if (lane + 64 < D) A1 += w * src[lane + 64];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (lane + 64 * k < D) A[k] += w * src[lane + 64 * k];
     }
     const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
-    if (lane < D) store_out<T>(p, ob + lane * p.os[3], A0 / L);  // no visible key: 0/0 = NaN like the reference
-    if (lane + 64 < D) store_out<T>(p, ob + (lane + 64) * p.os[3], A1 / L);
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (lane + 64 * k < D) store_out<T>(p, ob + (lane + 64 * k) * p.os[3], A[k] / L);  // no visible key: 0/0 = NaN
 }
 
 // ---- head_dim 129 .. 256 (Gemma-3's key length is 256) -------------------------------------------------------
@@ -380,7 +382,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     const int d0 = PFW_DH * hf;
 
     const int bh_count = p.B * p.H;
-    const int id = snake_order(blockIdx.x, gridDim.x, p.snake_cus);
+    const int nks = max(p.pf_nsplit, 1);
+    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
+    const int id = snake_order(blockIdx.x / nks, gridDim.x / nks, p.snake_cus);
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
     const int b = rem / p.H;
@@ -391,7 +395,14 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     const int q0 = qb * BM;
     const int qw0 = q0 + 32 * pr;
     const int query = qw0 + ln;
-    const RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    if (nks > 1) {  // this workgroup's share of the keys
+        const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
+        rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
+        rb.lo_w = max(rb.lo_w, c_lo), rb.hi_w = min(rb.hi_w, c_hi);
+        rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
+        rb.klo = max(rb.klo, c_lo), rb.khi = min(rb.khi, c_hi);
+    }
     const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const bool wave_has_rows = qw0 < p.Sq;
 
@@ -519,6 +530,24 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     }
 
     const float l_tot = half_swap_sum32(l);
+    if (nks > 1) {
+        // park this share's state (each wavefront of the pair its half of the dims); the merge kernel normalises
+        if (query < p.Sq) {
+            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * p.pf_pitch;
+#pragma unroll
+            for (int db = 0; db < PFW_DH / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int dim = d0 + 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                    if (dim < p.D) ws[dim] = o[db][r];
+                }
+            if (hf == 0 && h2 == 0) {
+                ws[p.D] = m;
+                ws[p.D + 1] = l_tot;
+            }
+        }
+        return;
+    }
     if (query < p.Sq) {
         const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
@@ -532,19 +561,23 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
 }
 
 template <typename T>
+static int launch_merge_t(const AttnParams &p, hipStream_t stream);
+
+template <typename T>
 static int launch_wide(const AttnParams &p, hipStream_t stream) {
     if (p.mask && !p.iv) {
         set_error("prefill f32: a mask tensor without its interval form is not supported above head_dim 128");
         return FHIP_ERR_UNSUPPORTED;
     }
     const int nqb = (p.Sq + 63) / 64;
-    const long blocks = (long)nqb * p.B * p.H;
+    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
     }
     hipLaunchKernelGGL(prefill_f32_wide_kernel<T>, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), 0, stream, p, nqb);
     FHIP_HIP_CHECK(hipGetLastError());
+    if (p.pf_nsplit > 1) return launch_merge_t<T>(p, stream);
     return FHIP_OK;
 }
 
@@ -595,8 +628,9 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
 void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk) {
     *nsplit = 1;
     *chunk = Skv;
-    if (D > 128 || causal_square) return;
-    const long wgs = (long)B * H * ((Sq + 31) / 32);  // at the finest query blocking the kernel has
+    if (causal_square) return;
+    const int bm = D > 128 ? 64 : 32;  // the finest query blocking the kernel has
+    const long wgs = (long)B * H * ((Sq + bm - 1) / bm);
     if (wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy (two workgroups per CU)
     const long want = (2L * compute_units + wgs - 1) / wgs;
     const long most = Skv / 512;

@@ -526,7 +526,7 @@ def test_decode_over_a_very_long_cache(device, dtype, D):
 
 
 @pytest.mark.parametrize("dtype,D", [(fa.F32, 128), (fa.F32, 64), (fa.F32, 80), (fa.F16, 80), (fa.BF16, 40), (fa.F16, 128),
-                                     (fa.BF16, 64), (fa.F16, 96)])
+                                     (fa.BF16, 64), (fa.F16, 96), (fa.F32, 256), (fa.F16, 192)])
 @pytest.mark.parametrize("case", ["causal_offset", "window", "mask_tensor", "bias_tensor", "kv_lens", "full"])
 def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
     """A new chat turn on a long cached context: few query blocks, thousands of keys.  Both tiled prefill kernels
@@ -543,6 +543,8 @@ def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
         mask, kind = oracle.get_mask(Sq, Skv - Sq), "qk"
         mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
     elif case == "bias_tensor":
+        if D > 128:
+            pytest.skip("mask tensors without an interval form go to the general kernel above head_dim 128")
         mask, kind = np.random.default_rng(4).normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
         mask[:, 700:2100] = NEG_INF
         mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
