@@ -44,6 +44,12 @@ def configs():
                    q_pos_offset=3584, window=4096),
         "C5": dict(kind="decode", B=32, H=32, Hkv=32, Sq=1, Skv=32768, D=96, dtype="f16", std=1.0, causal=False,
                    ragged=(128, 32768)),
+        # not a headline configuration: a new chat turn, 128 query rows on 8192 cached keys (the shape at which the
+        # prefill kernels split the keys over workgroups), in the reference's f32 and in f16
+        "T1": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=128, Skv=8192, D=128, dtype="f32", std=1.0, causal=True,
+                   q_pos_offset=8064),
+        "T2": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=128, Skv=8192, D=128, dtype="f16", std=1.0, causal=True,
+                   q_pos_offset=8064),
     }
 
 

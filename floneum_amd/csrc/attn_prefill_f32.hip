@@ -334,17 +334,35 @@ __global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
     const int h = (int)((row / p.Sq) % p.H), b = (int)(row / p.Sq / p.H);
     const int D = p.D, ns = p.pf_nsplit, pitch = p.pf_pitch;
     const float *ws = p.partials + row * ns * pitch;
-    float M = -INFINITY;
-    for (int sp = 0; sp < ns; sp++) M = fmaxf(M, ws[sp * pitch + D]);
-    const float Ms = (M == -INFINITY) ? 0.0f : M;
-    float L = 0.0f, A[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // dims lane, lane + 64, lane + 128, lane + 192
-    for (int sp = 0; sp < ns; sp++) {
-        const float *src = ws + sp * pitch;
-        const float w = __builtin_amdgcn_exp2f(src[D] - Ms);
-        L += w * src[D + 1];
+    // eight shares per round of loads (a round costs one memory latency)
+    float M = -INFINITY, L = 0.0f, A[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // dims lane, lane + 64, lane + 128, lane + 192
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+        float ms[8], ls[8], av[8][4];
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-            if (lane + 64 * k < D) A[k] += w * src[lane + 64 * k];
+        for (int u = 0; u < 8; u++) {
+            const bool ok = s0 + u < ns;
+            const float *src = ws + (ok ? s0 + u : s0) * pitch;
+            ms[u] = ok ? src[D] : -INFINITY;
+            ls[u] = ok ? src[D + 1] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) av[u][k] = (ok && lane + 64 * k < D) ? src[lane + 64 * k] : 0.0f;
+        }
+        float Mn = M;
+#pragma unroll
+        for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
+        const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+        const float c = __builtin_amdgcn_exp2f(M - Ms);
+        L *= c;
+#pragma unroll
+        for (int k = 0; k < 4; k++) A[k] *= c;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
+            L += w * ls[u];
+#pragma unroll
+            for (int k = 0; k < 4; k++) A[k] += w * av[u][k];
+        }
+        M = Mn;
     }
     const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)query * p.os[2];
 #pragma unroll
