@@ -166,16 +166,13 @@ static bool output_is_empty(const fhip_attn_args *a) {
 }
 static bool no_keys(const fhip_attn_args *a) { return a->k.shape[2] == 0; }
 
-static bool aligned16(const void *p, uint64_t off_elems, int eb) {
-    return (((uintptr_t)p + off_elems * (uint64_t)eb) & 15u) == 0;
-}
-
-static bool rows_vectorizable(const fhip_tensor4 &t, int eb) {
-    const int per16 = 16 / eb;
+// rows readable in pieces of `bytes` (16, or 8 for the four-element pieces of a 16-bit row)
+static bool rows_vectorizable(const fhip_tensor4 &t, int eb, int bytes = 16) {
+    const int per = bytes / eb;
     if (t.shape[3] > 1 && t.stride[3] != 1) return false;
-    if (!aligned16(t.ptr, t.offset, eb)) return false;
+    if ((((uintptr_t)t.ptr + t.offset * (uint64_t)eb) & (uintptr_t)(bytes - 1)) != 0) return false;
     for (int i = 0; i < 3; i++)
-        if (t.shape[i] > 1 && (t.stride[i] % per16) != 0) return false;
+        if (t.shape[i] > 1 && (t.stride[i] % per) != 0) return false;
     return true;
 }
 
@@ -212,8 +209,9 @@ static bool prefill_f32_eligible(const fhip_attn_args *a) {
     const uint32_t D = a->q.shape[3];
     if (D % 4 != 0 || D > 256) return false;  // rows are padded with zeros to the tile width on the way into LDS
     if (!(a->scale > 0.0f)) return false;
-    const int eb = elem_bytes(a->dtype);
-    if (!rows_vectorizable(a->q, eb) || !rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;
+    const int eb = elem_bytes(a->dtype), piece = 4 * eb;  // rows are read four elements at a time
+    if (!rows_vectorizable(a->q, eb, piece) || !rows_vectorizable(a->k, eb, piece) || !rows_vectorizable(a->v, eb, piece))
+        return false;
     return true;
 }
 
