@@ -134,6 +134,11 @@ SYMBOLS = {
     "fhip_kv_cache_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
                                                  ctypes.POINTER(CTensor4)]),
+    "fhip_kv_cache_qkv_rope_append": (ctypes.c_int, [_P, _P, ctypes.POINTER(CRmsNorm), ctypes.POINTER(CRmsNorm),
+                                                     ctypes.POINTER(CRopeTables), ctypes.POINTER(CTensor4), ctypes.c_int,
+                                                     ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
+                                                     ctypes.POINTER(CTensor4), ctypes.c_int, ctypes.POINTER(CTensor4),
+                                                     ctypes.POINTER(CTensor4)]),
     "fhip_stream_begin_capture": (ctypes.c_int, [_P]),
     "fhip_stream_end_capture": (ctypes.c_int, [_P, _PP]),
     "fhip_graph_launch": (ctypes.c_int, [_P, _P]),
@@ -672,6 +677,29 @@ class KvCache:
             return Tensor(_View(self.device, c.ptr, self), self.dtype, tuple(c.shape), tuple(c.stride), c.offset)
 
         return wrap(ka), wrap(va)
+
+
+def _kv_step(self, rope, q, k, v, start_pos, interleaved=False, q_norm=None, k_norm=None, q_out_dtype=None):
+    """rope(norm(q)) and append(rope(norm(k)), v) in one launch; returns (q_rotated, k_all, v_all)."""
+    assert k.dtype == v.dtype
+    q_out = Tensor.empty(self.device, q.shape, q_out_dtype if q_out_dtype is not None else q.dtype)
+    cq, co, ck, cv = q._c4(), q_out._c4(), k._c4(), v._c4()
+    ka, va = CTensor4(), CTensor4()
+    tables = rope._tables(start_pos, interleaved)
+    qn = q_norm._c() if q_norm is not None else None
+    kn = k_norm._c() if k_norm is not None else None
+    check(lib().fhip_kv_cache_qkv_rope_append(self.handle, self.device.stream, ctypes.byref(qn) if qn is not None else None,
+                                              ctypes.byref(kn) if kn is not None else None, ctypes.byref(tables),
+                                              ctypes.byref(cq), q.dtype, ctypes.byref(co), q_out.dtype, ctypes.byref(ck),
+                                              ctypes.byref(cv), k.dtype, ctypes.byref(ka), ctypes.byref(va)))
+
+    def wrap(c):
+        return Tensor(_View(self.device, c.ptr, self), self.dtype, tuple(c.shape), tuple(c.stride), c.offset)
+
+    return q_out, wrap(ka), wrap(va)
+
+
+KvCache.qkv_rope_append = _kv_step
 
 
 def base_inverse_frequency(dim, rope_theta):

@@ -913,6 +913,7 @@ struct NewRows {
     fhip_dtype src_dtype;
     const fhip_rope_tables *rope;  // nullptr: plain copy
     const fhip_rms_norm *k_norm;   // with rope: the keys are normalised first (nullptr: not)
+    fhip::RowJobs *batch;          // not nullptr: the rotated / converted rows are queued here instead of launched
 };
 
 // rows [first, first + count) of the new block `src` -> dst (cache dtype, strides dst_st); side 0 = keys
@@ -925,6 +926,12 @@ static int write_new_rows(const fhip_kv_cache *c, hipStream_t st, int side, cons
     const int mode = side == 0 ? (nr.rope->interleaved ? 1 : 0) : 2;
     fhip::RowNorm norm;
     if (side == 0 && nr.k_norm) norm = {nr.k_norm->weight, nr.k_norm->bias, nr.k_norm->dtype, nr.k_norm->eps};
+    if (nr.batch && nr.batch->n < 3) {
+        fhip::fill_row_job(&nr.batch->job[nr.batch->n++], sp, src->stride, nr.src_dtype, dst, dst_st, c->dtype, shp,
+                           nr.rope->cos, nr.rope->sin, (int64_t)(nr.rope->start_pos + first), mode,
+                           side == 0 && nr.k_norm ? &norm : nullptr);
+        return FHIP_OK;
+    }
     return launch_rope_rows(sp, src->stride, nr.src_dtype, dst, dst_st, c->dtype, shp, nr.rope->cos, nr.rope->sin,
                             (int64_t)(nr.rope->start_pos + first), mode, side == 0 && nr.k_norm ? &norm : nullptr, st);
 }
@@ -1137,6 +1144,7 @@ int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k
     nr.src_dtype = c ? c->dtype : FHIP_F32;
     nr.rope = nullptr;
     nr.k_norm = nullptr;
+    nr.batch = nullptr;
     return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
 }
 
@@ -1215,7 +1223,7 @@ int fhip_norm_rope(fhip_stream *s, const fhip_rms_norm *norm, const fhip_rope_ta
 
 static int rope_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *k_norm, const fhip_rope_tables *rope,
                             const fhip_tensor4 *k_new, const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all,
-                            fhip_tensor4 *v_all) {
+                            fhip_tensor4 *v_all, fhip::RowJobs *batch = nullptr) {
     if (!k_new || !fhip::dtype_ok(in_dtype)) {
         set_error("kv_cache_rope_append: NULL argument or bad dtype");
         return FHIP_ERR_INVALID_ARG;
@@ -1226,12 +1234,44 @@ static int rope_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_nor
     nr.src_dtype = in_dtype;
     nr.rope = rope;
     nr.k_norm = k_norm;
+    nr.batch = batch;
     return kv_append_core(c, s, k_new, v_new, k_all, v_all, nr);
 }
 
 int fhip_kv_cache_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rope_tables *rope, const fhip_tensor4 *k_new,
                               const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
     return rope_append_core(c, s, nullptr, rope, k_new, v_new, in_dtype, k_all, v_all);
+}
+
+int fhip_kv_cache_qkv_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *q_norm, const fhip_rms_norm *k_norm,
+                                  const fhip_rope_tables *rope, const fhip_tensor4 *q, fhip_dtype q_dtype,
+                                  const fhip_tensor4 *q_out, fhip_dtype q_out_dtype, const fhip_tensor4 *k_new,
+                                  const fhip_tensor4 *v_new, fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all) {
+    if (!s || !q || !q_out || !q->ptr || !q_out->ptr || !fhip::dtype_ok(q_dtype) || !fhip::dtype_ok(q_out_dtype)) {
+        set_error("kv_cache_qkv_rope_append: NULL argument or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    for (int i = 0; i < 4; i++)
+        if (q->shape[i] != q_out->shape[i]) {
+            set_error("kv_cache_qkv_rope_append: q_out shape differs from q's");
+            return FHIP_ERR_INVALID_ARG;
+        }
+    int rc = check_rope(rope, q->shape[3], q->shape[2]);
+    if (rc) return rc;
+    if (q_norm && (rc = check_norm(q_norm))) return rc;
+    if (k_norm && (rc = check_norm(k_norm))) return rc;
+    fhip::RowJobs jobs;
+    jobs.n = 0;
+    fhip::RowNorm qn;
+    if (q_norm) qn = {q_norm->weight, q_norm->bias, q_norm->dtype, q_norm->eps};
+    const char *qp = (const char *)q->ptr + q->offset * (uint64_t)fhip::elem_bytes(q_dtype);
+    char *qo = (char *)q_out->ptr + q_out->offset * (uint64_t)fhip::elem_bytes(q_out_dtype);
+    fhip::fill_row_job(&jobs.job[jobs.n++], qp, q->stride, q_dtype, qo, q_out->stride, q_out_dtype, q->shape, rope->cos,
+                       rope->sin, (int64_t)rope->start_pos, rope->interleaved ? 1 : 0, q_norm ? &qn : nullptr);
+    // the cache bookkeeping (growth, truncation, their copies) runs as usual; the new rows join q's launch
+    rc = rope_append_core(c, s, k_norm, rope, k_new, v_new, in_dtype, k_all, v_all, &jobs);
+    if (rc) return rc;
+    return launch_row_jobs(jobs, s->s);
 }
 
 int fhip_kv_cache_norm_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *k_norm,

@@ -104,6 +104,29 @@ struct RowNorm {
     fhip_dtype dtype;
     float eps;
 };
+// one row-wise job: rows of `src` rotated / normalised / converted into `dst` (what launch_rope_rows does)
+struct RopeRows {
+    const void *src;
+    void *dst;
+    int64_t ss[4], ds[4];
+    uint32_t shape[4];  // [B, heads, rows, D]
+    int32_t src_dtype, dst_dtype;
+    const float *cos, *sin;
+    int64_t pos0;       // table row of row 0
+    int32_t mode;       // 0 normal, 1 interleaved, 2 convert only
+    const void *norm_w, *norm_b;  // [D] weight (nullptr: no norm) and optional bias, of norm_dtype
+    int32_t norm_dtype;
+    float eps;
+};
+struct RowJobs {
+    RopeRows job[3];
+    int32_t n;
+};
+void fill_row_job(RopeRows *out, const void *src, const int64_t sstride[4], fhip_dtype src_dtype, void *dst,
+                  const int64_t dstride[4], fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos, const float *sin,
+                  int64_t pos0, int mode, const RowNorm *norm);
+// all jobs in ONE launch
+int launch_row_jobs(const RowJobs &jobs, hipStream_t stream);
 int launch_rope_rows(const void *src, const int64_t sstride[4], fhip_dtype src_dtype, void *dst,
                      const int64_t dstride[4], fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos,
                      const float *sin, int64_t pos0, int mode, const RowNorm *norm, hipStream_t stream);

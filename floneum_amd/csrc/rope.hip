@@ -36,20 +36,6 @@ __device__ __forceinline__ void store_from_f32(void *p, int64_t idx, int dtype, 
     else ((bf16_t *)p)[idx] = from_float<bf16_t>(v);
 }
 
-struct RopeRows {
-    const void *src;
-    void *dst;
-    int64_t ss[4], ds[4];
-    uint32_t shape[4];  // [B, heads, rows, D]
-    int32_t src_dtype, dst_dtype;
-    const float *cos, *sin;
-    int64_t pos0;       // table row of row 0
-    int32_t mode;       // 0 normal, 1 interleaved, 2 convert only
-    const void *norm_w, *norm_b;  // [D] weight (nullptr: no norm) and optional bias, of norm_dtype
-    int32_t norm_dtype;
-    float eps;
-};
-
 __device__ __forceinline__ float round_through(float v, int dtype) {
     if (dtype == FHIP_F16) return (float)(half_t)v;
     if (dtype == FHIP_BF16) return to_float(from_float<bf16_t>(v));
@@ -60,8 +46,7 @@ __device__ __forceinline__ float round_through(float v, int dtype) {
 // reference's left-to-right order (the order fixes the rounding, so the sum is not split over lanes), the
 // row's rms goes through LDS, then one lane per pair normalises and rotates as below.
 constexpr int NORM_ROPE_MAX_ROWS = 256;
-__global__ __launch_bounds__(256) void norm_rope_rows_kernel(RopeRows a) {
-    __shared__ float rms_of[NORM_ROPE_MAX_ROWS];
+__device__ __forceinline__ void norm_rope_rows_body(const RopeRows &a, float *rms_of) {
     const uint32_t D = a.shape[3], half = D / 2;
     const int64_t rows = (int64_t)a.shape[0] * a.shape[1] * a.shape[2];
     const int rpb = half >= 256 ? 1 : 256 / half;  // rows per group
@@ -116,7 +101,12 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(RopeRows a) {
     }
 }
 
-__global__ __launch_bounds__(256) void rope_rows_kernel(RopeRows a) {
+__global__ __launch_bounds__(256) void norm_rope_rows_kernel(RopeRows a) {
+    __shared__ float rms_of[NORM_ROPE_MAX_ROWS];
+    norm_rope_rows_body(a, rms_of);
+}
+
+__device__ __forceinline__ void rope_rows_body(const RopeRows &a) {
     const uint32_t D = a.shape[3], half = D / 2;
     const int64_t per_row = a.mode == 2 ? D : half;
     const int64_t total = (int64_t)a.shape[0] * a.shape[1] * a.shape[2] * per_row;
@@ -146,10 +136,21 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(RopeRows a) {
     }
 }
 
-int launch_rope_rows(const void *src, const int64_t ss[4], fhip_dtype src_dtype, void *dst, const int64_t ds[4],
-                     fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos, const float *sin, int64_t pos0,
-                     int mode, const RowNorm *norm, hipStream_t stream) {
-    RopeRows a;
+__global__ __launch_bounds__(256) void rope_rows_kernel(RopeRows a) { rope_rows_body(a); }
+
+// Several row jobs in one launch (blockIdx.y picks the job): the rotation of q, the rotated keys and the values of
+// one decode step are three tiny jobs whose launch cost exceeds their run time.
+__global__ __launch_bounds__(256) void row_jobs_kernel(RowJobs js) {
+    __shared__ float rms_of[NORM_ROPE_MAX_ROWS];
+    const RopeRows &a = js.job[blockIdx.y];
+    if (a.norm_w) norm_rope_rows_body(a, rms_of);
+    else rope_rows_body(a);
+}
+
+void fill_row_job(RopeRows *out, const void *src, const int64_t ss[4], fhip_dtype src_dtype, void *dst, const int64_t ds[4],
+                  fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos, const float *sin, int64_t pos0, int mode,
+                  const RowNorm *norm) {
+    RopeRows &a = *out;
     a.src = src;
     a.dst = dst;
     for (int i = 0; i < 4; i++) {
@@ -167,6 +168,34 @@ int launch_rope_rows(const void *src, const int64_t ss[4], fhip_dtype src_dtype,
     a.norm_b = norm ? norm->bias : nullptr;
     a.norm_dtype = norm ? norm->dtype : FHIP_F32;
     a.eps = norm ? norm->eps : 0.0f;
+}
+
+static int64_t job_blocks(const RopeRows &a) {
+    const int64_t rows = (int64_t)a.shape[0] * a.shape[1] * a.shape[2];
+    if (rows == 0 || a.shape[3] == 0) return 0;
+    if (a.norm_w) {
+        const int rpb = a.shape[3] / 2 >= 256 ? 1 : 256 / (a.shape[3] / 2);
+        return (rows + rpb - 1) / rpb;
+    }
+    const int64_t total = rows * (a.mode == 2 ? a.shape[3] : a.shape[3] / 2);
+    return (total + 255) / 256;
+}
+
+int launch_row_jobs(const RowJobs &js, hipStream_t stream) {
+    if (js.n <= 0) return FHIP_OK;
+    int64_t blocks = 0;
+    for (int i = 0; i < js.n; i++) blocks = blocks > job_blocks(js.job[i]) ? blocks : job_blocks(js.job[i]);
+    if (blocks == 0) return FHIP_OK;  // the bodies stride over their own work, so an over-sized grid.x is harmless
+    hipLaunchKernelGGL(row_jobs_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536), (unsigned)js.n), dim3(256), 0, stream, js);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+int launch_rope_rows(const void *src, const int64_t ss[4], fhip_dtype src_dtype, void *dst, const int64_t ds[4],
+                     fhip_dtype dst_dtype, const uint32_t shape[4], const float *cos, const float *sin, int64_t pos0,
+                     int mode, const RowNorm *norm, hipStream_t stream) {
+    RopeRows a;
+    fill_row_job(&a, src, ss, src_dtype, dst, ds, dst_dtype, shape, cos, sin, pos0, mode, norm);
     if (a.norm_w) {
         const int64_t rows = (int64_t)shape[0] * shape[1] * shape[2];
         if (rows == 0 || shape[3] == 0) return FHIP_OK;

@@ -315,6 +315,17 @@ int fhip_kv_cache_norm_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_
                                    const fhip_rope_tables *rope, const fhip_tensor4 *k_new, const fhip_tensor4 *v_new,
                                    fhip_dtype in_dtype, fhip_tensor4 *k_all, fhip_tensor4 *v_all);
 
+/* One decode (or prefill) step's preparation in ONE launch: q_out = rope(norm(q)), and the new keys / values
+ * appended as fhip_kv_cache_norm_rope_append does (q_norm / k_norm may be NULL: no norm).  Three tiny row-wise
+ * jobs whose launch cost exceeds their run time; bit-identical to the separate calls.  No counterpart in the
+ * reference, which runs these as a dozen tensor ops (models/kalosm-llama/src/raw/attention_layer.rs:217-280,
+ * 400-420). */
+int fhip_kv_cache_qkv_rope_append(fhip_kv_cache *c, fhip_stream *s, const fhip_rms_norm *q_norm,
+                                  const fhip_rms_norm *k_norm, const fhip_rope_tables *rope, const fhip_tensor4 *q,
+                                  fhip_dtype q_dtype, const fhip_tensor4 *q_out, fhip_dtype q_out_dtype,
+                                  const fhip_tensor4 *k_new, const fhip_tensor4 *v_new, fhip_dtype in_dtype,
+                                  fhip_tensor4 *k_all, fhip_tensor4 *v_all);
+
 /* Library version string, e.g. "fusor-hip 0.1 (gfx950)". */
 const char *fhip_version(void);
 

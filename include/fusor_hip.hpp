@@ -387,6 +387,21 @@ class KvCache {
     }
     /// append(rope(k), v): the rotation of RopeCache::forward / forward_interleaved and the conversion to
     /// the cache's element type happen in the pass that writes the new rows
+    /// q_out = rope(norm(q)) and append(rope(norm(k)), v) in ONE launch (a decode step's three tiny row-wise jobs);
+    /// returns (k_all, v_all); q_out is a pre-allocated tensor of q's shape
+    std::pair<Tensor<4>, Tensor<4>> qkv_rope_append(const fhip_rope_tables &tables, const Tensor<4> &q, Tensor<4> &q_out,
+                                                    const Tensor<4> &k, const Tensor<4> &v,
+                                                    const fhip_rms_norm *q_norm = nullptr, const fhip_rms_norm *k_norm = nullptr) {
+        if (k.dtype() != v.dtype()) throw Panic("qkv_rope_append: keys and values differ in element type");
+        fhip_tensor4 qn = q.c4(), qo = q_out.c4(), kn = k.c4(), vn = v.c4(), ka{}, va{};
+        check(fhip_kv_cache_qkv_rope_append(in_->c, dev_.stream(), q_norm, k_norm, &tables, &qn, (fhip_dtype)q.dtype(), &qo,
+                                            (fhip_dtype)q_out.dtype(), &kn, &vn, (fhip_dtype)k.dtype(), &ka, &va));
+        auto wrap = [&](const fhip_tensor4 &t) {
+            Tensor<4> r(std::make_shared<Buffer>(dev_, t.ptr), dtype_, t.shape, t.stride, t.offset, in_);
+            return r;
+        };
+        return {wrap(ka), wrap(va)};
+    }
     /// k_norm (RmsNorm::c()): the keys are RMS-normalised before the rotation (attention_k_norm)
     std::pair<Tensor<4>, Tensor<4>> append_rope(const fhip_rope_tables &tables, const Tensor<4> &k, const Tensor<4> &v,
                                                 const fhip_rms_norm *k_norm = nullptr) {

@@ -188,6 +188,15 @@ static void test_rms_norm(const Device &d) {  // rms_norm.rs:163-186 (values), n
     auto kv = cache.append_rope(rope.tables(0, false), t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4), t4(d, {5.0f, 6.0f, 7.0f, 8.0f}, 1, 1, 1, 4), &n);
     auto kc = host(kv.first), vc = host(kv.second);
     EXPECT(kc[0] == 2.0f && kc[3] == 8.0f && vc[0] == 5.0f && vc[3] == 8.0f, "norm fused into the cache append");
+    // q, k and v of a step prepared by one launch
+    KvCache cache2(d, 2, 8);
+    const uint32_t qshape[4] = {1, 1, 1, 4};
+    auto q_out = Tensor<4>::empty(d, DType::F32, qshape);
+    auto kv2 = cache2.qkv_rope_append(rope.tables(0, false), t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4), q_out,
+                                      t4(d, {2.0f, -2.0f, 2.0f, -2.0f}, 1, 1, 1, 4), t4(d, {5.0f, 6.0f, 7.0f, 8.0f}, 1, 1, 1, 4), &n, nullptr);
+    auto qo = host(q_out), k2 = host(kv2.first), v2 = host(kv2.second);
+    EXPECT(qo[0] == 2.0f && qo[1] == -2.0f && qo[2] == 1.5f && qo[3] == 8.0f, "q normalised in the one-launch step: %g %g %g %g", qo[0], qo[1], qo[2], qo[3]);
+    EXPECT(k2[0] == 2.0f && k2[1] == -2.0f && k2[3] == -2.0f && v2[0] == 5.0f && v2[3] == 8.0f, "k (no norm) and v in the one-launch step");
 }
 
 static void test_capture(const Device &d) {  // a recorded rope call replays on new contents of the same buffers

@@ -182,3 +182,29 @@ def test_kv_cache_norm_rope_append(device, cache_dtype, in_dtype):
         assert np.array_equal(ka.to_numpy().view(np.uint8), np.ascontiguousarray(rk).view(np.uint8)), f"keys, step {step}"
         assert np.array_equal(va.to_numpy().view(np.uint8), np.ascontiguousarray(rv).view(np.uint8)), f"values, step {step}"
         pos += n
+
+
+@pytest.mark.parametrize("cache_dtype,in_dtype,norms", [(fa.F32, fa.F32, False), (fa.F16, fa.F32, True), (fa.F16, fa.F16, True),
+                                                        (fa.F32, fa.F32, True)])
+def test_q_k_v_prepared_in_one_launch_equals_the_separate_calls(device, cache_dtype, in_dtype, norms):
+    """fhip_kv_cache_qkv_rope_append (q rotated, new keys rotated and appended, new values appended, all in one launch)
+    against fhip_rope / fhip_norm_rope + fhip_kv_cache_(norm_)rope_append, through first append, growth, in-place appends
+    and truncation."""
+    B, H, Hkv, D, max_len = 2, 4, 2, 64, 40
+    rc = fa.RopeCache(D, 128, 10000.0, device)
+    rng = np.random.default_rng(7)
+    qn = fa.RmsNorm(rng.normal(1, 0.2, D).astype(np.float32), None, 1e-6, in_dtype, device) if norms else None
+    kn = fa.RmsNorm(rng.normal(1, 0.2, D).astype(np.float32), None, 1e-6, in_dtype, device) if norms else None
+    fused, separate = fa.KvCache(2, max_len, cache_dtype, device), fa.KvCache(2, max_len, cache_dtype, device)
+    pos = 0
+    for step, n in enumerate([5, 1, 1, 9, 1, 17, 1, 1, 12, 3]):
+        q, k, v = _x(500 + step, (B, H, n, D)), _x(600 + step, (B, Hkv, n, D)), _x(700 + step, (B, Hkv, n, D))
+        tq, tk, tv = (fa.Tensor.from_numpy(device, a, in_dtype) for a in (q, k, v))
+        q1, k1, v1 = fused.qkv_rope_append(rc, tq, tk, tv, pos, False, qn, kn, q_out_dtype=cache_dtype)
+        q2 = rc.apply(tq, pos, False, out_dtype=cache_dtype, norm=qn)
+        k2, v2 = separate.append_rope(rc, tk, tv, pos, False, k_norm=kn)
+        assert k1.shape == k2.shape and v1.shape == v2.shape
+        for a, b_, what in ((q1, q2, "q"), (k1, k2, "keys"), (v1, v2, "values")):
+            assert np.array_equal(a.to_numpy().view(np.uint8), b_.to_numpy().view(np.uint8)), f"{what}, step {step}"
+        pos += n
+    assert fused.current_seq_len() == max_len
