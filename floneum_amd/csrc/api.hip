@@ -694,6 +694,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     AttnParams p;
     fill_params(args, &p);
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    p.cus = s->dev->prop.multiProcessorCount;
     if (id == FHIP_KERNEL_PREFILL_F32) {
         // few query rows on a long cache: split the keys over workgroups if the caller brought the scratch for it
         int ns, chunk;

@@ -673,8 +673,7 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
     // workgroups per CU: the longest (last causal) query block then sets the run time, and halving it pays
     // even when every CU has work.  Measured break-even: about 4 workgroups per CU at head_dim <= 64, 2 above
     // (the bigger tiles leave less to gain).  A single wavefront moves a whole tile only up to head_dim 64.
-    int cus = 256, dev = 0;
-    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int cus = p.cus > 0 ? p.cus : 256;
     const long bh = (long)p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     const long wg1 = bh * ((p.Sq + 127) / 128), wg2 = bh * ((p.Sq + 63) / 64);
     const bool small_dim = p.D <= 64;

@@ -22,6 +22,7 @@ struct AttnParams {
     int64_t q_pos_offset, window;
     float scale;
     int32_t out_f32;        // 1: out is f32 although the inputs are 16-bit
+    int32_t cus;            // compute units of the device the call runs on (launch planning)
     // split-KV decode only
     float *partials;        // [B, H, nsplit, D + 2] per-split (acc, m, l)
     int32_t chunk;          // keys per split
