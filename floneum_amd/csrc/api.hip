@@ -872,16 +872,22 @@ int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has
 // ---- growable KV cache on the device ---------------------------------------------------------------
 
 struct fhip_tensor_cache_side {
-    void *buf = nullptr;    // [B, Hkv, allocated, D] contiguous
-    void *spare = nullptr;  // second buffer of max_sequence_len rows, used once the cache is full
+    void *buf = nullptr;  // [B, Hkv, rows, D] contiguous; rows = allocated while growing, 2 * max_len once full
 };
 
+// Once the cache is full (max_sequence_len rows) it slides: the buffer holds 2 * max_len rows per (batch, head), the
+// valid window starts at row `start`, new rows go behind it and the window moves; only when the buffer's end is
+// reached are the kept rows copied back to row 0.  The caller sees exactly what the reference's truncating branch
+// returns (the last max_len positions, in order, as one narrowed view), but an append moves O(new rows) bytes
+// instead of re-concatenating the whole window every time (tensor_cache.rs:55-78).
 struct fhip_kv_cache {
     fhip_device *dev;
     fhip_dtype dtype;
     uint64_t max_len;
     uint32_t B, Hkv, D;  // fixed by the first append
     uint64_t current, allocated;
+    bool sliding = false;
+    uint64_t start = 0;  // first valid row while sliding
     fhip_tensor_cache_side side[2];  // 0 = keys, 1 = values
 };
 
@@ -892,9 +898,9 @@ static void kv_contig_strides(const fhip_kv_cache *c, uint64_t alloc, int64_t st
     st[0] = (int64_t)c->Hkv * st[1];
 }
 
-static void kv_view(const fhip_kv_cache *c, void *buf, uint64_t alloc, uint64_t len, fhip_tensor4 *t) {
+static void kv_view(const fhip_kv_cache *c, void *buf, uint64_t alloc, uint64_t len, fhip_tensor4 *t, uint64_t first_row = 0) {
     t->ptr = buf;
-    t->offset = 0;
+    t->offset = first_row * c->D;
     t->shape[0] = c->B;
     t->shape[1] = c->Hkv;
     t->shape[2] = (uint32_t)len;
@@ -967,10 +973,11 @@ static int kv_release(fhip_kv_cache *c) {
     if (hipSetDevice(c->dev->ordinal) != hipSuccess) rc = FHIP_ERR_HIP;
     for (int s = 0; s < 2; s++) {
         if (c->side[s].buf && hipFree(c->side[s].buf) != hipSuccess) rc = FHIP_ERR_HIP;
-        if (c->side[s].spare && hipFree(c->side[s].spare) != hipSuccess) rc = FHIP_ERR_HIP;
-        c->side[s].buf = c->side[s].spare = nullptr;
+        c->side[s].buf = nullptr;
     }
     c->current = c->allocated = 0;
+    c->sliding = false;
+    c->start = 0;
     c->B = c->Hkv = c->D = 0;
     if (rc) set_error("kv_cache: hipFree failed");
     return rc;
@@ -1053,36 +1060,57 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
 
     if (required > c->max_len) {
         // keep the last max_len positions of old[new_start..] ++ new (tensor_cache.rs:55-78)
-        const uint64_t mx = c->max_len;
-        const uint64_t new_start = required - mx;
+        const uint64_t mx = c->max_len, cap = 2 * mx;
+        const uint64_t new_start = required - mx;  // rows dropped from the front of old ++ new
         const uint64_t keep_old = c->current > new_start ? c->current - new_start : 0;  // rows kept from the cache
         const uint64_t take_new = mx - keep_old;                                          // last rows of the new block
+        const bool behind = c->sliding && c->start + c->current + n <= cap;  // room behind the window: nothing moves
+        int64_t cap_st[4];
+        kv_contig_strides(c, cap, cap_st);
+        uint64_t start_after = 0;
         for (int sd = 0; sd < 2; sd++) {
             fhip_tensor_cache_side &S = c->side[sd];
-            if (!S.spare) FHIP_HIP_CHECK(hipMalloc(&S.spare, row_elems * mx * eb));
-            int64_t dst_st[4];
-            kv_contig_strides(c, mx, dst_st);
-            if (keep_old) {
-                int64_t src_st[4];
-                kv_contig_strides(c, c->allocated, src_st);
-                const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
-                int rc = launch_copy_rows((const char *)S.buf + new_start * c->D * eb, src_st, S.spare, dst_st, shp,
-                                          eb, s->s);
+            if (!c->sliding) {
+                // the cache has just filled up: move what is kept into a buffer with room to slide
+                void *nb = nullptr;
+                FHIP_HIP_CHECK(hipMalloc(&nb, row_elems * cap * eb));
+                if (keep_old) {
+                    int64_t src_st[4];
+                    kv_contig_strides(c, c->allocated, src_st);
+                    const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
+                    int rc = launch_copy_rows((const char *)S.buf + new_start * c->D * eb, src_st, nb, cap_st, shp, eb, s->s);
+                    if (rc) return rc;
+                }
+                int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
+                                        (char *)nb + keep_old * c->D * eb, cap_st, nr);
                 if (rc) return rc;
+                if (S.buf) FHIP_HIP_CHECK(hipFree(S.buf));  // waits for the copy
+                S.buf = nb;
+                start_after = 0;
+            } else if (behind) {
+                // keep_old > 0 here, so every new row is kept
+                int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n,
+                                        (char *)S.buf + (c->start + c->current) * c->D * eb, cap_st, nr);
+                if (rc) return rc;
+                start_after = c->start + new_start;
+            } else {
+                // the end of the buffer: the kept rows go back to row 0 (they lie beyond row max_len - n, so source
+                // and destination do not overlap), the new ones behind them
+                if (keep_old) {
+                    const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
+                    int rc = launch_copy_rows((const char *)S.buf + (c->start + new_start) * c->D * eb, cap_st, S.buf, cap_st,
+                                              shp, eb, s->s);
+                    if (rc) return rc;
+                }
+                int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
+                                        (char *)S.buf + keep_old * c->D * eb, cap_st, nr);
+                if (rc) return rc;
+                start_after = 0;
             }
-            int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
-                                    (char *)S.spare + keep_old * c->D * eb, dst_st, nr);
-            if (rc) return rc;
-            if (S.buf && c->allocated != mx) {
-                // the growing buffer is retired; hipFree waits for the copies above
-                FHIP_HIP_CHECK(hipFree(S.buf));
-                S.buf = nullptr;
-            }
-            void *t = S.buf;
-            S.buf = S.spare;
-            S.spare = t;
-            kv_view(c, S.buf, mx, mx, alls[sd]);
+            kv_view(c, S.buf, cap, mx, alls[sd], start_after);
         }
+        c->sliding = true;
+        c->start = start_after;
         c->current = mx;
         c->allocated = mx;
         return FHIP_OK;
@@ -1125,10 +1153,6 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
             }
             FHIP_HIP_CHECK(hipFree(S.buf));  // waits for the copy
             S.buf = nb;
-            if (S.spare) {
-                FHIP_HIP_CHECK(hipFree(S.spare));
-                S.spare = nullptr;
-            }
         }
         int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, (char *)S.buf + c->current * c->D * eb, dst_st, nr);
         if (rc) return rc;

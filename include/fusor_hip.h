@@ -250,7 +250,9 @@ int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has
  * first append stores the tensor, later appends grow the allocation to the next power of two and
  * write the new rows in place, the returned view is the valid prefix (stride[1] = allocated *
  * D), and once max_sequence_len would be exceeded only the last max_sequence_len positions are
- * kept.  Unlike the reference, growth copies once and in-place appends copy only the new rows. */
+ * kept.  Unlike the reference, growth copies once, in-place appends copy only the new rows, and a full
+ * cache slides through a buffer of 2 * max_sequence_len rows (the returned view then has stride[1] =
+ * 2 * max_sequence_len * D and a moving offset) instead of being re-concatenated on every append. */
 typedef struct fhip_kv_cache fhip_kv_cache;
 int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequence_len, fhip_kv_cache **out);
 int fhip_kv_cache_destroy(fhip_kv_cache *c);

@@ -161,7 +161,37 @@ def test_kv_cache_growth_matches_reference_semantics(device):
                 ok, ov = oc.append(kn, vn)
                 assert ka.shape == ok.shape and cache.current_seq_len() == oc.current_seq_len()
                 assert cache.allocated_seq_len() == oc.key.allocated_seq_len
-                assert ka.strides[1] == cache.allocated_seq_len() * 16  # the view keeps the allocation's stride
+                # the view keeps the buffer's stride: the allocation while it grows, twice max_len once it slides
+                assert ka.strides[1] in (cache.allocated_seq_len() * 16, 2 * max_len * 16)
                 assert np.array_equal(ka.to_numpy(), ok) and np.array_equal(va.to_numpy(), ov)
             cache.reset()
             assert cache.current_seq_len() == 0
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_full_kv_cache_slides_without_recopying(device, dtype):
+    """Once max_sequence_len rows are cached every append drops the oldest rows (tensor_cache.rs:55-78).  The device
+    cache slides a window through a buffer of twice that length, so the values and the order the caller sees are the
+    reference's, through many wrap-arounds and with blocks of every size up to beyond the window."""
+    rng = np.random.default_rng(9)
+    W, B, Hkv, D = 16, 2, 2, 32
+    cache, oc = fa.KvCache(2, W, dtype, device), oracle.KvCache(2, W)
+    npdt = np.float32 if dtype == fa.F32 else np.float16
+    sizes = [5, 9, 3] + [1] * 40 + [7, 1, 16, 1, 1, 15, 2, 40, 1, 1, 1, 17, 1] + [2] * 20
+    pos = 0
+    q = rng.standard_normal((B, 4, 1, D)).astype(np.float32)
+    tq = fa.Tensor.from_numpy(device, q, dtype)
+    for step, n in enumerate(sizes):
+        kn = rng.standard_normal((B, Hkv, n, D)).astype(npdt)
+        vn = rng.standard_normal((B, Hkv, n, D)).astype(npdt)
+        ka, va = cache.append(device, fa.Tensor.from_numpy(device, kn, dtype), fa.Tensor.from_numpy(device, vn, dtype))
+        ok, ov = oc.append(kn, vn)
+        assert ka.shape == ok.shape and cache.current_seq_len() == oc.current_seq_len(), f"step {step}"
+        assert cache.allocated_seq_len() == oc.key.allocated_seq_len, f"step {step}"
+        assert np.array_equal(ka.to_numpy(), ok) and np.array_equal(va.to_numpy(), ov), f"step {step}"
+        pos += n
+        if step % 7 == 0:  # the moving view feeds the attention call as it is
+            out = tq.flash_attention(ka, va, D ** -0.5).to_numpy()
+            ref = oracle.flash_attention(np.asarray(q, np.float32).astype(npdt).astype(np.float32), ok.astype(np.float32),
+                                         ov.astype(np.float32), D ** -0.5)
+            assert_parity(out, ref, TOL_F32 if dtype == fa.F32 else TOL_16, f"attention over the window, step {step}")
