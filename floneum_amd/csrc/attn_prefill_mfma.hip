@@ -21,6 +21,10 @@
 // phase uses no dot-product instructions: on this chip they queue behind the MFMAs of the other
 // wavefront instead of running beside them.
 // All accumulation is f32; P is rounded to the input type for the second product.
+// Key-split form (template parameter KS): the workgroup owns 128 query rows and its two wavefront groups
+// take alternate key tiles of the same rows, each through the same matrix / vector phases, and merge their
+// (m, l, O) through LDS at the end: twice the workgroups, half the longest one, for grids that do not fill
+// the chip (see use_key_split_form).
 // Masking is by interval: every query row sees one range of keys, known analytically (causal with
 // offset, sliding window, per-batch kv length, tail of the key axis) or read from the interval form
 // of a dense mask tensor (attn_bounds.h, mask_intervals.hip); key tiles that are invisible to the
@@ -87,7 +91,7 @@ struct Mma<bf16_t> {
 //     column) fall 16 bytes apart modulo the 256-byte bank period            (K: pitch 8 D + 16)
 //   - the 4 rows x 64 bytes a half-wavefront reads with the transposing load fall 64 bytes apart
 //                                                                            (V: pitch 8 D + 64)
-template <int D>
+template <int D, bool KS>
 struct PfCfg {
     static constexpr int ROWB = D * 2;                               // bytes per tile row
     static constexpr int KG = 4 * ROWB + 16;                         // K group pitch, bytes
@@ -96,7 +100,12 @@ struct PfCfg {
     static constexpr int V_BYTES = 16 * VG;
     static constexpr int CPR = D / 8;                                // 16-byte chunks per row
     static constexpr int LOAD_LANES = 4 * CPR;                       // lanes of a wavefront-wide tile load (<= 64)
-    static constexpr int NS = 3;                                     // tile stages in LDS
+    // tile buffers.  Unsplit form: three stages of (K tile, V tile), tile t in stage t % 3.  Key-split form
+    // (KS): a ring of five K tiles followed by a ring of four V tiles (see the slot schedule in the kernel).
+    static constexpr int STAGE = K_BYTES + V_BYTES;
+    static constexpr int NK = KS ? 5 : 3, NV = KS ? 4 : 3;
+    static constexpr int LDS_BYTES = KS ? NK * K_BYTES + NV * V_BYTES : 3 * STAGE;
+    static constexpr int BM = KS ? PF_BM / 2 : PF_BM;                // query rows per workgroup
 };
 
 __device__ __forceinline__ float half_swap_max(float x) {
@@ -114,13 +123,13 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 // on almost every tile.
 constexpr float PF_RESCALE_SLACK = 8.0f;
 
-template <typename T, int D>
+template <typename T, int D, bool KS>
 __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnParams p, int nqb, int out_vec) {
-    typedef PfCfg<D> C;
+    typedef PfCfg<D, KS> C;
     typedef typename Mma<T>::vec8 vec8;
-    constexpr int STAGE = C::K_BYTES + C::V_BYTES;
-    constexpr int NS = C::NS;
-    __shared__ __attribute__((aligned(16))) char smem[NS * STAGE];
+    constexpr int STAGE = C::STAGE;
+    constexpr int BM = C::BM;
+    __shared__ __attribute__((aligned(16))) char smem[C::LDS_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
@@ -144,10 +153,10 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
 
-    const int q0 = qb * PF_BM;
-    const int qw0 = q0 + 32 * wave;
+    const int q0 = qb * BM;
+    const int qw0 = q0 + 32 * (KS ? (wave & 3) : wave);  // KS: both groups own the same 128 rows
     const int query = qw0 + ln;
-    RowBounds rb = row_bounds(p, b, q0, PF_BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
     if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -197,26 +206,36 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 
     using std::integral_constant;
     // ---- tile movement: global -> LDS directly (no registers) --------------------------------------
-    // The four wavefronts of a group move one whole tile with four loads each: group 1 moves the K
-    // tiles, group 0 the V tiles.  Load j of wavefront w writes LDS group w + 4 j; lane i of it
-    // fetches row 16 (i / CPR) + w + 4 j, 16-byte column i % CPR, so the lanes of one load land
-    // contiguously (which is what the hardware does with a direct load) and the four loads of a
-    // wavefront differ by a uniform offset only.
+    // The four wavefronts of a group move one whole tile with four loads each.  Load j of wavefront w
+    // writes LDS group w + 4 j; lane i of it fetches row 16 (i / CPR) + w + 4 j, 16-byte column i % CPR, so
+    // the lanes of one load land contiguously (which is what the hardware does with a direct load) and the
+    // four loads of a wavefront differ by a uniform offset only.
+    // Unsplit form: group 1 moves the K tiles, group 0 the V tiles.  Key-split form: the group that is in
+    // its vector phase moves one K and one V tile.
+    // The tensors as raw buffer descriptors (base, no stride, size in bytes, 32-bit raw format): a row beyond
+    // the end of the key axis reads as zero.
     const bool moves_k = group == 1;
-    const int mrow_bytes = moves_k ? krow_bytes : vrow_bytes;
-    // the moved tensor as a raw buffer descriptor (base, no stride, size in bytes, 32-bit raw format)
-    const uint64_t mptr = (uint64_t)(moves_k ? kg : vg);
-    const uint4_t mrs = {(uint32_t)mptr, (uint32_t)(mptr >> 32) & 0xffffu,
-                         (uint32_t)((p.Skv - 1) * mrow_bytes + D * 2), 0x00020000u};
     const int wv = wave & 3;
-    const int gofs = (16 * (lane / C::CPR) + wv) * mrow_bytes + (lane % C::CPR) * 16;
-    const int lds_move_base = (moves_k ? 0 : C::K_BYTES) + wv * (moves_k ? C::KG : C::VG);
-    const int lds_move_step = 4 * (moves_k ? C::KG : C::VG);
+    auto descriptor = [&](const uint16_t *base, int row_bytes) __attribute__((always_inline)) {
+        const uint64_t ptr = (uint64_t)base;
+        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((p.Skv - 1) * row_bytes + D * 2),
+                       0x00020000u};
+    };
+    const uint4_t krs = descriptor(kg, krow_bytes), vrs = descriptor(vg, vrow_bytes);
+    const int gofs_k = (16 * (lane / C::CPR) + wv) * krow_bytes + (lane % C::CPR) * 16;
+    const int gofs_v = (16 * (lane / C::CPR) + wv) * vrow_bytes + (lane % C::CPR) * 16;
+    // where tile t lives in LDS
+    auto k_stage = [&](int t) __attribute__((always_inline)) { return KS ? (t % C::NK) * C::K_BYTES : (t % 3) * STAGE; };
+    auto v_stage = [&](int t) __attribute__((always_inline)) {
+        return KS ? C::NK * C::K_BYTES + (t % C::NV) * C::V_BYTES : (t % 3) * STAGE + C::K_BYTES;
+    };
     // a tile that starts beyond the key axis is never used: clamp the (uniform) offset so it stays
     // inside 32 bits; rows past Skv inside a used tile are out of range of the buffer and read 0
-    auto issue_tile = [&](int tile) __attribute__((always_inline)) {
-        const int soff = min(j_begin + tile * PF_BN, p.Skv) * mrow_bytes;
-        const int lbase = (tile % NS) * STAGE + lds_move_base;
+    auto issue_loads = [&](const uint4_t rs, int gofs, int row_bytes, int tile, int lbase, int lstep)
+                           __attribute__((always_inline)) {
+        // (uniform values; pinned to scalar registers, which is what the instruction takes)
+        const int soff = __builtin_amdgcn_readfirstlane(min(j_begin + tile * PF_BN, p.Skv) * row_bytes);
+        lbase = __builtin_amdgcn_readfirstlane(lbase);
         if (C::LOAD_LANES == 64 || lane < C::LOAD_LANES) {
             // written as assembly on purpose: the compiler would otherwise make every later LDS read
             // of this wavefront wait for these loads, whose data is not due before the next barrier
@@ -224,22 +243,44 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             for (int j = 0; j < 4; j++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                              :
-                             : "s"(lbase + j * lds_move_step), "v"(gofs), "s"(mrs), "s"(soff + 4 * j * mrow_bytes)
+                             : "s"(lbase + j * lstep), "v"(gofs), "s"(rs), "s"(soff + 4 * j * row_bytes)
                              : "memory", "m0");
         }
     };
-    // all but the `newer` most recent tile loads of this wavefront have landed
+    auto issue_k = [&](int tile) __attribute__((always_inline)) {
+        issue_loads(krs, gofs_k, krow_bytes, tile, k_stage(tile) + wv * C::KG, 4 * C::KG);
+    };
+    auto issue_v = [&](int tile) __attribute__((always_inline)) {
+        issue_loads(vrs, gofs_v, vrow_bytes, tile, v_stage(tile) + wv * C::VG, 4 * C::VG);
+    };
+    // unsplit form: this group's tensor, tile `tile`
+    const uint4_t mrs = moves_k ? krs : vrs;
+    const int mgofs = moves_k ? gofs_k : gofs_v, mrow_bytes = moves_k ? krow_bytes : vrow_bytes;
+    const int lds_move_base = (moves_k ? 0 : C::K_BYTES) + wv * (moves_k ? C::KG : C::VG);
+    const int lds_move_step = 4 * (moves_k ? C::KG : C::VG);
+    auto issue_tile = [&](int tile) __attribute__((always_inline)) {
+        issue_loads(mrs, mgofs, mrow_bytes, tile, (tile % 3) * STAGE + lds_move_base, lds_move_step);
+    };
+    // key-split form, slot s: K(s + 4) and V(s + 1)
+    auto issue_slot = [&](int slot) __attribute__((always_inline)) {
+        issue_k(slot + 4);
+        issue_v(slot + 1);
+    };
+    // all but the loads of this wavefront's most recent `newer` vector phases have landed
     auto wait_tiles = [&](auto newer) __attribute__((always_inline)) {
         if constexpr (decltype(newer)::value == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else if constexpr (KS) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     };
+    // local tile index -> tile: in the key-split form group g owns the tiles t with t % 2 == g
+    auto tile_of = [&](int i) __attribute__((always_inline)) { return KS ? 2 * i + group : i; };
 
     float16_t s[2];     // S^T of the tile in flight
     uint32_t pk[2][8];  // its probabilities, packed pairs in the MFMA operand order
 
-    // S^T = K . Q^T for tile i
+    // S^T = K . Q^T for this group's tile i (local index; see tile_of)
     auto qk = [&](int i) __attribute__((always_inline)) {
-        const int kbase = (i % NS) * STAGE + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
+        const int kbase = k_stage(tile_of(i)) + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
 #pragma unroll
@@ -254,7 +295,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     auto pv = [&](int i) __attribute__((always_inline)) {
         const int i16 = lane & 15;
         const int bl = (lane & 31) >> 4;
-        const int vbase = (i % NS) * STAGE + C::K_BYTES + (4 * h2 + (i16 >> 2)) * C::VG + (16 * bl + 4 * (i16 & 3)) * 2;
+        const int vbase = v_stage(tile_of(i)) + (4 * h2 + (i16 >> 2)) * C::VG + (16 * bl + 4 * (i16 & 3)) * 2;
 #pragma unroll
         for (int gq = 0; gq < 4; gq++) {  // gq = 2 t + kk: rows 16 gq + 4 h2 + {0..3} and + 8
             const int t = gq >> 1, kk = gq & 1;
@@ -279,7 +320,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     constexpr int PFK = (D == 128) ? 2 : 4;  // K operand slices in flight (register budget)
     uint4_t ka[PFK][2];
     auto prefetch_k = [&](int ik) __attribute__((always_inline)) {
-        const int kbase = (ik % NS) * STAGE + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
+        const int kbase = k_stage(tile_of(ik)) + (ln & 15) * C::KG + (ln >> 4) * C::ROWB + h2 * 16;
 #pragma unroll
         for (int kb = 0; kb < PFK; kb++)
 #pragma unroll
@@ -289,7 +330,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         constexpr bool PV = decltype(do_pv)::value;
         constexpr bool PRE = decltype(prefetched)::value;
         constexpr int NDB = D / 32, NKB = D / 16;
-        const int vstage = (ip % NS) * STAGE + C::K_BYTES, kstage = (ik % NS) * STAGE;
+        const int vstage = v_stage(tile_of(ip)), kstage = k_stage(tile_of(ik));
         const int i16 = lane & 15;
         const int bl = (lane & 31) >> 4;
         const int vbase = vstage + (4 * h2 + (i16 >> 2)) * C::VG + (16 * bl + 4 * (i16 & 3)) * 2;
@@ -359,7 +400,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     };
     // mask + online softmax (log2 domain, lazily rescaled) of tile i: s -> pk
     auto softmax = [&](int i) __attribute__((always_inline)) {
-        const int j0 = j_begin + i * PF_BN;
+        const int j0 = j_begin + tile_of(i) * PF_BN;
         if (!(j0 >= full_lo_w && j0 + PF_BN <= full_hi_w)) {
             // element r of block t is key j0 + 32 t + 8 (r / 4) + 4 h2 + r % 4
 #pragma unroll
@@ -421,11 +462,26 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // The tiles visible to a wavefront form one contiguous range [ia, ib).  Each group walks the slot
     // sequence in five static segments (nothing / first tile / steady state / last tile / nothing) so
     // that the steady-state loop body is branch-free and no state changes registers between phases.
+    //
+    // Key-split form (KS): both groups own the same 128 rows and group g takes the tiles t with t % 2 == g,
+    // so a slot is the matrix phase of tile s for one group and the vector phase of tile s-1 for the other;
+    // the groups' (m, l, O) are merged at the end.  K(t) is read in slot t (its first operands at the end of
+    // slot t-1), V(t) in slot t+2.  The group in its vector phase in slot s issues K(s+4) into the stage K(s-1)
+    // has just left (ring of 5) and V(s+1) into the stage of V(s-3), last read in slot s-1 (ring of 4), and
+    // makes sure its loads of slot s-2, K(s+2) and V(s-1), have landed: each is published by a barrier one
+    // slot before its first reader and has had two slots to arrive.  The segments below then run on the
+    // group's own tile count: local tile i of group g is tile 2 i + g.
     int ia = 0, ib = 0;
     if (wave_has_rows && hi_w > lo_w) {
         ia = (lo_w - j_begin) / PF_BN;
         ib = min(ntiles, (hi_w - j_begin + PF_BN - 1) / PF_BN);
         if (ib < ia) ib = ia;
+    }
+    int n_iter = ntiles + 1;  // iterations (two slots each) of either group
+    if constexpr (KS) {
+        ia = (ia + 1 - group) >> 1;  // this group's tiles below ia / below ib
+        ib = (ib + 1 - group) >> 1;
+        n_iter = (ntiles + 3) >> 1;
     }
     // MODE bit 0: S^T of tile i; bit 1: P.V of tile i-1; bit 2: softmax of tile i (group 0) / i-1 (group 1);
     // bit 3: the K operands of tile i were prefetched by the preceding vector phase
@@ -441,9 +497,10 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         __builtin_amdgcn_s_setprio(0);
     };
     // next_k: the tile whose S^T this wavefront computes in its next matrix phase
-    auto vector_phase = [&](int i, int tile_to_load, int next_k, auto mode) __attribute__((always_inline)) {
+    auto vector_phase = [&](int i, int tile_to_load, int slot, int next_k, auto mode) __attribute__((always_inline)) {
         constexpr int MODE = decltype(mode)::value;
-        issue_tile(tile_to_load);
+        if constexpr (KS) issue_slot(slot);
+        else issue_tile(tile_to_load);
         if constexpr ((MODE & 4) != 0) softmax(i);
         if constexpr ((MODE & 16) != 0) prefetch_k(next_k);
         wait_tiles(integral_constant<int, 1>{});  // the tile issued one vector phase ago has landed
@@ -453,20 +510,29 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         for (int i = i0; i < i1; i++) {
             matrix_phase(i, mode);
             lds_barrier();
-            vector_phase(i, i + 1, i + 1, mode);
+            vector_phase(i, i + 1, 2 * i + 1, i + 1, mode);
             lds_barrier();
         }
     };
     auto segment1 = [&](int i0, int i1, auto mode) __attribute__((always_inline)) {  // group 1: slot 2i vector (tile i-1) + K(i+1), slot 2i+1 matrix
         for (int i = i0; i < i1; i++) {
-            vector_phase(i - 1, i + 2, i, mode);
+            vector_phase(i - 1, i + 2, 2 * i, i, mode);
             lds_barrier();
             matrix_phase(i, mode);
             lds_barrier();
         }
     };
     if (ntiles > 0) {
-        if (moves_k) {
+        if constexpr (KS) {  // what slots -4 .. -1 would have issued
+            if (group == 0) {
+                issue_k(0);
+                issue_k(2);
+                issue_v(0);
+            } else {
+                issue_k(1);
+                issue_k(3);
+            }
+        } else if (moves_k) {
             issue_tile(0);
             issue_tile(1);
         } else {
@@ -483,9 +549,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                 segment0(ia, ia + 1, integral_constant<int, 1 | 4 | 16>{});
                 segment0(ia + 1, ib, integral_constant<int, 1 | 2 | 4 | 8 | 16>{});
                 segment0(ib, ib + 1, integral_constant<int, 2>{});
-                segment0(ib + 1, ntiles + 1, integral_constant<int, 0>{});
+                segment0(ib + 1, n_iter, integral_constant<int, 0>{});
             } else {
-                segment0(ia, ntiles + 1, integral_constant<int, 0>{});
+                segment0(ia, n_iter, integral_constant<int, 0>{});
             }
         } else {
             // iteration i: softmax(i-1), then S^T(i) and P.V(i-1)
@@ -494,9 +560,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                 segment1(ia, ia + 1, integral_constant<int, 1 | 8 | 16>{});
                 segment1(ia + 1, ib, integral_constant<int, 1 | 2 | 4 | 8 | 16>{});
                 segment1(ib, ib + 1, integral_constant<int, 2 | 4>{});
-                segment1(ib + 1, ntiles + 1, integral_constant<int, 0>{});
+                segment1(ib + 1, n_iter, integral_constant<int, 0>{});
             } else {
-                segment1(ia, ntiles + 1, integral_constant<int, 0>{});
+                segment1(ia, n_iter, integral_constant<int, 0>{});
             }
         }
     }
@@ -504,6 +570,36 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // the epilogue reuses the tile buffers: no tile load may still be on its way into them
     wait_tiles(integral_constant<int, 0>{});
     lds_barrier();
+    constexpr int SLICE = 32 * (D * 2 + 16);  // bytes per wavefront of the output transposition below
+    if constexpr (KS) {
+        // Group 1 hands its state to group 0, which holds the other half of the keys of the same rows:
+        // log-sum-exp merge, as the split-KV combine does.  One f32 per lane per slot, above the slices the
+        // output transposition uses.
+        constexpr int PARK = 4 * SLICE;
+        constexpr int NSLOT = D / 2 + 2;
+        static_assert(PARK + NSLOT * 1024 <= C::LDS_BYTES, "merge area exceeds the tile buffers");
+        auto park = (__attribute__((address_space(3))) float *)(lds_base + PARK) + (wave & 3) * 64 + lane;
+        if (group == 1) {
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) park[(db * 16 + r) * 256] = o[db][r];
+            park[(D / 2) * 256] = m;
+            park[(D / 2 + 1) * 256] = l;
+        }
+        lds_barrier();
+        if (group == 1) return;
+        const float m1 = park[(D / 2) * 256], l1 = park[(D / 2 + 1) * 256];
+        const float mn = fmaxf(m, m1);
+        const float c0 = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m - mn);
+        const float c1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m1 - mn);
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[db][r] = o[db][r] * c0 + park[(db * 16 + r) * 256] * c1;
+        l = l * c0 + l1 * c1;
+        m = mn;
+    }
     // ---- epilogue: out[query][dim] = O^T[dim][query] / l ----------------------------------------------
     const float l_tot = half_swap_sum(l);
     // With the keys split over workgroups the "output" is this share's row in the partials: O unnormalised
@@ -526,8 +622,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         // 16-byte piece of a contiguous row; 32 rows per round for 2-byte outputs, 16 for f32
         const int esz = out_f32 ? 4 : 2;
         const int pitch = D * esz + 16;                      // rows stay 16-byte aligned, 4 banks apart
-        constexpr int SLICE = 32 * (D * 2 + 16);             // bytes per wavefront
-        static_assert(PF_WAVES * SLICE <= NS * STAGE, "epilogue staging exceeds the tile buffers");
+        static_assert(PF_WAVES * SLICE <= C::LDS_BYTES, "epilogue staging exceeds the tile buffers");
         auto wbase = lds_base + wave * SLICE;
         const int rounds = out_f32 ? 2 : 1;
         const int rows_per_round = 32 / rounds;
@@ -578,9 +673,25 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     }
 }
 
+// Query blocks of 256 rows leave CUs idle when there are few of them (short prompts, a few new rows on a long
+// cache), and a causal prompt's last blocks are several times longer than its first.  The key-split form (128
+// rows, twice the workgroups, the longest one half as long) costs about 7 % per tile and a longer prologue and
+// epilogue; measured, it wins (1.1-1.35 x) while the 256-row grid fills at most half the CUs, for up to 128
+// query rows (where the second wavefront group would have no rows at all), and for one workgroup per CU when a
+// head has 8 or more query blocks; it loses with fewer than three key tiles.
+static bool use_key_split_form(const AttnParams &p) {
+    const int cus = p.cus > 0 ? p.cus : 256;
+    const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
+    const long wgs = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
+    if (p.Skv <= 2 * PF_BN) return false;
+    return p.Sq <= PF_BM / 2 || 2 * wgs <= cus || (wgs <= cus && nqb >= 8);
+}
+
 template <typename T>
 static int launch_t(const AttnParams &p, hipStream_t stream) {
-    const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
+    const bool ks = use_key_split_form(p);
+    const int bm = ks ? PF_BM / 2 : PF_BM;
+    const int nqb = (p.Sq + bm - 1) / bm;
     const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
@@ -592,12 +703,16 @@ static int launch_t(const AttnParams &p, hipStream_t stream) {
     int out_vec = (p.os[3] == 1 || p.D == 1) && ((uintptr_t)p.out % 16 == 0);
     for (int i = 0; i < 3; i++)
         if ((p.os[i] * oeb) % 16 != 0) out_vec = 0;
+#define PF_LAUNCH(DIM)                                                                                         \
+    if (ks) hipLaunchKernelGGL((prefill_mfma_kernel<T, DIM, true>), grid, block, 0, stream, p, nqb, out_vec);   \
+    else hipLaunchKernelGGL((prefill_mfma_kernel<T, DIM, false>), grid, block, 0, stream, p, nqb, out_vec)
     switch (p.D) {
-        case 64: hipLaunchKernelGGL((prefill_mfma_kernel<T, 64>), grid, block, 0, stream, p, nqb, out_vec); break;
-        case 96: hipLaunchKernelGGL((prefill_mfma_kernel<T, 96>), grid, block, 0, stream, p, nqb, out_vec); break;
-        case 128: hipLaunchKernelGGL((prefill_mfma_kernel<T, 128>), grid, block, 0, stream, p, nqb, out_vec); break;
+        case 64: PF_LAUNCH(64); break;
+        case 96: PF_LAUNCH(96); break;
+        case 128: PF_LAUNCH(128); break;
         default: set_error("prefill MFMA kernel: head_dim %d not in {64, 96, 128}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
+#undef PF_LAUNCH
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.pf_nsplit > 1) return launch_prefill_merge(p, sizeof(T) == 2 && std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     return FHIP_OK;

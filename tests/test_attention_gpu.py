@@ -233,6 +233,32 @@ def test_prefill_f32_key_split_forms(device, D, B, H, Sq, Skv, analytic, form):
     assert_parity(out, ref, TOL_F32, f"f32 D{D} {form}")
 
 
+@pytest.mark.parametrize("dtype,D,B,H,Sq,Skv,analytic,form", [
+    (fa.F16, 128, 2, 40, 600, 600, (True, 0, 0), "256-row blocks"),
+    (fa.BF16, 64, 3, 32, 520, 900, (True, 380, 200), "256-row blocks, window and cached keys"),
+    (fa.F16, 96, 4, 32, 300, 300, None, "256-row blocks, no mask"),
+    (fa.F16, 128, 1, 8, 600, 600, (True, 0, 0), "key-split"),
+    (fa.BF16, 64, 1, 8, 100, 1000, (True, 900, 300), "key-split, few rows, window and cached keys"),
+    (fa.F16, 96, 2, 6, 333, 333, None, "key-split, no mask"),
+    (fa.F16, 128, 1, 8, 130, 190, (True, 60, 0), "key-split, three key tiles"),
+    (fa.F16, 128, 1, 32, 2000, 2000, (True, 0, 0), "key-split, one 256-row block per CU"),
+])
+def test_prefill_16_bit_workgroup_forms(device, dtype, D, B, H, Sq, Skv, analytic, form):
+    """The 16-bit kernel runs 256 query rows per workgroup, or 128 rows with the key tiles alternating between
+    its two wavefront groups, depending on how many workgroups the call has; each form is checked at ragged
+    sizes (the grid sizes here select the form named)."""
+    Hkv = H // 2
+    q, k, v = _normal_qkv(13, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == fa.KERNEL_PREFILL_MFMA
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    mask = None if analytic is None else _analytic_mask(Sq, Skv, *analytic)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                 "qk" if mask is not None else None)
+    tol = dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16
+    assert_parity(out, ref, tol, f"D{D} {form}")
+
+
 @pytest.mark.parametrize("D", [80, 48, 4, 100, 124, 20])
 @pytest.mark.parametrize("case", ["causal", "full_ragged", "bias"])
 def test_prefill_f32_head_dims_between_the_tile_widths(device, D, case):
