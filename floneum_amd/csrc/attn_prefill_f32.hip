@@ -16,6 +16,9 @@
 // forms (template parameter S = 2, 4): the four wavefronts form S groups that own the SAME 128 / S query
 // rows, group g walks the key tiles t with t % S == g through its own LDS buffers, and the groups'
 // (m, l, O) states are merged through LDS at the end.  S times the workgroups, 1 / S of the tiles each.
+// With S = 4 a group is one wavefront; above head_dim 64 it cannot hold a K and a V tile in staging
+// registers at once, so the two take turns in one register set and one LDS buffer, with no workgroup
+// barrier inside the loop.
 //
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199; this is the data
 // type kalosm-llama always calls with (models/kalosm-llama/src/raw/attention_layer.rs:400-448).
@@ -80,7 +83,13 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     constexpr int GT = 64 * WPG;    // threads of a group
     constexpr int NCH = PF32_BN * CPR / GT;
     static_assert(PF32_BN * CPR % GT == 0, "a group's threads must cover a tile evenly");
-    __shared__ __attribute__((aligned(16))) char smem[S * 2 * K_BYTES];
+    // SOLO: a group is a single wavefront and the tile is too wide to stage K and V in registers at the same
+    // time.  The wavefront then moves its tiles alone: K and V take turns in one register set and one LDS
+    // buffer (V is fetched during S^T, the next K during P.V), and the loop needs no workgroup barrier.
+    constexpr bool SOLO = (WPG == 1 && D > 64);
+    static_assert(!(SOLO && BIAS), "the bias registers leave no room for this form");
+    constexpr int G_BYTES = SOLO ? K_BYTES : 2 * K_BYTES;  // a group's tile buffers
+    __shared__ __attribute__((aligned(16))) char smem[S * G_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     if constexpr (BIAS) {
@@ -96,7 +105,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int grp = wave / WPG;     // key-split group
     const int wig = wave % WPG;     // wavefront inside the group: which 32 rows
     const int gtid = tid % GT;      // thread inside the group
-    const int gbase = grp * 2 * K_BYTES;  // the group's tile buffers
+    const int gbase = grp * G_BYTES;
 
     const int bh_count = p.B * p.H;
     const int nks = max(p.pf_nsplit, 1);
@@ -148,47 +157,12 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     if constexpr (BIAS)
         mrow = (const T *)p.mask + (int64_t)(p.mask_kind == FHIP_MASK_QK ? min(query, p.Sq - 1) : b) * p.ms0;
 
-    float4_t kst[NCH], vst[NCH];
-    auto load_tile = [&](int j0) {
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-            const int cid = gtid + GT * i;
-            const int row = cid / CPR, col = cid % CPR;
-            const int key = min(j0 + row, p.Skv - 1);
-            const bool in_row = col * 4 < p.D;  // a head_dim below D is padded with zeros
-            kst[i] = in_row ? load4(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
-            vst[i] = in_row ? load4(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
-        }
-    };
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-            const int cid = gtid + GT * i;
-            const int row = cid / CPR, col = cid % CPR;
-            *LDS32_PTR(float4_t, gbase + row * KP + col * 16) = kst[i];
-            *LDS32_PTR(float4_t, gbase + K_BYTES + row * KP + col * 16) = vst[i];
-        }
-    };
-
-    // group g takes the tiles j_begin + (it * S + g) * 32; every group runs the same number of iterations
-    // (the barriers are workgroup-wide), a group without a tile in the last one idles through it
     const int j_begin = (lo_wg / PF32_BN) * PF32_BN;
     const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PF32_BN - 1) / PF32_BN : 0;
-    const int niter = (ntiles + S - 1) / S;
-    if (grp < ntiles) load_tile(j_begin + grp * PF32_BN);
 
-    for (int it = 0; it < niter; it++) {
-        const int t = it * S + grp;
-        const int j0 = j_begin + t * PF32_BN;
-        const bool have = t < ntiles;
-        lds_barrier();  // everyone finished reading the previous tile (LDS-only barrier: the prefetch
-        if (have) store_tile();  // issued below stays in flight across the math)
-        lds_barrier();
-        if (t + S < ntiles) load_tile(j0 + S * PF32_BN);
-
-        const bool tile_visible = have && wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;
-        if (!tile_visible) continue;
-
+    // One tile's math: S^T from the K image at the start of the group's buffer, online softmax, then `between`
+    // (how the single-wavefront form swaps V into the buffer), then O^T += V^T . P^T from the V image at `voff`.
+    auto tile_math = [&](int j0, int voff, auto &&between) __attribute__((always_inline)) {
         float bias[BIAS ? 16 : 1];
         if constexpr (BIAS) {  // requested before the matrix work that hides their latency
 #pragma unroll
@@ -243,15 +217,97 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 #pragma unroll
             for (int r = 0; r < 16; r++) o[db][r] *= corr;
 
+        between();
+
         // O^T += V^T . P^T: contraction step r pairs this half-wave's key 8 (r/4) + 4 h2 + r%4
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int krow = 8 * (r >> 2) + 4 * h2 + (r & 3);
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
-                const float a = *LDS32_PTR(float, gbase + K_BYTES + krow * KP + (32 * db + ln) * 4);
+                const float a = *LDS32_PTR(float, gbase + voff + krow * KP + (32 * db + ln) * 4);
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db], 0, 0, 0);
             }
+        }
+    };
+
+    if constexpr (SOLO) {
+        // this wavefront's own tiles: those of its group (t % S == grp) among the tiles its rows see
+        int ta = 0, tb = 0;
+        if (wave_has_rows && hi_w > lo_w) {
+            ta = (lo_w - j_begin) / PF32_BN;
+            tb = min(ntiles, (hi_w - j_begin + PF32_BN - 1) / PF32_BN);
+        }
+        float4_t st[NCH];
+        auto load_rows = [&](const T *base, int64_t stride, int j0) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int cid = lane + 64 * i;
+                const int row = cid / CPR, col = cid % CPR;
+                const int key = min(j0 + row, p.Skv - 1);
+                st[i] = col * 4 < p.D ? load4(base + (int64_t)key * stride + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        };
+        auto store_rows = [&]() __attribute__((always_inline)) {
+            wave_lds_sync();  // the reads of the image being replaced are done
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int cid = lane + 64 * i;
+                *LDS32_PTR(float4_t, gbase + (cid / CPR) * KP + (cid % CPR) * 16) = st[i];
+            }
+            wave_lds_sync();
+        };
+        int t = ta + ((grp - ta) % S + S) % S;
+        if (t < tb) load_rows(kg, p.ks[2], j_begin + t * PF32_BN);
+        for (; t < tb; t += S) {
+            const int j0 = j_begin + t * PF32_BN;
+            store_rows();                  // K(t)
+            load_rows(vg, p.vs[2], j0);    // V(t) arrives during S^T
+            tile_math(j0, 0, [&]() __attribute__((always_inline)) {
+                store_rows();              // V(t) replaces K(t)
+                if (t + S < tb) load_rows(kg, p.ks[2], j0 + S * PF32_BN);  // K of the next tile arrives during P.V
+            });
+        }
+    } else {
+        float4_t kst[NCH], vst[NCH];
+        auto load_tile = [&](int j0) {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int cid = gtid + GT * i;
+                const int row = cid / CPR, col = cid % CPR;
+                const int key = min(j0 + row, p.Skv - 1);
+                const bool in_row = col * 4 < p.D;  // a head_dim below D is padded with zeros
+                kst[i] = in_row ? load4(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+                vst[i] = in_row ? load4(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        };
+        auto store_tile = [&]() {
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const int cid = gtid + GT * i;
+                const int row = cid / CPR, col = cid % CPR;
+                *LDS32_PTR(float4_t, gbase + row * KP + col * 16) = kst[i];
+                *LDS32_PTR(float4_t, gbase + K_BYTES + row * KP + col * 16) = vst[i];
+            }
+        };
+
+        // group g takes the tiles j_begin + (it * S + g) * 32; every group runs the same number of iterations
+        // (the barriers are workgroup-wide), a group without a tile in the last one idles through it
+        const int niter = (ntiles + S - 1) / S;
+        if (grp < ntiles) load_tile(j_begin + grp * PF32_BN);
+
+        for (int it = 0; it < niter; it++) {
+            const int t = it * S + grp;
+            const int j0 = j_begin + t * PF32_BN;
+            const bool have = t < ntiles;
+            lds_barrier();  // everyone finished reading the previous tile (LDS-only barrier: the prefetch
+            if (have) store_tile();  // issued below stays in flight across the math)
+            lds_barrier();
+            if (t + S < ntiles) load_tile(j0 + S * PF32_BN);
+
+            const bool tile_visible = have && wave_has_rows && j0 < hi_w && j0 + PF32_BN > lo_w;
+            if (!tile_visible) continue;
+            tile_math(j0, K_BYTES, []() {});
         }
     }
 
@@ -259,7 +315,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         // merge the groups: groups 1.. park (m, l, O) in LDS, one value per lane and register, group 0
         // folds them into its own state (log-sum-exp merge, as the split-KV combine does)
         constexpr int NR = 16 * (D / 32) + 2;            // registers per lane
-        static_assert((S - 1) * WPG * NR * 256 <= S * 2 * K_BYTES, "merge staging exceeds the tile buffers");
+        static_assert((S - 1) * WPG * NR * 256 <= S * G_BYTES, "merge staging exceeds the tile buffers");
         lds_barrier();  // the tile buffers are free
         if (grp > 0) {
             const int slot = ((grp - 1) * WPG + wig) * NR * 256 + lane * 4;
@@ -627,10 +683,10 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
         case 32: hipLaunchKernelGGL((prefill_f32_kernel<T, 32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 64: hipLaunchKernelGGL((prefill_f32_kernel<T, 64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
         case 96:
-            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4)) hipLaunchKernelGGL((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         case 128:
-            if constexpr (S <= (BIAS ? 1 : 2)) hipLaunchKernelGGL((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4)) hipLaunchKernelGGL((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, 0, stream, p, nqb);
             break;
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
@@ -672,14 +728,15 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
     // Split the keys of a query block over 2 or 4 wavefront groups while the unsplit grid is only a few
     // workgroups per CU: the longest (last causal) query block then sets the run time, and halving it pays
     // even when every CU has work.  Measured break-even: about 4 workgroups per CU at head_dim <= 64, 2 above
-    // (the bigger tiles leave less to gain).  A single wavefront moves a whole tile only up to head_dim 64.
+    // (the bigger tiles leave less to gain).  Four groups: below two 64-row workgroups per CU at head_dim <= 64;
+    // above, where each wavefront moves its tiles alone, up to one per CU.
     const int cus = p.cus > 0 ? p.cus : 256;
     const long bh = (long)p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     const long wg1 = bh * ((p.Sq + 127) / 128), wg2 = bh * ((p.Sq + 63) / 64);
     const bool small_dim = p.D <= 64;
     int split = 1;
     if (wg1 <= (small_dim ? 4L : 2L) * cus) split = 2;
-    if (split == 2 && small_dim && wg2 < 2L * cus) split = 4;
+    if (split == 2 && (small_dim ? wg2 < 2L * cus : (wg2 < cus || (wg2 == cus && p.Skv >= 256)))) split = 4;
     if (sizeof(T) != 4) split = 1;
     // a mask tensor without its interval form is added element by element (the 16 bias registers leave no
     // room for the key-split form at head_dim 96 / 128)

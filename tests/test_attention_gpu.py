@@ -216,8 +216,12 @@ def test_prefill_tiled(device, dtype, D, case):
     (32, 1, 6, 333, 333, None, "four groups, no mask"),
     (64, 2, 32, 700, 700, (True, 0, 0), "two groups"),
     (64, 4, 48, 900, 900, (True, 0, 300), "one group"),
-    (128, 1, 4, 300, 300, (True, 0, 0), "two groups"),
-    (96, 1, 4, 161, 417, (True, 256, 0), "two groups, cached keys"),
+    (128, 1, 4, 300, 300, (True, 0, 0), "four groups of one wavefront that moves its tiles alone"),
+    (96, 1, 4, 161, 417, (True, 256, 0), "four single-wavefront groups, cached keys"),
+    (128, 1, 8, 95, 700, (True, 605, 150), "four single-wavefront groups, window and cached keys"),
+    (100, 2, 6, 333, 333, None, "four single-wavefront groups, no mask, head_dim below the tile width"),
+    (128, 1, 32, 700, 700, (True, 0, 0), "two groups"),
+    (96, 2, 16, 700, 900, (True, 200, 0), "two groups, cached keys"),
     (128, 2, 40, 1000, 1000, (True, 0, 0), "one group"),
 ])
 def test_prefill_f32_key_split_forms(device, D, B, H, Sq, Skv, analytic, form):
