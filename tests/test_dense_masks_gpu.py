@@ -133,15 +133,17 @@ def test_masks_that_are_not_intervals_fall_back(device, dtype, D, shape):
         assert np.isnan(out[0, :, r]).all() and np.isnan(ref[0, :, r]).all()
 
 
-def test_rows_without_visible_keys_and_negative_zero(device):
-    """Empty rows give NaN like the reference; -0.0 counts as zero; a one-key row works."""
-    D, Sq, Skv = 128, 70, 90
+@pytest.mark.parametrize("Skv", [90, 330])
+def test_rows_without_visible_keys_and_negative_zero(device, Skv):
+    """Empty rows give NaN like the reference; -0.0 counts as zero; a one-key row works.  (330 keys: the workgroup
+    form whose two wavefront groups merge their halves of the keys, some rows seeing keys in one half only.)"""
+    D, Sq = 128, 70
     q, k, v = _normal_qkv(24, 1, 2, 2, Sq, Skv, D)
     mask = np.full((Sq, Skv), NEG_INF, np.float32)
     for r in range(Sq):
         if r % 7 == 3:
             continue                      # nothing visible
-        lo = (r * 5) % 40
+        lo = (r * 37) % (Skv - 75)
         mask[r, lo:lo + 1 + r] = -0.0 if r % 2 else 0.0
     tq, tk, tv, tm = _tensors(device, fa.F16, q, k, v, mask)
     out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
