@@ -496,8 +496,8 @@ int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes) {
         return FHIP_ERR_INVALID_ARG;
     }
     if (!bytes) return FHIP_OK;
-    FHIP_HIP_CHECK(hipMemsetAsync(dst, value, bytes, s->s));
-    return FHIP_OK;
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return launch_fill_bytes(dst, value, bytes, s->s);  // a kernel, not a memset node: safe to record into a graph
 }
 
 // ---- stream capture: a sequence of calls recorded once and replayed with one launch --------------------

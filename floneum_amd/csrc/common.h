@@ -92,6 +92,7 @@ size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream);
 int launch_fill_zero_bytes(void *dst, size_t bytes, hipStream_t stream);
+int launch_fill_bytes(void *dst, int value, size_t bytes, hipStream_t stream);
 int launch_fill_zero_rows(void *dst, const int64_t dstride[4], const uint32_t shape[4], int elem_bytes,
                           hipStream_t stream);
 

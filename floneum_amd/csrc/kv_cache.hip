@@ -119,6 +119,29 @@ int launch_fill_zero_bytes(void *dst, size_t bytes, hipStream_t stream) {
     return FHIP_OK;
 }
 
+// memset by a kernel: unaligned head and tail byte by byte, the body in 16-byte stores
+__global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *dst, size_t bytes, unsigned char value, size_t head,
+                                                         size_t vecs) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, nthreads = (size_t)gridDim.x * 256;
+    const uint32_t w = value * 0x01010101u;
+    uint4 *body = (uint4 *)(dst + head);
+    for (size_t i = tid; i < vecs; i += nthreads) body[i] = make_uint4(w, w, w, w);
+    const size_t tail0 = head + vecs * 16;
+    for (size_t i = tid; i < head; i += nthreads) dst[i] = value;
+    for (size_t i = tail0 + tid; i < bytes; i += nthreads) dst[i] = value;
+}
+
+int launch_fill_bytes(void *dst, int value, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return FHIP_OK;
+    size_t head = (16 - ((uintptr_t)dst & 15)) & 15;
+    if (head > bytes) head = bytes;
+    const size_t vecs = (bytes - head) / 16;
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(grid_for((int64_t)(vecs > 256 ? vecs : 256))), dim3(256), 0, stream,
+                       (unsigned char *)dst, bytes, (unsigned char)value, head, vecs);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream) {
     return copy_or_zero(src, sstride, dst, dstride, shape, elem_bytes, false, stream);

@@ -170,7 +170,7 @@ int fhip_free(fhip_device *dev, void *ptr);
 int fhip_memcpy_h2d(fhip_stream *s, void *dst, const void *src, size_t bytes);
 int fhip_memcpy_d2h(fhip_stream *s, void *dst, const void *src, size_t bytes); /* synchronises */
 int fhip_memcpy_d2d(fhip_stream *s, void *dst, const void *src, size_t bytes);
-int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes);
+int fhip_memset(fhip_stream *s, void *dst, int value, size_t bytes); /* a fill kernel: may be recorded into a graph */
 
 /* Stream capture.  A decode step is a handful of short launches (rope, cache write, attention, merge), so a
  * serving loop is bound by launch cost; everything this library queues between begin and end is recorded

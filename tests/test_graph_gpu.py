@@ -99,3 +99,40 @@ def test_masked_prefill_replayed(device):
         ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk")
         assert_parity(got, ref, TOL_F32, f"replay {it}")
         _ = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()   # unrelated eager work between the replays
+
+
+def test_memset_is_a_kernel_and_replays(device):
+    """fhip_memset at odd addresses and sizes, eagerly and recorded into a graph that is replayed over dirtied memory
+    (a memset node in a captured graph is not reliable on these machines; the library fills with a kernel)."""
+    L = fa.lib()
+    n = 5000
+    buf = fa.Buffer(device, n)
+    host = np.empty(n, np.uint8)
+
+    def dirty():
+        src = np.full(n, 0xEE, np.uint8)
+        fa.check(L.fhip_memcpy_h2d(device.stream, ctypes.c_void_p(buf.ptr), src.ctypes.data_as(ctypes.c_void_p), n))
+
+    def read():
+        fa.check(L.fhip_memcpy_d2h(device.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(buf.ptr), n))
+        return host.copy()
+
+    cases = [(0, n, 0x00), (1, 1, 0x7F), (3, 11, 0xAB), (13, 4099, 0x01), (16, 4096, 0xFF), (7, 0, 0x55), (4990, 10, 0x33)]
+    for off, size, val in cases:
+        dirty()
+        fa.check(L.fhip_memset(device.stream, ctypes.c_void_p(buf.ptr + off), val, size))
+        want = np.full(n, 0xEE, np.uint8)
+        want[off:off + size] = val
+        assert np.array_equal(read(), want), (off, size, val)
+
+    with device.capture() as cap:
+        for off, size, val in cases[1:5]:
+            fa.check(L.fhip_memset(device.stream, ctypes.c_void_p(buf.ptr + off), val, size))
+    want = np.full(n, 0xEE, np.uint8)
+    for off, size, val in cases[1:5]:
+        want[off:off + size] = val
+    for _ in range(3):
+        dirty()
+        device.synchronize()
+        cap.graph.launch()
+        assert np.array_equal(read(), want)
