@@ -77,6 +77,12 @@ template <typename T, int D, int S, bool BIAS>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnParams p, int nqb) {
     constexpr int WPG = PF32_WAVES / S;   // wavefronts per key-split group
     constexpr int BM = 32 * WPG;          // query rows per workgroup
+    // Which head dims a 32-row block of O^T holds.  With 2 or 4 blocks, row i of block db is dim NDB i + db: the
+    // V operands of all blocks for one key then sit side by side and one 8- or 16-byte LDS read feeds NDB matrix
+    // instructions (a 4-byte read per instruction leaves a lone wavefront waiting on LDS latency most of the time).
+    constexpr int NDB = D / 32;
+    constexpr bool PACKED = (NDB == 2 || NDB == 4);
+    auto dim_of = [](int db, int i) __attribute__((always_inline)) { return PACKED ? NDB * i + db : 32 * db + i; };
     constexpr int KP = D * 4 + 16;  // row pitch in bytes: rows 4 banks apart -> conflict-free b128 reads
     constexpr int K_BYTES = PF32_BN * KP;
     constexpr int CPR = D / 4;      // 16-byte chunks per row
@@ -159,6 +165,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 
     const int j_begin = (lo_wg / PF32_BN) * PF32_BN;
     const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PF32_BN - 1) / PF32_BN : 0;
+    // a thread's chunks of a tile are a fixed number of rows apart when its group's threads cover whole rows
+    constexpr bool AFFINE = (GT % CPR == 0);
+    constexpr int RSTEP = AFFINE ? GT / CPR : 0;
+    const bool whole_rows = p.D == D;
 
     // One tile's math: S^T from the K image at the start of the group's buffer, online softmax, then `between`
     // (how the single-wavefront form swaps V into the buffer), then O^T += V^T . P^T from the V image at `voff`.
@@ -223,10 +233,21 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int krow = 8 * (r >> 2) + 4 * h2 + (r & 3);
+            if constexpr (NDB == 4) {
+                const float4_t a = *LDS32_PTR(float4_t, gbase + voff + krow * KP + ln * 16);
 #pragma unroll
-            for (int db = 0; db < D / 32; db++) {
-                const float a = *LDS32_PTR(float, gbase + voff + krow * KP + (32 * db + ln) * 4);
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db], 0, 0, 0);
+                for (int db = 0; db < 4; db++) o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[db], s[r], o[db], 0, 0, 0);
+            } else if constexpr (NDB == 2) {
+                typedef float float2_t __attribute__((ext_vector_type(2)));
+                const float2_t a = *LDS32_PTR(float2_t, gbase + voff + krow * KP + ln * 8);
+#pragma unroll
+                for (int db = 0; db < 2; db++) o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[db], s[r], o[db], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int db = 0; db < NDB; db++) {
+                    const float a = *LDS32_PTR(float, gbase + voff + krow * KP + (32 * db + ln) * 4);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db], 0, 0, 0);
+                }
             }
         }
     };
@@ -240,6 +261,15 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         }
         float4_t st[NCH];
         auto load_rows = [&](const T *base, int64_t stride, int j0) __attribute__((always_inline)) {
+            if (AFFINE && whole_rows && j0 + PF32_BN <= p.Skv) {
+                // a tile inside the key axis with rows as wide as the kernel's: one address per thread, the
+                // chunks a fixed number of rows apart, no clamp and no branch per chunk
+                const T *p0 = base + (int64_t)(j0 + lane / CPR) * stride + (lane % CPR) * 4;
+                const int64_t step = (int64_t)RSTEP * stride;
+#pragma unroll
+                for (int i = 0; i < NCH; i++) st[i] = load4(p0 + i * step);
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
                 const int cid = lane + 64 * i;
@@ -271,6 +301,17 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     } else {
         float4_t kst[NCH], vst[NCH];
         auto load_tile = [&](int j0) {
+            if (AFFINE && whole_rows && j0 + PF32_BN <= p.Skv) {  // see load_rows above
+                const T *pk = kg + (int64_t)(j0 + gtid / CPR) * p.ks[2] + (gtid % CPR) * 4;
+                const T *pv = vg + (int64_t)(j0 + gtid / CPR) * p.vs[2] + (gtid % CPR) * 4;
+                const int64_t kstep = (int64_t)RSTEP * p.ks[2], vstep = (int64_t)RSTEP * p.vs[2];
+#pragma unroll
+                for (int i = 0; i < NCH; i++) {
+                    kst[i] = load4(pk + i * kstep);
+                    vst[i] = load4(pv + i * vstep);
+                }
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < NCH; i++) {
                 const int cid = gtid + GT * i;
@@ -354,7 +395,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                    const int dim = dim_of(db, 8 * (r >> 2) + 4 * h2 + (r & 3));
                     if (dim < p.D) ws[dim] = o[db][r];
                 }
             if (h2 == 0) {
@@ -370,7 +411,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int dim = 32 * db + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                const int dim = dim_of(db, 8 * (r >> 2) + 4 * h2 + (r & 3));
                 if (dim < p.D) store_out<T>(p, ob + dim * p.os[3], o[db][r] / l_tot);  // no visible key: 0/0 = NaN like the reference
             }
     }
