@@ -14,7 +14,7 @@
 //     products on v_dot2, DPP reductions; every group of LPK lanes keeps its own softmax state.
 // Both keep (m, l, acc) in the log2 domain, merge lanes -> wavefront -> workgroup at the end and
 // write one partial (acc[D], m, l) per (batch, head, split).
-// Pass 2 (decode_combine_kernel): log-sum-exp merge of the partials of each (batch, head).
+// Pass 2 (decode_combine_kernel, decode_combine4_kernel): log-sum-exp merge of the partials of each (batch, head).
 // With a single split pass 1 writes the final output and pass 2 is not launched.
 //
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199 (f32 accumulation
@@ -689,11 +689,98 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
     }
 }
 
+// Few (batch, head) rows with many splits (batch 1 on a long cache): one wavefront per row leaves the chip empty
+// and issues every load of a row from 64 lanes.  Here four wavefronts share a row, each merges a quarter of the
+// splits (U in flight per lane), and the first folds the four states through LDS.
+template <typename T, int U>
+__global__ __launch_bounds__(256) void decode_combine4_kernel(AttnParams p) {
+    __shared__ float part[4][2 + 128];
+    const int bh = blockIdx.x;
+    const int h = bh % p.H, b = bh / p.H;
+    const int D = p.D;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int ns = p.nsplit;
+    if (p.kv_lens) {
+        const int len = min(p.Skv, max(p.kv_lens[b], 0));
+        ns = max(1, min(ns, (len + p.chunk - 1) / p.chunk));  // split 0 is always written
+    }
+    const float *ws = (const float *)p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
+    const int64_t ob = b * p.os[0] + h * p.os[1];
+    const int per = (ns + 3) / 4, s_lo = wave * per, s_hi = min(ns, s_lo + per);
+    for (int dbase = 0; dbase < D; dbase += 128) {
+        const int d0 = dbase + lane, d1 = dbase + lane + 64;
+        float M = -INFINITY, L = 0.0f, A0 = 0.0f, A1 = 0.0f;
+        for (int s0 = s_lo; s0 < s_hi; s0 += U) {
+            float ms[U], ls[U], a0[U], a1[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const bool ok = s0 + u < s_hi;
+                const float *src = ws + (int64_t)(ok ? s0 + u : s0) * (D + 2);
+                ms[u] = ok ? src[D] : -INFINITY;
+                ls[u] = ok ? src[D + 1] : 0.0f;
+                a0[u] = (ok && d0 < D) ? src[d0] : 0.0f;
+                a1[u] = (ok && d1 < D) ? src[d1] : 0.0f;
+            }
+            float Mn = M;
+#pragma unroll
+            for (int u = 0; u < U; u++) Mn = fmaxf(Mn, ms[u]);
+            const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+            const float c = __builtin_amdgcn_exp2f(M - Ms);
+            L *= c;
+            A0 *= c;
+            A1 *= c;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
+                L += w * ls[u];
+                A0 += w * a0[u];
+                A1 += w * a1[u];
+            }
+            M = Mn;
+        }
+        if (dbase > 0) __syncthreads();  // the previous round's states have been read
+        part[wave][2 + lane] = A0;
+        part[wave][2 + 64 + lane] = A1;
+        if (lane == 0) {
+            part[wave][0] = M;
+            part[wave][1] = L;
+        }
+        __syncthreads();
+        if (wave == 0) {
+            float Mn = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < 4; w++) Mn = fmaxf(Mn, part[w][0]);
+            const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+            float Lt = 0.0f, B0 = 0.0f, B1 = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const float c = __builtin_amdgcn_exp2f(part[w][0] - Ms);
+                Lt += c * part[w][1];
+                B0 += c * part[w][2 + lane];
+                B1 += c * part[w][2 + 64 + lane];
+            }
+            if (d0 < D) {
+                const float val = B0 / Lt;  // no visible key: 0/0 = NaN like the reference
+                if (p.out_f32) ((float *)p.out)[ob + d0 * p.os[3]] = val;
+                else ((T *)p.out)[ob + d0 * p.os[3]] = from_float<T>(val);
+            }
+            if (d1 < D) {
+                const float val = B1 / Lt;
+                if (p.out_f32) ((float *)p.out)[ob + d1 * p.os[3]] = val;
+                else ((T *)p.out)[ob + d1 * p.os[3]] = from_float<T>(val);
+            }
+        }
+    }
+}
+
 template <typename T>
 static void launch_combine(const AttnParams &p, hipStream_t stream) {
     const dim3 grid((unsigned)(p.B * p.H)), block(64);
+    const int cus = p.cus > 0 ? p.cus : 256;
     if (p.nsplit <= 8) hipLaunchKernelGGL((decode_combine_kernel<T, 8>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((decode_combine_kernel<T, 32>), grid, block, 0, stream, p);
+    else if ((long)p.B * p.H > 2L * cus) hipLaunchKernelGGL((decode_combine_kernel<T, 32>), grid, block, 0, stream, p);
+    else if (p.nsplit <= 32) hipLaunchKernelGGL((decode_combine4_kernel<T, 8>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((decode_combine4_kernel<T, 16>), grid, dim3(256), 0, stream, p);
 }
 
 template <typename T, int LPK>
