@@ -401,6 +401,27 @@ def test_decode_f32_with_the_masks_the_reference_passes(device):
     assert_parity(out, oracle.flash_attention(q, k, v, D ** -0.5), TOL_F32, "f32 decode, cache views")
 
 
+@pytest.mark.parametrize("dtype,B,H,Hkv,D,Skv", [(fa.F16, 1, 8, 2, 128, 6000), (fa.F32, 1, 4, 2, 256, 5200),
+                                                  (fa.F32, 2, 6, 3, 64, 9000), (fa.BF16, 3, 4, 1, 96, 7000)])
+def test_decode_with_many_splits_and_few_rows(device, dtype, B, H, Hkv, D, Skv):
+    """One chat stream on a long cache: tens of splits per (batch, head) row and only a few rows, which the combine
+    pass handles with four wavefronts per row (two rounds of 128 dims at head_dim 256); ragged lengths on top."""
+    q, k, v = _normal_qkv(31, B, H, Hkv, 1, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+    out = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5)
+    assert_parity(out, ref, tol, "all keys")
+    lens = np.array([Skv - 7, 300, 4097][:B], np.int32)
+    out = tq.flash_attention(tk, tv, D ** -0.5, kv_lens=fa.IntTensor(device, lens)).to_numpy()
+    for b in range(B):
+        n = int(lens[b])
+        ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                     rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+        assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
+
+
 def test_decode_ragged_kv_lens(device):
     # per-sequence lengths == un-padded calls == -inf BatchKeyMask padding
     B, H, Hkv, D, Smax = 5, 4, 4, 96, 3000
