@@ -235,7 +235,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                            __attribute__((always_inline)) {
         // (uniform values; pinned to scalar registers, which is what the instruction takes)
         const int soff = __builtin_amdgcn_readfirstlane(min(j_begin + tile * PF_BN, p.Skv) * row_bytes);
-        lbase = __builtin_amdgcn_readfirstlane(lbase);
+        // M0 takes an LDS address, not an offset into the tile buffers (they are the kernel's only LDS variable and
+        // start at 0, which the compiler folds in)
+        lbase = __builtin_amdgcn_readfirstlane(lbase + (int)(uint32_t)(uintptr_t)lds_base);
         if (C::LOAD_LANES == 64 || lane < C::LOAD_LANES) {
             // written as assembly on purpose: the compiler would otherwise make every later LDS read
             // of this wavefront wait for these loads, whose data is not due before the next barrier
