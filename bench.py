@@ -50,6 +50,11 @@ def configs():
                    q_pos_offset=8064),
         "T2": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=128, Skv=8192, D=128, dtype="f16", std=1.0, causal=True,
                    q_pos_offset=8064),
+        # not headline configurations either: one chat stream, i.e. a batch-1 decode step on 4096 cached keys in the
+        # reference's f32 and in f16, and in f16 on 32768 keys (latency-bound: two dependent launches)
+        "S1": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
+        "S2": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
+        "S3": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=32768, D=128, dtype="f16", std=0.5, causal=False),
     }
 
 
