@@ -57,7 +57,15 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // few (batch, kv head) units, e.g. batch 1: down to one workgroup step of 128 keys per split, because a
     // workgroup's steps run one after the other and each costs a memory latency.  Up to 256 keys the matrix-core
     // variant is quicker unsplit than with a second launch to merge two splits (measured 6.6 vs 8.6 us).
-    const int min_chunk = 128;
+    // (the vector variant's step is 16 rows of 64 / LPK keys: 64 keys at head_dim 128 in f32, where one step
+    // per workgroup is one memory round trip less than two)
+    int step_keys = 128;
+    if (!decode_use_mfma(D, f32)) {
+        const int lpk = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
+        step_keys = 16 * (64 / lpk);
+        if (step_keys > 128) step_keys = 128;
+    }
+    const int min_chunk = step_keys;
     long ns = (target + units - 1) / units;
     const long ns_max = (Skv + min_chunk - 1) / min_chunk;
     const long ns_min = (Skv + max_chunk - 1) / max_chunk;
@@ -65,7 +73,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     if (ns < ns_min) ns = ns_min;
     if (ns < 1 || (Skv <= 256 && decode_use_mfma(D, f32))) ns = 1;
     long c = (Skv + ns - 1) / ns;
-    c = (c + 127) / 128 * 128;  // a workgroup step covers 128 keys
+    c = (c + step_keys - 1) / step_keys * step_keys;  // whole workgroup steps
     *chunk = (int)c;
     *nsplit = (int)((Skv + c - 1) / c);
 }
