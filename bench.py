@@ -42,6 +42,10 @@ def configs():
         # mask is get_mask(512, 16384, Some(4096)) = 3584 visible columns + a causal 512x512 block
         "C4": dict(kind="prefill", B=4, H=32, Hkv=8, Sq=512, Skv=4096, D=128, dtype="f16", std=1.0, causal=True,
                    q_pos_offset=3584, window=4096),
+        # absolute-position form of the same chunk (not a parity claim against the reference's truncating cache): the
+        # whole 16896-key cache is passed and the analytic window leaves every query exactly 4096 keys
+        "C4B": dict(kind="prefill", B=4, H=32, Hkv=8, Sq=512, Skv=16896, D=128, dtype="f16", std=1.0, causal=True,
+                    q_pos_offset=16384, window=4096),
         "C5": dict(kind="decode", B=32, H=32, Hkv=32, Sq=1, Skv=32768, D=96, dtype="f16", std=1.0, causal=False,
                    ragged=(128, 32768)),
         # not a headline configuration: a new chat turn, 128 query rows on 8192 cached keys (the shape at which the
