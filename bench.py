@@ -320,6 +320,7 @@ def run_config(name, steps, warmup, with_cpu=True):
     roof["kernel"] = kernel
     roof["kernel_ms_mean"] = main_ms_mean
     roof["kernel_ms_median"] = main_ms_med
+    roof["kernel_ms_min"] = float(main_ms.min())
     roof["kernel_ms_events_raw"] = main_ms_raw
     roof["event_pair_empty_ms"] = empty_ms
     roof["call_ms_events"] = call_ms
