@@ -54,6 +54,9 @@ def configs():
                    q_pos_offset=8064),
         "T2": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=128, Skv=8192, D=128, dtype="f16", std=1.0, causal=True,
                    q_pos_offset=8064),
+        # short prompts (latency-bound grids that do not fill the chip): 1024 tokens in f16, 512 tokens in f32
+        "P1": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=1024, Skv=1024, D=128, dtype="f16", std=1.0, causal=True),
+        "P2": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=128, dtype="f32", std=1.0, causal=True),
         # not headline configurations either: one chat stream, i.e. a batch-1 decode step on 4096 cached keys in the
         # reference's f32 and in f16, and in f16 on 32768 keys (latency-bound: two dependent launches)
         "S1": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
