@@ -201,6 +201,28 @@ def test_workspace_bytes():
     assert L.fhip_flash_attention(None, ctypes.byref(a)) == fa.ERR_INVALID_ARG
 
 
+def test_decode_split_planning_on_256_cus():
+    """How many key splits the planner asks a workspace for (partials of D + 2 floats per (batch, head, split)):
+    1024-key chunks for a batch that fills the chip, down to one workgroup step per split for one chat stream
+    (128 keys for the matrix-core variant, 64 for the vector variant at head_dim 128), unsplit up to 256 keys."""
+    need = ctypes.c_size_t()
+    L = fa.lib()
+
+    def splits(B, H, Hkv, Skv, D, dtype):
+        a = make_args(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D, dtype=dtype)
+        assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
+        per = B * H * (D + 2) * 4
+        assert need.value % per == 0
+        return need.value // per
+
+    assert splits(16, 32, 8, 4096, 128, fa.F16) == 4     # C2
+    assert splits(1, 32, 8, 4096, 128, fa.F16) == 32     # one stream, 128-key steps
+    assert splits(1, 32, 8, 32768, 128, fa.F16) == 64
+    assert splits(1, 32, 8, 4096, 128, fa.F32) == 64     # vector variant: 64-key steps
+    assert splits(1, 32, 8, 1024, 128, fa.F32) == 16
+    assert splits(1, 32, 8, 256, 128, fa.F16) == 0       # unsplit: no partials, no second launch
+
+
 # ---- masks: bit-exact against the checker and the reference's vectors -----------------------------------
 
 NEG_BITS = {fa.F32: 0xFF800000, fa.F16: 0xFC00, fa.BF16: 0xFF80}
