@@ -223,6 +223,28 @@ def test_decode_split_planning_on_256_cus():
     assert splits(1, 32, 8, 256, 128, fa.F16) == 0       # unsplit: no partials, no second launch
 
 
+def test_prefill_key_split_planning_on_256_cus():
+    """Few query rows on a long cache: the keys are split over workgroups (partials of D + 2 floats per row and share
+    for the f32-arithmetic kernel, D + 4 for the 16-bit one); a square causal prompt is not split."""
+    need = ctypes.c_size_t()
+    L = fa.lib()
+
+    def shares(Sq, Skv, dtype, pitch, analytic=True):
+        a = make_args(B=1, H=32, Hkv=8, Sq=Sq, Skv=Skv, D=128, dtype=dtype)
+        if analytic:
+            a.analytic.enabled, a.analytic.causal, a.analytic.q_pos_offset = 1, 1, Skv - Sq
+        assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
+        per = 32 * Sq * pitch * 4
+        assert need.value % per == 0
+        return need.value // per
+
+    assert shares(128, 8192, fa.F32, 130) == 4    # a new chat turn: 4 query blocks x 32 heads x 4 shares of 2048 keys
+    assert shares(128, 8192, fa.F16, 132) == 8    # one 128-row block per head x 8 shares of 1024 keys
+    assert shares(32, 32768, fa.F16, 132) == 16
+    assert shares(512, 512, fa.F32, 130) == 0     # square causal prompts are left alone
+    assert shares(2048, 2048, fa.F16, 132) == 0
+
+
 # ---- masks: bit-exact against the checker and the reference's vectors -----------------------------------
 
 NEG_BITS = {fa.F32: 0xFF800000, fa.F16: 0xFC00, fa.BF16: 0xFF80}
