@@ -221,6 +221,7 @@ class Device:
         self.arch = info.arch.decode()
         self._workspace = None
         self._workspace_bytes = 0
+        self._pool, self._sizes, self._pooled = {}, {}, 0  # cached free blocks by size, block sizes, bytes cached
 
     @classmethod
     def default(cls):
@@ -234,13 +235,39 @@ class Device:
         rc = lib().fhip_device_count(ctypes.byref(n))
         return n.value if rc == OK else 0
 
+    # Freed blocks are kept by size and handed out again, as the reference's device keeps an allocation cache
+    # (fusor-ml/core/src/device.rs:305-354): hipMalloc / hipFree cost tens of microseconds and hipFree waits for
+    # the device.  Safe because this object has a single stream: a reused block is only touched by work queued
+    # after the work of its previous owner.
+    _CACHE_LIMIT = 1 << 30
+
     def malloc(self, nbytes):
+        size = (max(int(nbytes), 1) + 255) & ~255
+        free_list = self._pool.get(size)
+        if free_list:
+            self._pooled -= size
+            return free_list.pop()
         p = ctypes.c_void_p()
-        check(lib().fhip_malloc(self.handle, nbytes, ctypes.byref(p)))
+        check(lib().fhip_malloc(self.handle, size, ctypes.byref(p)))
+        self._sizes[p.value] = size
         return p.value
 
     def free(self, ptr):
+        size = self._sizes.get(ptr)
+        if size is not None and self._pooled + size <= self._CACHE_LIMIT:
+            self._pool.setdefault(size, []).append(ptr)
+            self._pooled += size
+            return
+        self._sizes.pop(ptr, None)
         check(lib().fhip_free(self.handle, ctypes.c_void_p(ptr)))
+
+    def release_cached_memory(self):
+        """Give the cached blocks back to the driver."""
+        for ptrs in self._pool.values():
+            for ptr in ptrs:
+                self._sizes.pop(ptr, None)
+                check(lib().fhip_free(self.handle, ctypes.c_void_p(ptr)))
+        self._pool, self._pooled = {}, 0
 
     def synchronize(self):
         check(lib().fhip_stream_synchronize(self.stream))
