@@ -49,8 +49,19 @@ __global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const cha
         // contiguous, 16-byte aligned rows: 16 bytes per lane and step
         constexpr int EPV = 16 / EB;
         const int nvec = cols / EPV;
-        for (int c = lane; c < nvec; c += 64) {
-            const uint4_t raw = __builtin_nontemporal_load((const uint4_t *)(mrow) + c);
+        // a piece that is all -inf or all zero (nearly every piece of a real mask) is settled with four word
+        // compares; four pieces are in flight per lane
+        const uint32_t ninf_word = EB == 4 ? 0xFF800000u : (ninf16 | (ninf16 << 16));
+        const uint32_t abs_word = EB == 4 ? 0x7FFFFFFFu : 0x7FFF7FFFu;
+        auto take_piece = [&](int c, const uint4_t raw) {
+            const bool all_ninf = raw[0] == ninf_word && raw[1] == ninf_word && raw[2] == ninf_word && raw[3] == ninf_word;
+            if (all_ninf) return;
+            if (((raw[0] | raw[1] | raw[2] | raw[3]) & abs_word) == 0) {
+                lo = min(lo, c * EPV);
+                hi = max(hi, c * EPV + EPV);
+                zeros += EPV;
+                return;
+            }
 #pragma unroll
             for (int e = 0; e < EPV; e++) {
                 uint32_t bits;
@@ -58,7 +69,16 @@ __global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const cha
                 else bits = (raw[e >> 1] >> (16 * (e & 1))) & 0xffffu;
                 take(c * EPV + e, bits);
             }
+        };
+        int c = lane;
+        for (; c + 192 < nvec; c += 256) {
+            uint4_t raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) raw[u] = __builtin_nontemporal_load((const uint4_t *)(mrow) + c + 64 * u);
+#pragma unroll
+            for (int u = 0; u < 4; u++) take_piece(c + 64 * u, raw[u]);
         }
+        for (; c < nvec; c += 64) take_piece(c, __builtin_nontemporal_load((const uint4_t *)(mrow) + c));
         for (int j = nvec * EPV + lane; j < cols; j += 64) {
             uint32_t bits = EB == 4 ? *(const uint32_t *)(mrow + (int64_t)j * 4) : *(const uint16_t *)(mrow + (int64_t)j * 2);
             take(j, bits);
