@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <new>
 
 #include "common.h"
@@ -732,6 +733,8 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         // call: the f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
+        static std::atomic<uint32_t> next_tag{0x5eed0001u};
+        p.bad_tag = (int32_t)next_tag.fetch_add(1, std::memory_order_relaxed);
         rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
         if (rc) return rc;
         AttnParams pt = p;

@@ -21,7 +21,7 @@ __global__ __launch_bounds__(64 * GEN_WAVES) void attn_generic_kernel(AttnParams
     const int64_t row = (int64_t)blockIdx.x * GEN_WAVES + wave;
     const int64_t total = (int64_t)p.B * p.H * p.Sq;
     if (row >= total) return;  // whole wavefront leaves together; no workgroup barrier is used below
-    if (p.only_if_bad && *p.only_if_bad == 0) return;  // a tiled kernel has taken this call
+    if (p.only_if_bad && *p.only_if_bad != p.bad_tag) return;  // a tiled kernel has taken this call
     const int i = (int)(row % p.Sq);
     const int h = (int)((row / p.Sq) % p.H);
     const int b = (int)(row / ((int64_t)p.Sq * p.H));

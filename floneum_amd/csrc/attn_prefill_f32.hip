@@ -99,9 +99,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     if constexpr (BIAS) {
-        if (p.only_if_bad && *p.only_if_bad == 0) return;  // the interval form of the mask has served the call
+        if (p.only_if_bad && *p.only_if_bad != p.bad_tag) return;  // the interval form of the mask has served the call
     } else {
-        if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the BIAS form takes the call
+        if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the BIAS form takes the call
     }
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -426,7 +426,7 @@ __global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
     const int64_t rows = (int64_t)p.B * p.H * p.Sq;
     if (row >= rows) return;
     // the same hand-over between the interval form and the mask-adding form as in the main kernel
-    if ((p.iv_bad && *p.iv_bad != 0) || (p.only_if_bad && *p.only_if_bad == 0)) return;
+    if ((p.iv_bad && *p.iv_bad == p.bad_tag) || (p.only_if_bad && *p.only_if_bad != p.bad_tag)) return;
     const int query = (int)(row % p.Sq);
     const int h = (int)((row / p.Sq) % p.H), b = (int)(row / p.Sq / p.H);
     const int D = p.D, ns = p.pf_nsplit, pitch = p.pf_pitch;
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     __shared__ __attribute__((aligned(16))) char smem[2 * K_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
-    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
+    if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the general kernel takes the call
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;

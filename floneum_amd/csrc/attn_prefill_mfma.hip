@@ -132,7 +132,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     __shared__ __attribute__((aligned(16))) char smem[C::LDS_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
-    if (p.iv_bad && *p.iv_bad != 0) return;  // the mask is not made of intervals: the general kernel takes the call
+    if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the general kernel takes the call
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it is uniform
     const int lane = tid & 63;

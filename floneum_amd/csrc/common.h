@@ -36,6 +36,10 @@ struct AttnParams {
     const int2 *iv;
     const int32_t *iv_bad;
     const int32_t *only_if_bad;
+    // What the scan writes to *iv_bad when a row is not of that form: a value unique to the call, so that the word
+    // needs no clearing beforehand (whatever the workspace held, it is not this call's tag, short of a 2^-32
+    // coincidence that only costs the fast path).  "*iv_bad != 0" above reads "*iv_bad == bad_tag".
+    int32_t bad_tag;
     // Tiled f32 prefill only.  Workgroups are numbered longest first.  When the whole grid is resident at once
     // (two workgroups per CU) nothing is rebalanced at run time, so the second half of the numbers is walked
     // backwards: a CU's two workgroups are then a long and a short one.  0: off; else the number of CUs.

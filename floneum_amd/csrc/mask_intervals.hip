@@ -5,7 +5,7 @@
 // produce (causal, sliding window, their concatenation with a cached prefix) and every padding mask
 // has, per row, ONE run of zeros.  This kernel checks that per row and writes the run as {lo, hi}; the
 // tiled attention kernels then mask by interval and never read the [rows, kv_seq_len] tensor again.  A
-// row that is anything else (finite biases, several runs, NaN) is counted in *bad and the call falls
+// row that is anything else (finite biases, several runs, NaN) marks *bad with the call's tag and the call falls
 // back to a kernel that adds the mask values as the reference does
 // (fusor-ml/fusor/src/composite/flash_attention.rs:161-176).
 //
@@ -23,7 +23,7 @@ constexpr int MI_WAVES = 4;
 template <int EB>
 __global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const char *mask, int64_t ms0, int64_t ms1,
                                                                       int rows, int cols, uint32_t ninf16, int vec_ok,
-                                                                      int2 *iv, int32_t *bad) {
+                                                                      int2 *iv, int32_t *bad, int32_t bad_tag) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * MI_WAVES + (threadIdx.x >> 6);
     if (row >= rows) return;  // whole wavefront
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const cha
         if (hi == 0) lo = 0;  // no visible key at all: the empty interval
         const bool ok = others == 0 && zeros == hi - lo;  // only zeros and -inf, and the zeros are one run
         iv[row] = int2{lo, hi};
-        if (!ok) atomicAdd(bad, 1);
+        if (!ok) *(volatile int32_t *)bad = bad_tag;  // every such row stores the same value
     }
 }
 
@@ -110,18 +110,16 @@ size_t mask_intervals_bytes(int rows) { return ((size_t)rows * sizeof(int2) + 16
 int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32_t *bad, hipStream_t stream) {
     const int rows = p.mask_kind == FHIP_MASK_QK ? p.Sq : p.B;
     const int cols = p.Skv;
-    int rc = launch_fill_zero_bytes(bad, 16, stream);
-    if (rc) return rc;
     if (rows == 0) return FHIP_OK;
     const int eb = dtype == FHIP_F32 ? 4 : 2;
     const int vec_ok = (p.ms1 == 1 || cols <= 1) && ((uintptr_t)p.mask % 16 == 0) && ((p.ms0 * eb) % 16 == 0);
     dim3 grid((rows + MI_WAVES - 1) / MI_WAVES), block(64 * MI_WAVES);
     if (eb == 4)
         hipLaunchKernelGGL(mask_intervals_kernel<4>, grid, block, 0, stream, (const char *)p.mask, p.ms0, p.ms1, rows, cols,
-                           0u, vec_ok, iv, bad);
+                           0u, vec_ok, iv, bad, p.bad_tag);
     else
         hipLaunchKernelGGL(mask_intervals_kernel<2>, grid, block, 0, stream, (const char *)p.mask, p.ms0, p.ms1, rows, cols,
-                           dtype == FHIP_F16 ? 0xFC00u : 0xFF80u, vec_ok, iv, bad);
+                           dtype == FHIP_F16 ? 0xFC00u : 0xFF80u, vec_ok, iv, bad, p.bad_tag);
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
 }
