@@ -217,7 +217,7 @@ static bool prefill_f32_eligible(const fhip_attn_args *a) {
 }
 
 // A dense mask reaches the tiled prefill kernels in interval form (mask_intervals.hip), which needs
-// device scratch: 16 bytes for the count of rows that are not intervals, then {lo, hi} per row.
+// device scratch: 16 bytes for the mark of a mask whose rows are not all intervals, then {lo, hi} per row.
 static size_t mask_scratch_bytes(const fhip_attn_args *a) {
     if (a->mask_kind == FHIP_MASK_NONE) return 0;
     return mask_intervals_bytes(a->mask_kind == FHIP_MASK_QK ? (int)a->q.shape[2] : (int)a->q.shape[0]);
