@@ -30,15 +30,15 @@ struct AttnParams {
     hipEvent_t main_done;   // host-side only: recorded after the main kernel when not null
     // Dense additive mask reduced to intervals (see mask_intervals.hip).  iv[r] = {lo, hi}: row r of the
     // mask is 0 on keys [lo, hi) and -inf elsewhere; r is the query row (FHIP_MASK_QK) or the batch
-    // (FHIP_MASK_BATCH_KEY).  *iv_bad counts the rows that are NOT of that form.  A tiled kernel given
-    // `iv` does nothing when *iv_bad != 0; the general kernel given `only_if_bad` does nothing when
-    // *only_if_bad == 0: exactly one of the two computes the result.
+    // (FHIP_MASK_BATCH_KEY).  *iv_bad holds bad_tag when some row is NOT of that form.  A tiled kernel given
+    // `iv` does nothing when *iv_bad == bad_tag; the kernel given `only_if_bad` does nothing when
+    // *only_if_bad != bad_tag: exactly one of the two computes the result.
     const int2 *iv;
     const int32_t *iv_bad;
     const int32_t *only_if_bad;
     // What the scan writes to *iv_bad when a row is not of that form: a value unique to the call, so that the word
     // needs no clearing beforehand (whatever the workspace held, it is not this call's tag, short of a 2^-32
-    // coincidence that only costs the fast path).  "*iv_bad != 0" above reads "*iv_bad == bad_tag".
+    // coincidence that only costs the fast path).
     int32_t bad_tag;
     // Tiled f32 prefill only.  Workgroups are numbered longest first.  When the whole grid is resident at once
     // (two workgroups per CU) nothing is rebalanced at run time, so the second half of the numbers is walked
