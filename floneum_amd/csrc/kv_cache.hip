@@ -35,12 +35,13 @@ __global__ __launch_bounds__(256) void copy_rows_kernel(const char *src, char *d
     }
 }
 
-// Fully strided fallback (innermost stride != 1 on the source): one thread per element.
+// Fully strided fallback (innermost stride != 1 on either side): one thread per element.  `zero`: the destination
+// elements are cleared and `src` (null then) is never read.
 template <typename E>
 __global__ __launch_bounds__(256) void copy_elems_kernel(const E *src, E *dst, int64_t ss0, int64_t ss1, int64_t ss2,
                                                          int64_t ss3, int64_t ds0, int64_t ds1, int64_t ds2,
                                                          int64_t ds3, uint32_t n0, uint32_t n1, uint32_t n2,
-                                                         uint32_t n3) {
+                                                         uint32_t n3, bool zero) {
     const int64_t total = (int64_t)n0 * n1 * n2 * n3;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         const uint32_t i3 = (uint32_t)(i % n3);
@@ -49,7 +50,9 @@ __global__ __launch_bounds__(256) void copy_elems_kernel(const E *src, E *dst, i
         t /= n2;
         const uint32_t i1 = (uint32_t)(t % n1);
         const uint32_t i0 = (uint32_t)(t / n1);
-        dst[i0 * ds0 + i1 * ds1 + i2 * ds2 + i3 * ds3] = src[i0 * ss0 + i1 * ss1 + i2 * ss2 + i3 * ss3];
+        E val = 0;
+        if (!zero) val = src[i0 * ss0 + i1 * ss1 + i2 * ss2 + i3 * ss3];
+        dst[i0 * ds0 + i1 * ds1 + i2 * ds2 + i3 * ds3] = val;
     }
 }
 
@@ -92,11 +95,11 @@ static int copy_or_zero(const void *src, const int64_t *ss, void *dst, const int
     } else if (eb == 4) {
         hipLaunchKernelGGL(copy_elems_kernel<uint32_t>, dim3(grid_for(total_elems)), dim3(256), 0, stream,
                            (const uint32_t *)src, (uint32_t *)dst, ss[0], ss[1], ss[2], ss[3], ds[0], ds[1], ds[2],
-                           ds[3], shape[0], shape[1], shape[2], shape[3]);
+                           ds[3], shape[0], shape[1], shape[2], shape[3], zero);
     } else {
         hipLaunchKernelGGL(copy_elems_kernel<uint16_t>, dim3(grid_for(total_elems)), dim3(256), 0, stream,
                            (const uint16_t *)src, (uint16_t *)dst, ss[0], ss[1], ss[2], ss[3], ds[0], ds[1], ds[2],
-                           ds[3], shape[0], shape[1], shape[2], shape[3]);
+                           ds[3], shape[0], shape[1], shape[2], shape[3], zero);
     }
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
