@@ -32,6 +32,7 @@ KERNEL_AUTO, KERNEL_GENERIC, KERNEL_PREFILL_MFMA, KERNEL_PREFILL_F32, KERNEL_DEC
 KERNEL_NAMES = {1: "generic", 2: "prefill_mfma", 3: "prefill_f32", 4: "decode_splitkv"}
 
 OK, ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = 0, 1, 2, 3, 4
+NOALLOC_WORKSPACE_BYTES = 32 << 20  # FHIP_NOALLOC_WORKSPACE_BYTES
 
 
 class FhipError(RuntimeError):
@@ -114,6 +115,7 @@ SYMBOLS = {
     "fhip_flash_attention_workspace_bytes": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.c_int32,
                                                             ctypes.POINTER(ctypes.c_size_t)]),
     "fhip_flash_attention": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
+    "fhip_flash_attention_noalloc": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
     "fhip_mask_causal": (ctypes.c_int, [ctypes.c_int, ctypes.c_uint32, _P]),
     "fhip_mask_sliding_window": (ctypes.c_int, [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, _P]),
     "fhip_mask_get_mask_shape": (ctypes.c_int, [ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int32, ctypes.c_uint64,
@@ -496,6 +498,14 @@ class Tensor:
             args.workspace_bytes = nb
         check(L.fhip_flash_attention(dev.stream, ctypes.byref(args)))
         return args._out_tensor
+
+    def flash_attention_noalloc(self, k, v, scale, out, mask=None, *, analytic=None, kv_lens=None,
+                                force_kernel=KERNEL_AUTO):
+        """flash_attention into `out` on the library's own fixed workspace (fhip_flash_attention_noalloc): nothing
+        is allocated by the call, here or in the library."""
+        args = self._attn_args(k, v, scale, mask, analytic, kv_lens, out.dtype, force_kernel, out)
+        check(lib().fhip_flash_attention_noalloc(self.device.stream, ctypes.byref(args)))
+        return out
 
     def _attn_args(self, k, v, scale, mask, analytic, kv_lens, out_dtype, force_kernel, out):
         if not (k.device is self.device and v.device is self.device):

@@ -10,9 +10,19 @@
 
 #include "common.h"
 
+// Workspace of fhip_flash_attention_noalloc: device memory the library itself holds, so that the call needs no
+// allocation by anyone.  Each GPU the library runs on has its own copy of the array at its own address, looked
+// up once per device in fhip_device_create (the name below is only a host-side handle of the symbol, not a
+// device address).  Its contents are whatever the last call left: every user of the workspace (split-KV
+// partials, mask intervals and their per-call mark, prefill key shares) writes what it reads, so nothing has
+// to start at zero.
+constexpr size_t STATIC_WORKSPACE_BYTES = (size_t)FHIP_NOALLOC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_WORKSPACE_BYTES];
+
 struct fhip_device {
     int ordinal;
     hipDeviceProp_t prop;
+    void *scratch_ptr;  // this device's address of `scratch`
 };
 struct fhip_stream {
     fhip_device *dev;
@@ -369,6 +379,14 @@ int fhip_device_create(int32_t ordinal, fhip_device **out) {
         set_error("device %d is %s; this library carries gfx950 code only", ordinal, d->prop.gcnArchName);
         delete d;
         return FHIP_ERR_UNSUPPORTED;
+    }
+    // this device's copy of the static workspace (the lookup is per device: it must be the current one)
+    d->scratch_ptr = nullptr;
+    e = hipSetDevice(ordinal);
+    if (e == hipSuccess) e = hipGetSymbolAddress((void **)&d->scratch_ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !d->scratch_ptr) {
+        delete d;
+        return hip_fail(e, "hipGetSymbolAddress(scratch)");
     }
     *out = d;
     return FHIP_OK;
@@ -774,6 +792,27 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     }
     if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
     return rc;
+}
+
+// The same call on the library's own workspace (see `scratch` above): no hipMalloc / hipFree here or in anything
+// this calls, and none needed from the caller beyond the tensors.
+int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args) {
+    if (!s) {
+        set_error("stream is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    size_t need = 0;
+    int rc = fhip_flash_attention_workspace_bytes(args, s->dev->prop.multiProcessorCount, &need);
+    if (rc) return rc;
+    if (need > STATIC_WORKSPACE_BYTES) {
+        set_error("this call needs a workspace of %zu bytes; fhip_flash_attention_noalloc holds %zu (use "
+                  "fhip_flash_attention with a workspace of your own)", need, STATIC_WORKSPACE_BYTES);
+        return FHIP_ERR_WORKSPACE;
+    }
+    fhip_attn_args a = *args;
+    a.workspace = s->dev->scratch_ptr;
+    a.workspace_bytes = STATIC_WORKSPACE_BYTES;
+    return fhip_flash_attention(s, &a);
 }
 
 // ---- masks (host, bit-exact) --------------------------------------------------------------------

@@ -220,6 +220,17 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
  * is what the reference's [Sq, 0] x [0, D] product gives (fusor flash_attention.rs:141-199). */
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
 
+/* fhip_flash_attention for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels and
+ * the same results bit for bit, but the workspace is a fixed array of FHIP_NOALLOC_WORKSPACE_BYTES of device
+ * memory that the library holds on every GPU it is used on until the process ends; args->workspace and
+ * args->workspace_bytes are ignored.  Neither this function nor anything it calls allocates or frees memory.
+ * A call whose fhip_flash_attention_workspace_bytes exceeds the array fails with FHIP_ERR_WORKSPACE and does
+ * nothing.  All calls on one GPU share that GPU's array: two of them must not overlap in time (one stream, or
+ * ordered by events); nothing in it has to be cleared between calls. */
+#define FHIP_NOALLOC_WORKSPACE_BYTES (32u << 20)
+int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
+
 /* ---- masks: host builders, bit-exact with the reference ---------------------------------------
  * `out` is host memory of the given dtype (f32: 0x00000000 / 0xFF800000; f16: 0x0000 / 0xFC00;
  * bf16: 0x0000 / 0xFF80), row-major contiguous. */
