@@ -18,9 +18,14 @@ from test_attention_gpu import rounded
 pytestmark = pytest.mark.gpu
 
 NEG = float("-inf")
-# (max-abs, rel-L2) per element type; the mixed shapes here include rows dominated by one key, where a 16-bit output
-# is off by half a unit in the last place of a value of order 1, hence the head-room over the benchmark tolerances
-TOL = {fa.F32: (None, 2e-5), fa.F16: (1e-2, 2e-3), fa.BF16: (1e-1, 2e-2)}
+# The parity gate, (max-abs, rel-L2): f32 tensors relative L2 1e-5; f16 tensors max-abs 2e-3 and relative L2 1e-3.
+# 16-bit cases are held to it on the f32 output the ABI offers (out_dtype = F32): the arithmetic is the same, and the
+# comparison is then free of the final rounding to 16 bits, which alone is half a unit in the last place of the value
+# (4.9e-4 of a value of order 1 in f16).  bf16 is not a type the gate names: its probabilities carry 8 bits, the bound
+# below is what that allows.
+GATE = {fa.F32: (None, 1e-5), fa.F16: (2e-3, 1e-3), fa.BF16: (2e-2, 8e-3)}
+# second, looser check of the same call with the output in the tensors' own type (what the reference returns)
+NATIVE = {fa.F16: (1e-2, 2e-3), fa.BF16: (1e-1, 2e-2)}
 
 
 def _case(rng, device):
@@ -92,17 +97,20 @@ def test_mixed_feature_sweep(device, seed):
         tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
         scale = float(D) ** -0.5
         used.add(tq.selected_kernel(tk, tv, scale, mt, analytic=analytic, kv_lens=lens_t))
-        out = tq.flash_attention(tk, tv, scale, mt, analytic=analytic, kv_lens=lens_t).to_numpy()
         ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale,
                                      None if mask is None else rounded(mask, dtype), kind)
-        dead_out, dead_ref = np.isnan(out).any(-1), np.isnan(ref).any(-1)
-        assert np.array_equal(dead_out, dead_ref), f"case {it}: rows without a visible key differ: {what}"
+        dead_ref = np.isnan(ref).any(-1)
         live = ~dead_ref
-        if live.any():
-            tol_abs, tol_rel = TOL[dtype]
-            rl = rel_l2(out[live], ref[live])
-            assert rl <= tol_rel, f"case {it}: rel-L2 {rl:.3e}: {what}"
-            if tol_abs is not None:
-                ma = max_abs(out[live], ref[live])
-                assert ma <= tol_abs, f"case {it}: max-abs {ma:.3e}: {what}"
+        passes = [(fa.F32, GATE[dtype], "f32 output")] if dtype == fa.F32 else \
+                 [(fa.F32, GATE[dtype], "f32 output"), (dtype, NATIVE[dtype], "native output")]
+        for out_dtype, (tol_abs, tol_rel), label in passes:
+            out = tq.flash_attention(tk, tv, scale, mt, analytic=analytic, kv_lens=lens_t, out_dtype=out_dtype).to_numpy()
+            dead_out = np.isnan(out).any(-1)
+            assert np.array_equal(dead_out, dead_ref), f"case {it} ({label}): rows without a visible key differ: {what}"
+            if live.any():
+                rl = rel_l2(out[live], ref[live])
+                assert rl <= tol_rel, f"case {it} ({label}): rel-L2 {rl:.3e} > {tol_rel:.0e}: {what}"
+                if tol_abs is not None:
+                    ma = max_abs(out[live], ref[live])
+                    assert ma <= tol_abs, f"case {it} ({label}): max-abs {ma:.3e} > {tol_abs:.0e}: {what}"
     assert len(used) >= 3, "the sweep is meant to cross kernels"
