@@ -7,11 +7,14 @@ A step is one attention call through the C ABI on synthetic, seeded inputs that 
 HBM before the timed region.  The default workload is C2 (Llama-3-8B-shaped decode, batch 16, 4096
 f16 KV tokens per sequence): `value` is its KV-streaming rate in GB/s (algorithmic bytes per call /
 time per call, combine pass included).  The same JSON line also carries the C3 prefill figure
-(TFLOP/s, MFMA roofline) under "prefill", the HBM/MFMA roofline of the dominant kernel measured
-with HIP events on the launch stream, and the CPU checker timed on the host cores ("cpu_baseline").
+(TFLOP/s, MFMA roofline) under "prefill" and the other three benchmark configurations under
+"configs" (C1, C4, C5), each with the HBM/MFMA roofline of its dominant kernel (the kernel's own
+duration from HIP events carried by its dispatch on the launch stream) and the CPU checker timed on
+the host cores ("cpu_baseline").
 """
 import argparse
 import ctypes
+import hashlib
 import json
 import os
 import sys
@@ -27,9 +30,32 @@ PEAK_HBM_GBS = 8000.0
 PEAK_MFMA_F16_TFLOPS = 2500.0
 PEAK_MFMA_F32_TFLOPS = 157.3
 SEED = 0xF10E0000
-# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
-# same counter reads for a 256 MiB copy (profiles/decode_splitkv_C2.txt, profiles/prefill_mfma_C3.txt)
-MEASURED_TRAFFIC_BYTES = {"C2": 270.2e6, "C3": 214.6e6}
+# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
+# WRITE_SIZE), each scaled by what the same counter reads for a 256 MiB copy in the same run.  The record holds,
+# per configuration, the bytes and the SHA-256 of the kernel source they were measured on; a figure whose source
+# has changed since is not reported.  Written by --record-traffic from the counter CSVs.
+TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "traffic.json")
+KERNEL_SOURCES = {"decode_splitkv": "attn_decode.hip", "prefill_mfma": "attn_prefill_mfma.hip",
+                  "prefill_f32": "attn_prefill_f32.hip", "generic": "attn_generic.hip"}
+
+
+def source_hash(kernel):
+    path = os.path.join(ROOT, "floneum_amd", "csrc", KERNEL_SOURCES[kernel])
+    return hashlib.sha256(open(path, "rb").read()).hexdigest()
+
+
+def measured_traffic(name, kernel):
+    """(bytes per launch or None, note) from the committed counter record."""
+    try:
+        rec = json.load(open(TRAFFIC_RECORD)).get(name)
+    except (OSError, ValueError):
+        rec = None
+    if not rec:
+        return None, "no counter record for this configuration"
+    if rec.get("kernel") != kernel or rec.get("source_sha256") != source_hash(kernel):
+        return None, "the kernel source has changed since the counters were read"
+    return float(rec["fetch_bytes"]) + float(rec["write_bytes"]), \
+        f"FETCH_SIZE {rec['fetch_bytes']:.4g} B + WRITE_SIZE {rec['write_bytes']:.4g} B per launch"
 
 
 def configs():
@@ -160,13 +186,14 @@ def prepare(fa, dev, c, sets, lens_t):
             args._keep.append(ws)
         blocks.append(args)
     kid = ctypes.c_int32()
-    fa.check(L.fhip_flash_attention_select(ctypes.byref(blocks[0]), dev.compute_units, ctypes.byref(kid)))
+    fa.check(L.fhip_flash_attention_select(ctypes.byref(blocks[0]), ctypes.byref(kid)))
     return blocks, fa.KERNEL_NAMES[kid.value]
 
 
 def time_config(fa, dev, c, blocks, steps, warmup):
-    """Wall-clock over exactly `steps` calls (sync on both sides), then a second instrumented pass
-    of `steps` calls with HIP events around the main kernel of every call."""
+    """Wall-clock over exactly `steps` calls (sync on both sides), then a second instrumented pass of `steps`
+    calls in which the dispatch of every call's main kernel carries a pair of HIP events: their interval is the
+    kernel's own duration as the command processor stamps it (what a profiler's kernel trace reports)."""
     L = fa.lib()
     n = len(blocks)
     for i in range(warmup):
@@ -179,29 +206,17 @@ def time_config(fa, dev, c, blocks, steps, warmup):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
 
     starts = [Event(fa, dev) for _ in range(steps)]
-    mids = [Event(fa, dev) for _ in range(steps)]
-    ends = [Event(fa, dev) for _ in range(steps)]
+    dones = [Event(fa, dev) for _ in range(steps)]
     for i in range(steps):
         a = blocks[i % n]
-        a.main_kernel_done = mids[i].h
-        starts[i].record(dev)
+        a.main_kernel_start, a.main_kernel_done = starts[i].h, dones[i].h
         fa.check(L.fhip_flash_attention(dev.stream, ctypes.byref(a)))
-        ends[i].record(dev)
-        a.main_kernel_done = None
+        a.main_kernel_start = a.main_kernel_done = None
     dev.synchronize()
-    main_ms = np.array([mids[i].ms_since(starts[i]) for i in range(steps)])
-    call_ms = np.array([ends[i].ms_since(starts[i]) for i in range(steps)])
-    # What a pair of events reads with nothing between them (the second marker's own processing): a
-    # few microseconds, which matters for a 45 us kernel.  It is measured here and taken off the
-    # kernel intervals so that they are comparable with a profiler's dispatch durations.
-    for i in range(steps):
-        starts[i].record(dev)
-        mids[i].record(dev)
-    dev.synchronize()
-    empty_ms = float(np.median([mids[i].ms_since(starts[i]) for i in range(steps)]))
-    for e in starts + mids + ends:
+    kernel_ms = np.array([dones[i].ms_since(starts[i]) for i in range(steps)])
+    for e in starts + dones:
         L.fhip_event_destroy(e.h)
-    return wall_ms, main_ms - empty_ms, float(call_ms.mean()), empty_ms, float(main_ms.mean())
+    return wall_ms, kernel_ms
 
 
 def parity_spot_check(fa, oracle, c, out_t, host, lens):
@@ -245,28 +260,30 @@ def cpu_baseline(oracle, c, host, lens, flops, byts):
             # ragged: one un-padded call per sequence on a subset of sequences (upcast outside the clock,
             # as kalosm-llama keeps its cache in f32)
             pick = list(range(min(4, c["B"])))
-            dt = 0.0
-            for b in pick:
-                n = int(lens[b])
-                qb, kb, vb = f32(q[b:b + 1]), f32(k[b:b + 1, :, :n]), f32(v[b:b + 1, :, :n])
+            reps, dts = 3, []
+            seqs = [(f32(q[b:b + 1]), f32(k[b:b + 1, :, :int(lens[b])]), f32(v[b:b + 1, :, :int(lens[b])])) for b in pick]
+            for _ in range(reps):
                 t0 = time.perf_counter()
-                oracle.flash_attention(qb, kb, vb, scale)
-                dt += time.perf_counter() - t0
+                for qb, kb, vb in seqs:
+                    oracle.flash_attention(qb, kb, vb, scale)
+                dts.append(time.perf_counter() - t0)
             frac = float(np.sum(lens[pick])) / float(np.sum(lens))
-            sample = f"sequences {pick} of the batch, un-padded, f16 upcast to f32, 1 pass"
-            return dict(value=byts * frac / dt / 1e9, unit="GB/s", cores=threads, kind="port", sample=sample)
-        reps = 3
+            sample = f"sequences {pick} of the batch, un-padded, f16 upcast to f32, median of {reps} passes"
+            return dict(value=byts * frac / float(np.median(dts)) / 1e9, unit="GB/s", cores=threads, kind="port",
+                        sample=sample)
+        reps, dts = 3, []
         q, k, v = f32(q), f32(k), f32(v)
         oracle.flash_attention(q, k, v, scale)
-        t0 = time.perf_counter()
         for _ in range(reps):
+            t0 = time.perf_counter()
             oracle.flash_attention(q, k, v, scale)
-        dt = (time.perf_counter() - t0) / reps
-        return dict(value=byts / dt / 1e9, unit="GB/s", cores=threads, kind="port",
-                    sample=f"the full step (all {c['B']} sequences), f16 upcast to f32 first, mean of {reps} passes")
+            dts.append(time.perf_counter() - t0)
+        return dict(value=byts / float(np.median(dts)) / 1e9, unit="GB/s", cores=threads, kind="port",
+                    sample=f"the full step (all {c['B']} sequences), f16 upcast to f32 first, median of {reps} passes "
+                           "after one warm-up pass")
     # prefill: a subset of query rows of every head (rows are independent in the reference algorithm)
     q, k, v = f32(q), f32(k), f32(v)
-    target_flops = 4e11
+    target_flops = 2e11
     stride = max(1, int(np.ceil(flops / target_flops)))
     rows = np.arange(stride - 1, c["Sq"], stride, dtype=np.int32)
     off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
@@ -276,15 +293,19 @@ def cpu_baseline(oracle, c, host, lens, flops, byts):
     if c.get("window", 0):
         masked |= (j + c["window"]) <= i
     mask = np.where(masked, -np.inf, 0.0).astype(np.float32)
-    t0 = time.perf_counter()
-    oracle.flash_attention(q[:, :, rows], k, v, scale, mask, "qk")
-    dt = time.perf_counter() - t0
+    reps, dts = 3, []
+    qs = np.ascontiguousarray(q[:, :, rows])
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        oracle.flash_attention(qs, k, v, scale, mask, "qk")
+        dts.append(time.perf_counter() - t0)
+    dt = float(np.median(dts))
     # the CPU path has no tile skipping: it computes every (row, key) pair and masks afterwards, but
     # it is credited, like the GPU, with the visible pairs only
     sample_flops = 4 * c["D"] * c["H"] * c["B"] * int((~masked).sum())
     return dict(value=sample_flops / dt / 1e12, unit="TFLOP/s", cores=threads, kind="port",
                 sample=f"every {stride}th query row of every head ({len(rows)} of {c['Sq']} rows), dense "
-                       f"[rows, Skv] scores then mask, as the reference does")
+                       f"[rows, Skv] scores then mask, as the reference does; median of {reps} passes")
 
 
 def run_config(name, steps, warmup, with_cpu=True):
@@ -307,7 +328,7 @@ def run_config(name, steps, warmup, with_cpu=True):
         n_sets = 1  # 6.5 GB per step already dwarfs the cache; one padded set is 13 GB of HBM
     dt, sets, host = make_inputs(fa, synth, dev, c, cfg_id, n_sets)
     blocks, kernel = prepare(fa, dev, c, sets, lens_t)
-    wall_ms, main_ms, call_ms, empty_ms, main_ms_raw = time_config(fa, dev, c, blocks, steps, warmup)
+    wall_ms, main_ms = time_config(fa, dev, c, blocks, steps, warmup)
     main_ms_mean, main_ms_med = float(main_ms.mean()), float(np.median(main_ms))
     err = parity_spot_check(fa, oracle, c, blocks[0]._out_tensor, host, lens)
 
@@ -319,14 +340,11 @@ def run_config(name, steps, warmup, with_cpu=True):
         value, unit = flops / (wall_ms * 1e-3) / 1e12, "TFLOP/s"
         roof = dict(bound="mfma", achieved=flops / (main_ms_mean * 1e-3) / 1e12, peak=peak, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(name)
+    roof["traffic"], roof["traffic_note"] = measured_traffic(name, kernel)
     roof["kernel"] = kernel
     roof["kernel_ms_mean"] = main_ms_mean
     roof["kernel_ms_median"] = main_ms_med
     roof["kernel_ms_min"] = float(main_ms.min())
-    roof["kernel_ms_events_raw"] = main_ms_raw
-    roof["event_pair_empty_ms"] = empty_ms
-    roof["call_ms_events"] = call_ms
     res = dict(value=value, unit=unit, ms_per_step=wall_ms, roofline=roof,
                config=dict(workload=name, kind=c["kind"], batch=c["B"], q_heads=c["H"], kv_heads=c["Hkv"],
                            q_len=c["Sq"], kv_len=c["Skv"], head_dim=c["D"], causal=c["causal"],
@@ -341,7 +359,7 @@ def run_config(name, steps, warmup, with_cpu=True):
         eq_t = fa.IntTensor(dev, eq)
         _, eq_byts = algorithmic(c, eq)
         eq_blocks, _ = prepare(fa, dev, c, sets, eq_t)
-        eq_wall_ms, _, _, _, _ = time_config(fa, dev, c, eq_blocks, max(5, steps // 2), min(warmup, 5))
+        eq_wall_ms, _ = time_config(fa, dev, c, eq_blocks, max(5, steps // 2), min(warmup, 5))
         eq_value = eq_byts / (eq_wall_ms * 1e-3) / 1e9
         res["imbalance"] = dict(lens_min=int(lens.min()), lens_mean=float(lens.mean()), lens_max=int(lens.max()),
                                 equal_lengths_value=eq_value, unit=unit, ragged_over_equal=value / eq_value,
@@ -366,6 +384,48 @@ def calibration_copy(mib=256, reps=3):
         del cache
 
 
+def record_traffic(name, fetch_csv, write_csv):
+    """profiles/traffic.json entry of one configuration from the two counter CSVs (one counter per profiler run).
+    The copy kernel of --calibration-copy moves 256 MiB each way; its counts give the bytes per count."""
+    import csv
+
+    def per_kernel(path, counter):
+        sums = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] == counter:
+                sums.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return {k: float(np.mean(v)) for k, v in sums.items()}
+
+    copied = 256 * (1 << 20)
+    out = {}
+    kernel = None
+    for key, path, counter in (("fetch_bytes", fetch_csv, "FETCH_SIZE"), ("write_bytes", write_csv, "WRITE_SIZE")):
+        counts = per_kernel(path, counter)
+        copy = [v for k, v in counts.items() if "copy_rows_kernel" in k]
+        assert copy, f"{path}: no copy_rows_kernel dispatches (run bench.py with --calibration-copy)"
+        per_count = copied / copy[0]
+        main = {k: v for k, v in counts.items() if any(t in k for t in ("decode_mfma", "decode_vec", "prefill_mfma_kernel",
+                                                                       "prefill_f32_kernel", "prefill_f32_wide", "attn_generic"))}
+        assert len(main) == 1, f"{path}: expected one main kernel, found {sorted(main)}"
+        kname, count = next(iter(main.items()))
+        out[key] = count * per_count
+        out[key.replace("bytes", "bytes_per_count")] = per_count
+        kernel = "decode_splitkv" if "decode" in kname else "prefill_mfma" if "prefill_mfma" in kname else \
+            "prefill_f32" if "prefill_f32" in kname else "generic"
+        out["kernel_symbol"] = kname
+    out["kernel"] = kernel
+    out["source_sha256"] = source_hash(kernel)
+    try:
+        rec = json.load(open(TRAFFIC_RECORD))
+    except (OSError, ValueError):
+        rec = {}
+    rec[name] = out
+    with open(TRAFFIC_RECORD, "w") as f:
+        json.dump(rec, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({name: out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -373,7 +433,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="C2", choices=sorted(configs()))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the secondary (prefill C3) figure")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the other configurations (C3 under \"prefill\"; C1, C4, C5 under \"configs\")")
+    ap.add_argument("--record-traffic", nargs=3, metavar=("CONFIG", "FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: read the counter_collection CSVs of two `rocprofv3 --pmc FETCH_SIZE` / `--pmc "
+                         "WRITE_SIZE` runs of `bench.py --config CONFIG --no-cpu --no-extra --calibration-copy` and "
+                         "store the dominant kernel's HBM bytes per launch in profiles/traffic.json")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (the KV-cache row copy kernel) three times, so a "
                          "rocprofv3 --pmc run of this command has a kernel of known traffic to scale FETCH_SIZE / "
@@ -383,6 +448,10 @@ def main():
         print(f"bench.py: this build runs on exactly one GPU (no sharding, no collectives); --gpus {a.gpus} is "
               "not supported", file=sys.stderr)
         sys.exit(2)
+
+    if a.record_traffic:
+        record_traffic(*a.record_traffic)
+        return
 
     main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
     if a.calibration_copy:
@@ -406,6 +475,12 @@ def main():
                                                "frac_of_roofline", "spot_check_max_abs_err") if k in pre}
         if "cpu_baseline" in pre:
             line["prefill"]["cpu_baseline"] = pre["cpu_baseline"]
+        # the remaining benchmark configurations, each a line of its own in miniature
+        line["configs"] = {}
+        for name, (steps, warmup) in (("C1", (200, 20)), ("C4", (100, 100)), ("C5", (20, 3))):
+            r = run_config(name, steps, warmup, with_cpu=not a.no_cpu)
+            r["steps"], r["warmup"] = steps, warmup
+            line["configs"][name] = r
     print(json.dumps(line))
 
 

@@ -66,7 +66,8 @@ class CAttnArgs(ctypes.Structure):
                 ("dtype", ctypes.c_int), ("out_dtype", ctypes.c_int), ("scale", ctypes.c_float),
                 ("mask_kind", ctypes.c_int), ("mask", CTensor2), ("analytic", CAnalyticMask),
                 ("kv_lens", ctypes.c_void_p), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
-                ("force_kernel", ctypes.c_int32), ("main_kernel_done", ctypes.c_void_p)]
+                ("force_kernel", ctypes.c_int32), ("main_kernel_done", ctypes.c_void_p),
+                ("main_kernel_start", ctypes.c_void_p)]
 
 
 class CDeviceInfo(ctypes.Structure):
@@ -110,8 +111,7 @@ SYMBOLS = {
     "fhip_event_synchronize": (ctypes.c_int, [_P]),
     "fhip_event_elapsed_ms": (ctypes.c_int, [_P, _P, ctypes.POINTER(ctypes.c_float)]),
     "fhip_flash_attention_validate": (ctypes.c_int, [ctypes.POINTER(CAttnArgs)]),
-    "fhip_flash_attention_select": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.c_int32,
-                                                   ctypes.POINTER(ctypes.c_int32)]),
+    "fhip_flash_attention_select": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.POINTER(ctypes.c_int32)]),
     "fhip_flash_attention_workspace_bytes": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.c_int32,
                                                             ctypes.POINTER(ctypes.c_size_t)]),
     "fhip_flash_attention": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
@@ -553,7 +553,7 @@ class Tensor:
         args = self._attn_args(k, v, scale, mask, kw.get("analytic"), kw.get("kv_lens"), kw.get("out_dtype"),
                                kw.get("force_kernel", KERNEL_AUTO), kw.get("out"))
         kid = ctypes.c_int32()
-        check(lib().fhip_flash_attention_select(ctypes.byref(args), self.device.compute_units, ctypes.byref(kid)))
+        check(lib().fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
         return kid.value
 
 

@@ -23,6 +23,9 @@ struct fhip_device {
     int ordinal;
     hipDeviceProp_t prop;
     void *scratch_ptr;  // this device's address of `scratch`
+    // Source of the per-call marks of masked prefill calls (AttnParams::bad_tag): the one piece of state a device
+    // handle changes after its creation.
+    std::atomic<uint32_t> next_tag;
 };
 struct fhip_stream {
     fhip_device *dev;
@@ -370,6 +373,8 @@ int fhip_device_create(int32_t ordinal, fhip_device **out) {
         return FHIP_ERR_HIP;
     }
     d->ordinal = ordinal;
+    // handles of one device start their marks far apart, so that two of them sharing a workspace do not collide
+    d->next_tag.store(0x5eed0001u + (uint32_t)((uintptr_t)d >> 4) * 2654435761u, std::memory_order_relaxed);
     hipError_t e = hipGetDeviceProperties(&d->prop, ordinal);
     if (e != hipSuccess) {
         delete d;
@@ -642,8 +647,7 @@ int fhip_event_elapsed_ms(fhip_event *start, fhip_event *stop, float *ms) {
 
 int fhip_flash_attention_validate(const fhip_attn_args *args) { return validate(args); }
 
-int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id) {
-    (void)compute_units;
+int fhip_flash_attention_select(const fhip_attn_args *args, int32_t *kernel_id) {
     if (!kernel_id) {
         set_error("kernel_id is NULL");
         return FHIP_ERR_INVALID_ARG;
@@ -713,6 +717,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     AttnParams p;
     fill_params(args, &p);
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
+    p.main_start = args->main_kernel_start && p.main_done ? args->main_kernel_start->e : nullptr;
     p.cus = s->dev->prop.multiProcessorCount;
     if (id == FHIP_KERNEL_PREFILL_F32) {
         // few query rows on a long cache: split the keys over workgroups if the caller brought the scratch for it
@@ -742,7 +747,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     if (id == FHIP_KERNEL_PREFILL_F32 && args->mask_kind != FHIP_MASK_NONE && !mask_scratch_ok(args, false)) {
         // no scratch for the interval form: the f32 kernel adds the mask tensor element by element
         rc = launch_prefill_f32(p, args->dtype, s->s);
-        if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+        if (rc == FHIP_OK) FHIP_MARK_MAIN_DONE(p, s->s);
         return rc;
     }
     if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
@@ -751,8 +756,17 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         // call: the f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
-        static std::atomic<uint32_t> next_tag{0x5eed0001u};
-        p.bad_tag = (int32_t)next_tag.fetch_add(1, std::memory_order_relaxed);
+        do p.bad_tag = (int32_t)s->dev->next_tag.fetch_add(1, std::memory_order_relaxed);
+        while (p.bad_tag == 0);
+        // A recorded call is replayed with the mark it was recorded with: a replay whose mask is not made of intervals
+        // would leave that mark behind for every later replay.  Under capture the word is therefore cleared first
+        // (by a kernel, which is what a graph may hold); an eager call's mark is new every time and needs no clearing.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        FHIP_HIP_CHECK(hipStreamIsCapturing(s->s, &capturing));
+        if (capturing == hipStreamCaptureStatusActive) {
+            rc = launch_fill_zero_bytes(bad, 16, s->s);
+            if (rc) return rc;
+        }
         rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
         if (rc) return rc;
         AttnParams pt = p;
@@ -760,9 +774,10 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         pt.iv_bad = bad;
         rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, args->dtype, s->s);
         if (rc) return rc;
-        if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+        FHIP_MARK_MAIN_DONE(p, s->s);
         AttnParams pg = p;
         pg.only_if_bad = bad;
+        pg.main_start = pg.main_done = nullptr;  // the hook times the tiled kernel
         if (id == FHIP_KERNEL_PREFILL_MFMA) pg.pf_nsplit = 0;  // the split was planned for the other kernel's blocks
         return prefill_f32_eligible(args) && f32_adds_masks(args) ? launch_prefill_f32(pg, args->dtype, s->s)
                                                                   : launch_generic(pg, args->dtype, s->s);
@@ -790,7 +805,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         }
         default: set_error("internal: no kernel for id %d", id); return FHIP_ERR_UNSUPPORTED;
     }
-    if (rc == FHIP_OK && p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, s->s));
+    if (rc == FHIP_OK) FHIP_MARK_MAIN_DONE(p, s->s);
     return rc;
 }
 

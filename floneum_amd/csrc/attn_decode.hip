@@ -795,10 +795,10 @@ template <typename T, int LPK>
 static void launch_vec(const AttnParams &p, dim3 grid, hipStream_t stream, int gt) {
     dim3 block(64 * DEC_WAVES);
     switch (gt) {
-        case 1: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 1>), grid, block, 0, stream, p); break;
-        case 2: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 2>), grid, block, 0, stream, p); break;
-        case 4: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 4>), grid, block, 0, stream, p); break;
-        default: hipLaunchKernelGGL((decode_vec_kernel<T, LPK, 8>), grid, block, 0, stream, p); break;
+        case 1: FHIP_LAUNCH_MAIN((decode_vec_kernel<T, LPK, 1>), grid, block, stream, p, p); break;
+        case 2: FHIP_LAUNCH_MAIN((decode_vec_kernel<T, LPK, 2>), grid, block, stream, p, p); break;
+        case 4: FHIP_LAUNCH_MAIN((decode_vec_kernel<T, LPK, 4>), grid, block, stream, p, p); break;
+        default: FHIP_LAUNCH_MAIN((decode_vec_kernel<T, LPK, 8>), grid, block, stream, p, p); break;
     }
 }
 
@@ -816,13 +816,13 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     if constexpr (!F32) {
         if (decode_use_mfma(p.D, false)) {
             switch (p.D) {
-                case 32: hipLaunchKernelGGL((decode_mfma_kernel<T, 32>), grid, block, 0, stream, p); break;
-                case 64: hipLaunchKernelGGL((decode_mfma_kernel<T, 64>), grid, block, 0, stream, p); break;
-                case 96: hipLaunchKernelGGL((decode_mfma_kernel<T, 96>), grid, block, 0, stream, p); break;
-                default: hipLaunchKernelGGL((decode_mfma_kernel<T, 128>), grid, block, 0, stream, p); break;
+                case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32>), grid, block, stream, p, p); break;
+                case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64>), grid, block, stream, p, p); break;
+                case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96>), grid, block, stream, p, p); break;
+                default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128>), grid, block, stream, p, p); break;
             }
             FHIP_HIP_CHECK(hipGetLastError());
-            if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
+            FHIP_MARK_MAIN_DONE(p, stream);
             if (p.nsplit > 1) {
                 launch_combine<T>(p, stream);
                 FHIP_HIP_CHECK(hipGetLastError());
@@ -840,7 +840,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         launch_vec<T, 32>(p, grid, stream, gt);
     }
     FHIP_HIP_CHECK(hipGetLastError());
-    if (p.main_done) FHIP_HIP_CHECK(hipEventRecord(p.main_done, stream));
+    FHIP_MARK_MAIN_DONE(p, stream);
     if (p.nsplit > 1) {
         launch_combine<T>(p, stream);
         FHIP_HIP_CHECK(hipGetLastError());

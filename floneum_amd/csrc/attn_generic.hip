@@ -112,9 +112,9 @@ int launch_generic(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * GEN_WAVES);
     switch (dtype) {
-        case FHIP_F32: hipLaunchKernelGGL(attn_generic_kernel<float>, grid, block, 0, stream, p); break;
-        case FHIP_F16: hipLaunchKernelGGL(attn_generic_kernel<half_t>, grid, block, 0, stream, p); break;
-        case FHIP_BF16: hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, block, 0, stream, p); break;
+        case FHIP_F32: FHIP_LAUNCH_MAIN(attn_generic_kernel<float>, grid, block, stream, p, p); break;
+        case FHIP_F16: FHIP_LAUNCH_MAIN(attn_generic_kernel<half_t>, grid, block, stream, p, p); break;
+        case FHIP_BF16: FHIP_LAUNCH_MAIN(attn_generic_kernel<bf16_t>, grid, block, stream, p, p); break;
     }
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;

@@ -690,7 +690,7 @@ static int launch_wide(const AttnParams &p, hipStream_t stream) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(prefill_f32_wide_kernel<T>, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), 0, stream, p, nqb);
+    FHIP_LAUNCH_MAIN(prefill_f32_wide_kernel<T>, dim3((unsigned)blocks), dim3(64 * PF32_WAVES), stream, p, p, nqb);
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.pf_nsplit > 1) return launch_merge_t<T>(p, stream);
     return FHIP_OK;
@@ -721,13 +721,13 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
     switch ((p.D + 31) / 32 * 32) {  // the kernel's D is head_dim rounded up to a multiple of 32
-        case 32: hipLaunchKernelGGL((prefill_f32_kernel<T, 32, S, BIAS>), grid, block, 0, stream, p, nqb); break;
-        case 64: hipLaunchKernelGGL((prefill_f32_kernel<T, 64, S, BIAS>), grid, block, 0, stream, p, nqb); break;
+        case 32: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 32, S, BIAS>), grid, block, stream, p, p, nqb); break;
+        case 64: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 64, S, BIAS>), grid, block, stream, p, p, nqb); break;
         case 96:
-            if constexpr (S <= (BIAS ? 1 : 4)) hipLaunchKernelGGL((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4)) FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, stream, p, p, nqb);
             break;
         case 128:
-            if constexpr (S <= (BIAS ? 1 : 4)) hipLaunchKernelGGL((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, 0, stream, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4)) FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, stream, p, p, nqb);
             break;
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }

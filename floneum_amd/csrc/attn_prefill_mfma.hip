@@ -706,8 +706,8 @@ static int launch_t(const AttnParams &p, hipStream_t stream) {
     for (int i = 0; i < 3; i++)
         if ((p.os[i] * oeb) % 16 != 0) out_vec = 0;
 #define PF_LAUNCH(DIM)                                                                                         \
-    if (ks) hipLaunchKernelGGL((prefill_mfma_kernel<T, DIM, true>), grid, block, 0, stream, p, nqb, out_vec);   \
-    else hipLaunchKernelGGL((prefill_mfma_kernel<T, DIM, false>), grid, block, 0, stream, p, nqb, out_vec)
+    if (ks) FHIP_LAUNCH_MAIN((prefill_mfma_kernel<T, DIM, true>), grid, block, stream, p, p, nqb, out_vec);      \
+    else FHIP_LAUNCH_MAIN((prefill_mfma_kernel<T, DIM, false>), grid, block, stream, p, p, nqb, out_vec)
     switch (p.D) {
         case 64: PF_LAUNCH(64); break;
         case 96: PF_LAUNCH(96); break;

@@ -1,6 +1,7 @@
 // Internal declarations shared by the C-ABI layer and the kernel launchers.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/fusor_hip.h"
@@ -27,7 +28,9 @@ struct AttnParams {
     float *partials;        // [B, H, nsplit, D + 2] per-split (acc, m, l)
     int32_t chunk;          // keys per split
     int32_t nsplit;         // splits per (batch, kv head) over Skv
-    hipEvent_t main_done;   // host-side only: recorded after the main kernel when not null
+    // host-side only (profiling hook).  Both set: the dispatch of the main kernel carries the two events, which then
+    // hold its own begin and end timestamps.  Only main_done: recorded on the stream after the main kernel.
+    hipEvent_t main_start, main_done;
     // Dense additive mask reduced to intervals (see mask_intervals.hip).  iv[r] = {lo, hi}: row r of the
     // mask is 0 on keys [lo, hi) and -inf elsewhere; r is the query row (FHIP_MASK_QK) or the batch
     // (FHIP_MASK_BATCH_KEY).  *iv_bad holds bad_tag when some row is NOT of that form.  A tiled kernel given
@@ -62,7 +65,8 @@ int launch_prefill_merge(const AttnParams &p, fhip_dtype dtype, hipStream_t stre
 
 // bytes of device scratch the interval form of a dense mask needs
 size_t mask_intervals_bytes(int rows);
-// fills iv[rows] and *bad (zeroed first) from the mask described by p.mask / p.ms0 / p.ms1 / p.mask_kind
+// fills iv[rows] from the mask described by p.mask / p.ms0 / p.ms1 / p.mask_kind and stores p.bad_tag in *bad if some
+// row is not an interval (*bad is left alone otherwise: whatever it held is not this call's mark)
 int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32_t *bad, hipStream_t stream);
 
 // writes get_mask's [rows, cols] tensor (0 / -inf bit patterns of `dtype`) into device memory; off = cols - rows
@@ -77,6 +81,21 @@ int hip_fail(hipError_t e, const char *what);
     do {                                                      \
         hipError_t e__ = (expr);                              \
         if (e__ != hipSuccess) return fhip::hip_fail(e__, #expr); \
+    } while (0)
+
+// Launch of a call's main kernel: with both profiling events the dispatch itself is timestamped into them (what a
+// profiler's kernel trace reports), otherwise a plain launch.
+#define FHIP_LAUNCH_MAIN(kernel, grid, block, stream, p, ...)                                                    \
+    do {                                                                                                         \
+        if ((p).main_start && (p).main_done)                                                                     \
+            hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, (p).main_start, (p).main_done, 0, __VA_ARGS__); \
+        else                                                                                                     \
+            hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);                                      \
+    } while (0)
+// after the main kernel: the stream marker of the older form of the hook (main_done alone)
+#define FHIP_MARK_MAIN_DONE(p, stream)                                                                           \
+    do {                                                                                                         \
+        if ((p).main_done && !(p).main_start) FHIP_HIP_CHECK(hipEventRecord((p).main_done, stream));              \
     } while (0)
 
 // launchers (each returns a status code, all asynchronous on `stream`)

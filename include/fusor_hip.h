@@ -18,8 +18,10 @@
  *     (narrowed KV-cache views, transposed Q/V, broadcast strides of 0 on inputs).
  *   - The library never allocates or frees caller tensors.  The output buffer and the workspace
  *     are supplied by the caller.  Launches are asynchronous on the given stream.
- *   - Re-entrant: no global mutable state besides per-device handles and the thread-local error
- *     string.  One stream is used from one thread at a time.
+ *   - Re-entrant: the only mutable state lives in the handles (a device handle holds an atomic counter that
+ *     numbers masked prefill calls, a KV cache its buffers) and in the thread-local error string; there are no
+ *     global variables.  Calls on different streams may run concurrently from different threads; one stream, one
+ *     KV cache and one workspace are used by one thread at a time.
  */
 #ifndef FUSOR_HIP_H
 #define FUSOR_HIP_H
@@ -123,6 +125,10 @@ typedef struct {
      * main kernel of the call (before the split-KV combine pass, if there is one), so a benchmark
      * can time that kernel alone with HIP events. */
     fhip_event *main_kernel_done;
+    /* With main_kernel_done: when non-NULL too, the main kernel's dispatch itself carries the two events
+     * and they hold its begin and end as the command processor stamps them; fhip_event_elapsed_ms(start,
+     * done) is then the kernel's own duration, the figure a profiler's kernel trace gives. */
+    fhip_event *main_kernel_start;
 } fhip_attn_args;
 
 typedef enum {
@@ -204,8 +210,10 @@ int fhip_flash_attention_validate(const fhip_attn_args *args);
  * the mask turns out to be made of intervals (decided on the device) and otherwise hands over, inside
  * the same call, to the kernel that adds the mask values one by one (the mask-adding form of the
  * f32-arithmetic tiled kernel up to head_dim 128, the general kernel above); without the workspace it
- * names that kernel. */
-int fhip_flash_attention_select(const fhip_attn_args *args, int32_t compute_units, int32_t *kernel_id);
+ * names that kernel.  The answer does not depend on the device: how a kernel splits its work over the
+ * compute units is planned inside the call, and fhip_flash_attention_workspace_bytes takes their number
+ * because the scratch for those splits does. */
+int fhip_flash_attention_select(const fhip_attn_args *args, int32_t *kernel_id);
 
 /* Bytes of device workspace the call needs (0 for the single-pass kernels).  `compute_units`
  * is fhip_device_info.compute_units (split count depends on it). */

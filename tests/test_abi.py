@@ -36,7 +36,7 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(fa.CTensor4) == 8 + 8 + 16 + 32
     assert ctypes.sizeof(fa.CTensor2) == 8 + 8 + 8 + 16
     assert ctypes.sizeof(fa.CAnalyticMask) == 24
-    assert ctypes.sizeof(fa.CAttnArgs) == 4 * 64 + 16 + 40 + 24 + 8 + 8 + 8 + 8 + 8
+    assert ctypes.sizeof(fa.CAttnArgs) == 4 * 64 + 16 + 40 + 24 + 8 + 8 + 8 + 8 + 8 + 8
 
 
 def t4(shape, strides=None, ptr=FAKE, offset=0):
@@ -139,7 +139,7 @@ def test_validate_accepts_tensors_without_elements():
 
 def selected(a):
     kid = ctypes.c_int32()
-    rc = fa.lib().fhip_flash_attention_select(ctypes.byref(a), 256, ctypes.byref(kid))
+    rc = fa.lib().fhip_flash_attention_select(ctypes.byref(a), ctypes.byref(kid))
     return rc, kid.value
 
 

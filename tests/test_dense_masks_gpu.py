@@ -88,7 +88,7 @@ def test_block_diagonal_mask_of_the_vision_blocks(device, dtype, D):
     args = tq._attn_args(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask), None, None, None, fa.KERNEL_AUTO, out_t)
     args.workspace, args.workspace_bytes = ws, ws_bytes
     kid = ctypes.c_int32()
-    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), device.compute_units, ctypes.byref(kid)))
+    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
     assert kid.value == want
     out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
     ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "qk")
@@ -202,7 +202,7 @@ def test_padding_mask_with_a_large_finite_value(device, D, B, H, S, workspace):
         ws, ws_bytes = device.workspace(max(need.value, 16))
         args.workspace, args.workspace_bytes = ws, ws_bytes
     kid = ctypes.c_int32()
-    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), device.compute_units, ctypes.byref(kid)))
+    fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
     assert kid.value == fa.KERNEL_PREFILL_F32
     fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
     ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "batch_key")

@@ -78,8 +78,10 @@ def test_decode_step_replayed_with_growing_key_counts(device, dtype):
 
 def test_masked_prefill_replayed(device):
     """A prefill call with a mask tensor is three launches (interval scan, tiled kernel, the kernel for masks that are
-    not intervals) and a kernel that clears the scan's counter: all of it is recorded, and the mask content may
-    change between replays, including from the interval form to a bias."""
+    not intervals), plus, under capture, a kernel that clears the word the scan marks: all of it is recorded, and the
+    mask content may change between replays, from the interval form to a bias and back.  A replay whose mask is made
+    of intervals again must run on the interval form again (a mark left behind by the bias replay would send every
+    later replay to the mask-adding kernel): its result equals the eager call's bit for bit, and the analytic call's."""
     B, H, Hkv, S, D = 1, 4, 2, 200, 64
     q, k, v = _normal_qkv(52, B, H, Hkv, S, S, D)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
@@ -92,12 +94,20 @@ def test_masked_prefill_replayed(device):
     rng = np.random.default_rng(1)
     bias = rng.normal(0, 1, (S, S)).astype(np.float32)
     bias[:, 150:] = float("-inf")
-    for it, mask in enumerate((oracle.get_mask(S, 0), bias, oracle.get_mask(S, 0, 40), bias * 2)):
+    causal, window = oracle.get_mask(S, 0), oracle.get_mask(S, 0, 40)
+    analytic = {id(causal): (True, 0, 0), id(window): (True, 0, 40)}
+    for it, mask in enumerate((causal, bias, window, bias * 2, causal, causal)):
         _upload(device, tm, mask)
         cap.graph.launch()
         got = out.to_numpy()
         ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk")
         assert_parity(got, ref, TOL_F32, f"replay {it}")
+        fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))  # the same call, eagerly
+        eager = out.to_numpy()
+        assert np.array_equal(got.view(np.uint8), eager.view(np.uint8)), f"replay {it} differs from the eager call"
+        if id(mask) in analytic:
+            same = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic[id(mask)]).to_numpy()
+            assert np.array_equal(got.view(np.uint8), same.view(np.uint8)), f"replay {it} did not run on the interval form"
         _ = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()   # unrelated eager work between the replays
 
 

@@ -32,7 +32,7 @@ def _both(device, dtype, q, k, v, scale, mask=None, kind=None, analytic=None, ex
     args.workspace, args.workspace_bytes = ws.ptr, need.value
     if expect_kernel is not None:
         kid = ctypes.c_int32()
-        fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), device.compute_units, ctypes.byref(kid)))
+        fa.check(fa.lib().fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
         assert kid.value == expect_kernel, f"{what}: kernel {kid.value}"
     fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
     want = args._out_tensor.to_numpy()
