@@ -20,6 +20,7 @@
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199 (f32 accumulation
 // of 16-bit inputs as in fusor-ml/core/src/composite/flash_attention.rs:186-203,323-327).
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 #include "device_utils.h"
@@ -408,6 +409,8 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
 }
 
 constexpr int DM_KEYS = 32;  // keys per wavefront step
+constexpr int DM_DEPTH = 1;  // tiles in flight per wavefront beside the one in LDS (2 measured no faster: the stream
+                             // is not latency-bound with eight wavefronts per CU)
 constexpr int DM_HEADS = 16; // query heads per workgroup (MFMA N dimension)
 
 template <typename T, int D>
@@ -466,33 +469,41 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
     // one wavefront step = 32 consecutive keys; the four wavefronts interleave their steps
     const int lo_al = lo - (lo % DM_KEYS);
     const int step = DEC_WAVES * DM_KEYS;
-    uint4_t kst[NLD], vst[NLD];
-    auto load_tile = [&](int base) {
+    // Staging registers of the tiles in flight: DEPTH tiles per wavefront.
+    // Every lane always loads: a row outside [lo, hi) is replaced by the nearest one inside (its score is set to
+    // -inf below, so what it holds never counts).  Without branches around the loads the compiler can count them,
+    // and the wait in front of an LDS store is for that tile's loads only, not for everything in flight.
+    constexpr int DEPTH = DM_DEPTH;
+    uint4_t kst[DEPTH][NLD], vst[DEPTH][NLD];
+    auto load_tile = [&](int base, auto set) __attribute__((always_inline)) {
+        constexpr int S = decltype(set)::value;
 #pragma unroll
         for (int u = 0; u < NLD; u++) {
             const int cid = lane + 64 * u;
             const int row = cid / CPR, col = cid % CPR;
-            const int key = base + row;
-            kst[u] = uint4_t{0, 0, 0, 0};
-            vst[u] = uint4_t{0, 0, 0, 0};
-            if (key >= lo && key < hi) {
-                kst[u] = __builtin_nontemporal_load((const uint4_t *)(kbase + (int64_t)key * p.ks[2] + col * 8));
-                vst[u] = __builtin_nontemporal_load((const uint4_t *)(vbase + (int64_t)key * p.vs[2] + col * 8));
-            }
+            const int key = min(max(base + row, lo), hi - 1);
+            kst[S][u] = __builtin_nontemporal_load((const uint4_t *)(kbase + (int64_t)key * p.ks[2] + col * 8));
+            vst[S][u] = __builtin_nontemporal_load((const uint4_t *)(vbase + (int64_t)key * p.vs[2] + col * 8));
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](auto set) __attribute__((always_inline)) {
+        constexpr int S = decltype(set)::value;
 #pragma unroll
         for (int u = 0; u < NLD; u++) {
             const int cid = lane + 64 * u;
             const int row = cid / CPR, col = cid % CPR;
-            *DLDS_PTR(uint4_t, row * KP + col * 16) = kst[u];
-            *DLDS_PTR(uint4_t, K_BYTES + row * VP + col * 16) = vst[u];
+            *DLDS_PTR(uint4_t, row * KP + col * 16) = kst[S][u];
+            *DLDS_PTR(uint4_t, K_BYTES + row * VP + col * 16) = vst[S][u];
         }
     };
+    using set0 = std::integral_constant<int, 0>;
+    using set1 = std::integral_constant<int, DEPTH - 1>;
 
     int base = lo_al + wave * DM_KEYS;
-    if (base < hi) load_tile(base);  // issued first so the Q fetch below overlaps it
+    if (base < hi) {  // issued first so the Q fetch below overlaps them
+        load_tile(base, set0{});
+        if constexpr (DEPTH == 2) load_tile(base + step, set1{});
+    }
 
     // Q^T operand: head j, dims 32 kb + 8 q4 .. +8 (zero for the padding heads)
     vec8 qreg[KB];
@@ -519,11 +530,12 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
         }
     }
 
-    for (; base < hi; base += step) {
+    // one step: the staged tile `set` (keys base ..) goes to LDS, its registers take the tile DEPTH steps ahead, then the math
+    auto one_step = [&](int base, auto set) __attribute__((always_inline)) {
         wave_lds_sync();  // the previous step's LDS reads precede these writes
-        store_tile();
+        store_tile(set);
         wave_lds_sync();
-        if (base + step < hi) load_tile(base + step);  // in flight during the math below
+        load_tile(base + DEPTH * step, set);  // in flight during the math below (beyond the end: a row read again)
 
         // ---- S^T[key][head] = K . Q^T : two 16-key tiles --------------------------------------------
         float4_t s[2];
@@ -587,6 +599,11 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
             const uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
             o[nb] = DecMma<T>::mfma(__builtin_bit_cast(vec8, araw), pop, o[nb]);
         }
+    };
+    for (; base < hi; base += DEPTH * step) {
+        one_step(base, set0{});
+        if constexpr (DEPTH == 2)
+            if (base + step < hi) one_step(base + step, set1{});
     }
 
     // ---- merge: key groups -> wavefront -> workgroup ------------------------------------------------
