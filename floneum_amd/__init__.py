@@ -207,11 +207,12 @@ class Device:
 
     _default = None
 
-    def __init__(self, ordinal=0):
+    def __init__(self, ordinal=0, handle=None):
         L = lib()
-        h = ctypes.c_void_p()
-        check(L.fhip_device_create(ordinal, ctypes.byref(h)))
-        self.handle = h
+        if handle is None:
+            handle = ctypes.c_void_p()
+            check(L.fhip_device_create(ordinal, ctypes.byref(handle)))
+        self.handle = handle
         s = ctypes.c_void_p()
         check(L.fhip_stream_create(self.handle, ctypes.byref(s)))
         self.stream = s
@@ -224,12 +225,22 @@ class Device:
         self._workspace = None
         self._workspace_bytes = 0
         self._pool, self._sizes, self._pooled = {}, {}, 0  # cached free blocks by size, block sizes, bytes cached
+        # A recorded graph keeps the POINTERS of the buffers and of the workspace its calls used, not the buffers:
+        # while a capture is open or a Graph of this device is alive, freed blocks are parked instead of being
+        # handed out again (a replay would overwrite their new owner's data), and the workspace is neither
+        # recycled nor grown under a capture.
+        self._capturing, self._graphs_alive, self._parked = False, 0, []
 
     @classmethod
     def default(cls):
         if cls._default is None:
             cls._default = cls(0)
         return cls._default
+
+    def with_new_stream(self):
+        """The same device handle with a stream, allocation cache and workspace of its own: what a second host
+        thread uses (one stream and one workspace belong to one thread at a time)."""
+        return Device(handle=self.handle)
 
     @staticmethod
     def count():
@@ -255,6 +266,9 @@ class Device:
         return p.value
 
     def free(self, ptr):
+        if self._capturing or self._graphs_alive > 0:
+            self._parked.append(ptr)
+            return
         size = self._sizes.get(ptr)
         if size is not None and self._pooled + size <= self._CACHE_LIMIT:
             self._pool.setdefault(size, []).append(ptr)
@@ -262,6 +276,13 @@ class Device:
             return
         self._sizes.pop(ptr, None)
         check(lib().fhip_free(self.handle, ctypes.c_void_p(ptr)))
+
+    def _graph_gone(self):
+        self._graphs_alive -= 1
+        if self._graphs_alive == 0 and not self._capturing:
+            parked, self._parked = self._parked, []
+            for ptr in parked:
+                self.free(ptr)
 
     def release_cached_memory(self):
         """Give the cached blocks back to the driver."""
@@ -282,9 +303,13 @@ class Device:
         """A grow-only scratch buffer owned by the device object (the caller of the C ABI owns the
         workspace; this is the Python caller's)."""
         if nbytes > self._workspace_bytes:
+            if self._capturing:
+                raise FhipError(ERR_WORKSPACE, f"the workspace would have to grow to {nbytes} bytes inside a capture "
+                                "(allocation and synchronisation are not recordable): run the call once eagerly first")
             if self._workspace:
-                self.synchronize()
-                self.free(self._workspace)
+                if self._graphs_alive == 0:
+                    self.synchronize()
+                self.free(self._workspace)  # parked while a graph that recorded it is alive
             self._workspace = self.malloc(nbytes)
             self._workspace_bytes = nbytes
         return self._workspace, self._workspace_bytes
@@ -295,6 +320,7 @@ class Graph:
 
     def __init__(self, device, handle):
         self.device, self.handle = device, handle
+        device._graphs_alive += 1
 
     def launch(self):
         check(lib().fhip_graph_launch(self.handle, self.device.stream))
@@ -304,6 +330,7 @@ class Graph:
             if self.handle:
                 lib().fhip_graph_destroy(self.handle)
                 self.handle = None
+                self.device._graph_gone()
         except Exception:
             pass
 
@@ -314,14 +341,22 @@ class _Capture:
 
     def __enter__(self):
         check(lib().fhip_stream_begin_capture(self.device.stream))
+        self.device._capturing = True
         return self
 
     def __exit__(self, exc_type, exc, tb):
         h = ctypes.c_void_p()
         rc = lib().fhip_stream_end_capture(self.device.stream, ctypes.byref(h))
+        self.device._capturing = False
         if exc_type is None:
             check(rc)
             self.graph = Graph(self.device, h)
+        else:
+            if rc == OK and h:
+                lib().fhip_graph_destroy(h)  # the body raised: what was recorded so far is dropped
+            if self.device._graphs_alive == 0:
+                self.device._graphs_alive = 1  # hand the blocks parked during the failed capture back
+                self.device._graph_gone()
         return False
 
 

@@ -1115,6 +1115,32 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
     const fhip_tensor4 *news[2] = {k_new, v_new};
     fhip_tensor4 *alls[2] = {k_all, v_all};
 
+    // Branches that move the cache into new buffers allocate both sides' buffers before anything is queued and
+    // install them only after every launch into them was accepted: a failure on the way frees them and leaves the
+    // cache (buffers, lengths, strides) exactly as it was.
+    void *nb[2] = {nullptr, nullptr};
+    auto drop_new = [&]() {
+        for (int sd = 0; sd < 2; sd++)
+            if (nb[sd]) (void)hipFree(nb[sd]);
+    };
+    auto alloc_new = [&](size_t bytes) -> int {
+        for (int sd = 0; sd < 2; sd++) {
+            const hipError_t e = hipMalloc(&nb[sd], bytes);
+            if (e != hipSuccess) {
+                nb[sd] = nullptr;
+                drop_new();
+                return fhip::hip_fail(e, "hipMalloc (KV cache buffers)");
+            }
+        }
+        return FHIP_OK;
+    };
+    auto install_new = [&]() {
+        for (int sd = 0; sd < 2; sd++) {
+            if (c->side[sd].buf) (void)hipFree(c->side[sd].buf);  // waits for the copies out of it
+            c->side[sd].buf = nb[sd];
+        }
+    };
+
     if (required > c->max_len) {
         // keep the last max_len positions of old[new_start..] ++ new (tensor_cache.rs:55-78)
         const uint64_t mx = c->max_len, cap = 2 * mx;
@@ -1125,47 +1151,55 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
         int64_t cap_st[4];
         kv_contig_strides(c, cap, cap_st);
         uint64_t start_after = 0;
-        for (int sd = 0; sd < 2; sd++) {
-            fhip_tensor_cache_side &S = c->side[sd];
-            if (!c->sliding) {
-                // the cache has just filled up: move what is kept into a buffer with room to slide
-                void *nb = nullptr;
-                FHIP_HIP_CHECK(hipMalloc(&nb, row_elems * cap * eb));
+        if (!c->sliding) {
+            // the cache has just filled up: move what is kept into buffers with room to slide
+            int rc = alloc_new(row_elems * cap * eb);
+            if (rc) return rc;
+            for (int sd = 0; sd < 2 && !rc; sd++) {
                 if (keep_old) {
                     int64_t src_st[4];
                     kv_contig_strides(c, c->allocated, src_st);
                     const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
-                    int rc = launch_copy_rows((const char *)S.buf + new_start * c->D * eb, src_st, nb, cap_st, shp, eb, s->s);
-                    if (rc) return rc;
+                    rc = launch_copy_rows((const char *)c->side[sd].buf + new_start * c->D * eb, src_st, nb[sd], cap_st, shp,
+                                          eb, s->s);
                 }
-                int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
-                                        (char *)nb + keep_old * c->D * eb, cap_st, nr);
-                if (rc) return rc;
-                if (S.buf) FHIP_HIP_CHECK(hipFree(S.buf));  // waits for the copy
-                S.buf = nb;
-                start_after = 0;
-            } else if (behind) {
-                // keep_old > 0 here, so every new row is kept
-                int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n,
-                                        (char *)S.buf + (c->start + c->current) * c->D * eb, cap_st, nr);
-                if (rc) return rc;
-                start_after = c->start + new_start;
-            } else {
-                // the end of the buffer: the kept rows go back to row 0 (they lie beyond row max_len - n, so source
-                // and destination do not overlap), the new ones behind them
-                if (keep_old) {
-                    const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
-                    int rc = launch_copy_rows((const char *)S.buf + (c->start + new_start) * c->D * eb, cap_st, S.buf, cap_st,
-                                              shp, eb, s->s);
-                    if (rc) return rc;
-                }
-                int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
-                                        (char *)S.buf + keep_old * c->D * eb, cap_st, nr);
-                if (rc) return rc;
-                start_after = 0;
+                if (!rc)
+                    rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
+                                        (char *)nb[sd] + keep_old * c->D * eb, cap_st, nr);
             }
-            kv_view(c, S.buf, cap, mx, alls[sd], start_after);
+            if (rc) {
+                (void)hipStreamSynchronize(s->s);  // nothing queued may still write into the buffers being dropped
+                drop_new();
+                if (first) c->B = c->Hkv = c->D = 0;  // still empty
+                return rc;
+            }
+            install_new();
+        } else {
+            for (int sd = 0; sd < 2; sd++) {
+                fhip_tensor_cache_side &S = c->side[sd];
+                if (behind) {
+                    // keep_old > 0 here, so every new row is kept
+                    int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n,
+                                            (char *)S.buf + (c->start + c->current) * c->D * eb, cap_st, nr);
+                    if (rc) return rc;
+                    start_after = c->start + new_start;
+                } else {
+                    // the end of the buffer: the kept rows go back to row 0 (they lie beyond row max_len - n, so source
+                    // and destination do not overlap), the new ones behind them
+                    if (keep_old) {
+                        const uint32_t shp[4] = {c->B, c->Hkv, (uint32_t)keep_old, c->D};
+                        int rc = launch_copy_rows((const char *)S.buf + (c->start + new_start) * c->D * eb, cap_st, S.buf,
+                                                  cap_st, shp, eb, s->s);
+                        if (rc) return rc;
+                    }
+                    int rc = write_new_rows(c, s->s, sd, news[sd], n - take_new, (uint32_t)take_new,
+                                            (char *)S.buf + keep_old * c->D * eb, cap_st, nr);
+                    if (rc) return rc;
+                    start_after = 0;
+                }
+            }
         }
+        for (int sd = 0; sd < 2; sd++) kv_view(c, c->side[sd].buf, cap, mx, alls[sd], start_after);
         c->sliding = true;
         c->start = start_after;
         c->current = mx;
@@ -1175,15 +1209,18 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
 
     if (first) {
         // first append stores the tensor as it is (tensor_cache.rs:111-116)
-        for (int sd = 0; sd < 2; sd++) {
-            fhip_tensor_cache_side &S = c->side[sd];
-            FHIP_HIP_CHECK(hipMalloc(&S.buf, row_elems * n * eb));
-            int64_t dst_st[4];
-            kv_contig_strides(c, n, dst_st);
-            int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, S.buf, dst_st, nr);
-            if (rc) return rc;
-            kv_view(c, S.buf, n, n, alls[sd]);
+        int rc = alloc_new(row_elems * n * eb);
+        int64_t dst_st[4];
+        kv_contig_strides(c, n, dst_st);
+        for (int sd = 0; sd < 2 && !rc; sd++) rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, nb[sd], dst_st, nr);
+        if (rc) {
+            (void)hipStreamSynchronize(s->s);
+            drop_new();
+            c->B = c->Hkv = c->D = 0;  // still empty
+            return rc;
         }
+        install_new();
+        for (int sd = 0; sd < 2; sd++) kv_view(c, c->side[sd].buf, n, n, alls[sd]);
         c->current = n;
         c->allocated = n;
         return FHIP_OK;
@@ -1191,30 +1228,37 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
 
     uint64_t alloc = c->allocated;
     if (required > c->allocated) alloc = next_pow2(required);  // tensor_cache.rs:80-96
-    for (int sd = 0; sd < 2; sd++) {
-        fhip_tensor_cache_side &S = c->side[sd];
-        int64_t dst_st[4];
-        kv_contig_strides(c, alloc, dst_st);
-        if (alloc != c->allocated) {
-            void *nb = nullptr;
-            FHIP_HIP_CHECK(hipMalloc(&nb, row_elems * alloc * eb));
-            int64_t src_st[4];
-            kv_contig_strides(c, c->allocated, src_st);
-            const uint32_t shp_old[4] = {c->B, c->Hkv, (uint32_t)c->current, c->D};
-            int rc = launch_copy_rows(S.buf, src_st, nb, dst_st, shp_old, eb, s->s);
-            if (rc) return rc;
-            if (alloc > required) {  // the reference concatenates zeros behind the data
-                const uint32_t shp_z[4] = {c->B, c->Hkv, (uint32_t)(alloc - required), c->D};
-                rc = launch_fill_zero_rows((char *)nb + required * c->D * eb, dst_st, shp_z, eb, s->s);
-                if (rc) return rc;
-            }
-            FHIP_HIP_CHECK(hipFree(S.buf));  // waits for the copy
-            S.buf = nb;
-        }
-        int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, (char *)S.buf + c->current * c->D * eb, dst_st, nr);
+    int64_t dst_st[4];
+    kv_contig_strides(c, alloc, dst_st);
+    if (alloc != c->allocated) {
+        int rc = alloc_new(row_elems * alloc * eb);
         if (rc) return rc;
-        kv_view(c, S.buf, alloc, required, alls[sd]);
+        int64_t src_st[4];
+        kv_contig_strides(c, c->allocated, src_st);
+        for (int sd = 0; sd < 2 && !rc; sd++) {
+            const uint32_t shp_old[4] = {c->B, c->Hkv, (uint32_t)c->current, c->D};
+            rc = launch_copy_rows(c->side[sd].buf, src_st, nb[sd], dst_st, shp_old, eb, s->s);
+            if (!rc && alloc > required) {  // the reference concatenates zeros behind the data
+                const uint32_t shp_z[4] = {c->B, c->Hkv, (uint32_t)(alloc - required), c->D};
+                rc = launch_fill_zero_rows((char *)nb[sd] + required * c->D * eb, dst_st, shp_z, eb, s->s);
+            }
+            if (!rc)
+                rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, (char *)nb[sd] + c->current * c->D * eb, dst_st, nr);
+        }
+        if (rc) {
+            (void)hipStreamSynchronize(s->s);
+            drop_new();
+            return rc;
+        }
+        install_new();
+    } else {
+        for (int sd = 0; sd < 2; sd++) {
+            int rc = write_new_rows(c, s->s, sd, news[sd], 0, (uint32_t)n, (char *)c->side[sd].buf + c->current * c->D * eb,
+                                    dst_st, nr);
+            if (rc) return rc;
+        }
     }
+    for (int sd = 0; sd < 2; sd++) kv_view(c, c->side[sd].buf, alloc, required, alls[sd]);
     c->current = required;
     c->allocated = alloc;
     return FHIP_OK;

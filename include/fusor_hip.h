@@ -19,9 +19,11 @@
  *   - The library never allocates or frees caller tensors.  The output buffer and the workspace
  *     are supplied by the caller.  Launches are asynchronous on the given stream.
  *   - Re-entrant: the only mutable state lives in the handles (a device handle holds an atomic counter that
- *     numbers masked prefill calls, a KV cache its buffers) and in the thread-local error string; there are no
- *     global variables.  Calls on different streams may run concurrently from different threads; one stream, one
- *     KV cache and one workspace are used by one thread at a time.
+ *     numbers masked prefill calls, a KV cache its buffers) and in the thread-local error string.  The one
+ *     file-scope object is the fixed device array behind fhip_flash_attention_noalloc (one copy per GPU, shared
+ *     by that GPU's calls of that function only).  Calls on different streams may run concurrently from different
+ *     threads, also on one device handle; one stream, one KV cache and one workspace are used by one thread at a
+ *     time.
  */
 #ifndef FUSOR_HIP_H
 #define FUSOR_HIP_H
@@ -280,7 +282,9 @@ int fhip_kv_cache_current_seq_len(const fhip_kv_cache *c, uint64_t *len);
 int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len);
 /* k_new, v_new: [B, Hkv, n, D] strided device views of the cache dtype.  On return k_all/v_all
  * describe the cached keys/values including the new rows (views into cache-owned memory, valid
- * until the next append/reset/destroy). */
+ * until the next append/reset/destroy: an append that grows the allocation, and the first one that
+ * makes a full cache slide, move the rows to new buffers and free the old ones).  An append that
+ * fails leaves the cache as it was. */
 int fhip_kv_cache_append(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *k_new,
                          const fhip_tensor4 *v_new, fhip_tensor4 *k_all, fhip_tensor4 *v_all);
 

@@ -146,3 +146,48 @@ def test_memset_is_a_kernel_and_replays(device):
         device.synchronize()
         cap.graph.launch()
         assert np.array_equal(read(), want)
+
+
+def test_blocks_freed_after_capture_are_not_reused_while_the_graph_lives(device):
+    """The Python mirror caches freed device blocks by size.  A graph holds the pointers its calls recorded, not the
+    buffers: a tensor freed after the capture must not be handed to a new tensor while the graph can still be
+    replayed (the replay would write into the new owner's memory), and the device's workspace must neither be
+    recycled nor grow inside a capture."""
+    B, H, Hkv, S, D = 2, 8, 2, 1500, 128
+    q, k, v = _normal_qkv(77, B, H, Hkv, 1, S, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))
+    first = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()  # eager: sizes the device's workspace
+    ws_before = device.workspace(0)
+    with device.capture() as cap:
+        out = tq.flash_attention(tk, tv, D ** -0.5)            # the mirror's convenience call: output from the pool
+    out_ptr, nbytes = out.buffer.ptr, out.buffer.nbytes
+    del out                                                    # back to the mirror, but not for reuse yet
+    squatter = fa.Tensor.empty(device, (B, H, 1, D), fa.F16)   # same size: would have received the freed block
+    assert squatter.buffer.nbytes == nbytes and squatter.buffer.ptr != out_ptr
+    pattern = np.full((B, H, 1, D), 7.0, np.float16)
+    _upload(device, squatter, pattern)
+    cap.graph.launch()
+    device.synchronize()
+    assert np.array_equal(squatter.to_numpy(), pattern), "a replay wrote into a tensor allocated after the capture"
+    # the replay's own output is still where the graph put it
+    host = np.empty((B, H, 1, D), np.float16)
+    fa.check(fa.lib().fhip_memcpy_d2h(device.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(out_ptr), host.nbytes))
+    assert np.array_equal(host.view(np.uint8), first.view(np.uint8))
+    # a larger call while the graph lives: the old workspace is parked, not reused; the replay still works
+    k2, v2 = (fa.Tensor.from_numpy(device, np.concatenate([a, a, a, a], 2), fa.F16) for a in (k, v))
+    _ = tq.flash_attention(k2, v2, D ** -0.5).to_numpy()
+    assert ws_before[0] in device._parked or device.workspace(0)[0] == ws_before[0]
+    cap.graph.launch()
+    fa.check(fa.lib().fhip_memcpy_d2h(device.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(out_ptr), host.nbytes))
+    assert np.array_equal(host.view(np.uint8), first.view(np.uint8))
+    # growing the workspace inside a capture is refused (it would allocate and synchronise)
+    k3, v3 = (fa.Tensor.from_numpy(device, np.concatenate([a] * 16, 2), fa.F16) for a in (k, v))
+    out3 = fa.Tensor.empty(device, (B, H, 1, D), fa.F16)
+    with pytest.raises(fa.FhipError, match="inside a capture"):
+        with device.capture():
+            tq.flash_attention(k3, v3, D ** -0.5, out=out3)
+    parked = len(device._parked)
+    del cap                                                    # the last graph goes: parked blocks return to the cache
+    import gc
+    gc.collect()
+    assert device._graphs_alive == 0 and (parked == 0 or len(device._parked) < parked)
