@@ -88,6 +88,9 @@ def configs():
         "S1": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
         "S2": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
         "S3": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=32768, D=128, dtype="f16", std=0.5, causal=False),
+        # a multi-token decode step: C2's batch with four new rows per sequence at the end of the cache, causal among
+        # themselves (a draft being verified); the rows ride beside the heads of a GQA group, the cache is read once
+        "M1": dict(kind="decode", B=16, H=32, Hkv=8, Sq=4, Skv=4096, D=128, dtype="f16", std=0.5, causal=True),
     }
 
 
@@ -219,6 +222,14 @@ def time_config(fa, dev, c, blocks, steps, warmup):
     return wall_ms, kernel_ms
 
 
+def _decode_rows_mask(c, n):
+    """[Sq, n] mask of a multi-token decode step (row r sits at position n - Sq + r); None for a plain step."""
+    if not c["causal"]:
+        return None
+    i = np.arange(c["Sq"])[:, None] + (n - c["Sq"])
+    return np.where(np.arange(n)[None, :] > i, -np.inf, 0.0).astype(np.float32)
+
+
 def parity_spot_check(fa, oracle, c, out_t, host, lens):
     """A few output rows of the timed workload against the CPU checker (cheap: rows are independent)."""
     q, k, v = host
@@ -229,8 +240,9 @@ def parity_spot_check(fa, oracle, c, out_t, host, lens):
         worst = 0.0
         for b in bs:
             n = int(lens[b]) if lens is not None else c["Skv"]
+            mask = _decode_rows_mask(c, n)
             ref = oracle.flash_attention(f32(q[b:b + 1]), f32(k[b:b + 1, :, :n]), f32(v[b:b + 1, :, :n]),
-                                         c["D"] ** -0.5)
+                                         c["D"] ** -0.5, mask, None if mask is None else "qk")
             worst = max(worst, float(np.abs(out[b:b + 1] - ref).max()))
         return worst
     q, k, v = f32(q), f32(k), f32(v)
@@ -273,10 +285,12 @@ def cpu_baseline(oracle, c, host, lens, flops, byts):
                         sample=sample)
         reps, dts = 3, []
         q, k, v = f32(q), f32(k), f32(v)
-        oracle.flash_attention(q, k, v, scale)
+        mask = _decode_rows_mask(c, c["Skv"])
+        kind = None if mask is None else "qk"
+        oracle.flash_attention(q, k, v, scale, mask, kind)
         for _ in range(reps):
             t0 = time.perf_counter()
-            oracle.flash_attention(q, k, v, scale)
+            oracle.flash_attention(q, k, v, scale, mask, kind)
             dts.append(time.perf_counter() - t0)
         return dict(value=byts / float(np.median(dts)) / 1e9, unit="GB/s", cores=threads, kind="port",
                     sample=f"the full step (all {c['B']} sequences), f16 upcast to f32 first, median of {reps} passes "

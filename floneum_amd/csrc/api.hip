@@ -190,9 +190,14 @@ static bool rows_vectorizable(const fhip_tensor4 &t, int eb, int bytes = 16) {
     return true;
 }
 
+// Query rows per sequence the split-KV decode kernels take: the single row of a decode step, and the few rows of a
+// multi-token step (a draft being verified, a short piece of a prompt), which ride as further columns beside the
+// query heads that share a KV head.
+constexpr uint32_t DECODE_MAX_ROWS = 4;
+
 static bool decode_eligible(const fhip_attn_args *a) {
     const uint32_t D = a->q.shape[3];
-    if (a->q.shape[2] != 1) return false;
+    if (a->q.shape[2] < 1 || a->q.shape[2] > DECODE_MAX_ROWS) return false;
     if (D % 8 != 0 || D < 8 || D > 256) return false;
     const int eb = a->dtype == FHIP_F32 ? 4 : 2;
     if (!rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;
@@ -687,9 +692,10 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
         int chunk, nsplit;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
-        const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2];
-        decode_plan(B, Hkv, H / Hkv, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr, args->dtype == FHIP_F32, &chunk, &nsplit);
-        *bytes = decode_workspace_bytes(B, H, Hkv, D, nsplit);
+        const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2], rows = (int)args->q.shape[2];
+        decode_plan(B, Hkv, H / Hkv * rows, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr,
+                    args->dtype == FHIP_F32, &chunk, &nsplit);
+        *bytes = decode_workspace_bytes(B, H * rows, Hkv, D, nsplit);
     }
     return FHIP_OK;
 }
@@ -787,8 +793,9 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
-            decode_plan(p.B, p.Hkv, p.G, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr, args->dtype == FHIP_F32, &p.chunk, &p.nsplit);
-            const size_t need = decode_workspace_bytes(p.B, p.H, p.Hkv, p.D, p.nsplit);
+            decode_plan(p.B, p.Hkv, p.G * p.Sq, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr,
+                        args->dtype == FHIP_F32, &p.chunk, &p.nsplit);
+            const size_t need = decode_workspace_bytes(p.B, p.H * p.Sq, p.Hkv, p.D, p.nsplit);
             if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
                 set_error("decode needs a workspace of %zu bytes, got %zu", need,
                           args->workspace ? args->workspace_bytes : (size_t)0);

@@ -192,13 +192,17 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
     // first splits of a row of the grid have keys: taken as they come, XCD 0 would get up to one more busy
     // workgroup per (batch, head) than XCD 7.  Rotating the split by the row spreads them evenly.
     const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);
-    const int HB = (p.G + GT - 1) / GT;
+    // A workgroup serves up to GT columns = (query head, query row) pairs that share the KV head: column c is head
+    // c / rows, row c % rows of the group (one row per head in a plain decode step, a few in a multi-token step).
+    const int rows = p.Sq;
+    const int NC = p.G * rows;
+    const int HB = (NC + GT - 1) / GT;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
-    const int h0 = g * p.G + hb * GT;            // first query head of this block
-    const int nh = min(GT, p.G - hb * GT);       // real heads in this block
+    const int c0 = hb * GT;                      // first column of this block
+    const int nh = min(GT, NC - c0);             // columns in use
 
     // visible key range of this workgroup
     int kv_hi = p.Skv;
@@ -207,19 +211,31 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
         kv_hi = min(kv_hi, max(len, 0));
     }
     if (p.kv_lens && split * p.chunk >= kv_hi && split > 0) return;  // beyond this sequence: the combine skips it
+    // [lo, hi): the keys some row sees.  Row r sees key j when j - r lies in [first, limit): the causal limit and the
+    // start of the window move with the row (limits that do not apply are set out of reach).
     int lo = split * p.chunk;
     int hi = min(lo + p.chunk, kv_hi);
+    int limit = 0x3fffffff, first = -0x3fffffff;
     if (p.analytic) {
-        if (p.causal) hi = (int)min((int64_t)hi, p.q_pos_offset + 1);
-        if (p.window > 0) lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
+        if (p.causal) {
+            limit = (int)min((int64_t)limit, p.q_pos_offset + 1);
+            hi = (int)min((int64_t)hi, p.q_pos_offset + rows);
+        }
+        if (p.window > 0) {
+            first = (int)max((int64_t)first, p.q_pos_offset - p.window + 1);
+            lo = max(lo, first);
+        }
     }
 
-    // query rows of the GT heads: the 8 elements this lane owns
+    // query rows of the GT columns: the 8 elements this lane owns
     Vec8<T> q[GT];
+    int rr[GT];  // query row of each column
 #pragma unroll
     for (int hh = 0; hh < GT; hh++) {
-        const int h = h0 + min(hh, nh - 1);
-        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1];
+        const int col = c0 + min(hh, nh - 1);
+        const int h = g * p.G + col / rows;
+        rr[hh] = col % rows;
+        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)rr[hh] * p.qs[2];
         q[hh].zero();
         if (active) {
             // one 16 / 32-byte load when the row is contiguous and aligned, element by element otherwise
@@ -233,6 +249,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
     const T *mrow = nullptr;
     if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask;
     if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const T *)p.mask + b * p.ms0;
+    const bool row_masks = rows > 1 && p.mask_kind == FHIP_MASK_QK;  // every query row has its own mask row
     const float scale2 = p.scale * LOG2E;
 
     float m[GT], l[GT], acc[GT][8];
@@ -265,12 +282,16 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
         for (int u = 0; u < U; u++) {
             const bool visible = key[u] >= lo && key[u] < hi;
             float bias = 0.0f;
-            if (mrow && visible) bias = to_float(mrow[(int64_t)key[u] * p.ms1]) * LOG2E;
+            if (mrow && visible && !row_masks) bias = to_float(mrow[(int64_t)key[u] * p.ms1]) * LOG2E;
 #pragma unroll
             for (int hh = 0; hh < GT; hh++) {
                 float d = lpk_sum<LPK>(kk[u].dot(q[hh], 0.0f));
-                d = d * scale2 + bias;
-                s[u][hh] = visible ? d : -INFINITY;
+                const int rel = key[u] - rr[hh];
+                const bool vis = visible && rel < limit && rel >= first;
+                float bh = bias;
+                if (row_masks && vis) bh = to_float(mrow[(int64_t)rr[hh] * p.ms0 + (int64_t)key[u] * p.ms1]) * LOG2E;
+                d = d * scale2 + bh;
+                s[u][hh] = vis ? d : -INFINITY;
             }
         }
 #pragma unroll
@@ -347,14 +368,14 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void decode_vec_kernel(AttnParams p
             L += wgt * lds_ml[w][hh][1];
             A += wgt * lds_acc[w][hh][d];
         }
-        const int h = h0 + hh;
+        const int h = g * p.G + (c0 + hh) / rows, qr = (c0 + hh) % rows;
         if (p.nsplit == 1) {
             const float o = A / L;  // no visible key: 0/0 = NaN like the reference
-            const int64_t oi = b * p.os[0] + h * p.os[1] + d * p.os[3];
+            const int64_t oi = b * p.os[0] + h * p.os[1] + qr * p.os[2] + d * p.os[3];
             if (p.out_f32) ((float *)p.out)[oi] = o;
             else ((T *)p.out)[oi] = from_float<T>(o);
         } else {
-            float *ws = (float *)p.partials + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
+            float *ws = (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
             ws[d] = A;
             if (d == 0) {
                 ws[D] = M;
@@ -436,28 +457,42 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
     const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
-    const int HB = (p.G + DM_HEADS - 1) / DM_HEADS;
+    // The MFMA columns are the (query head, query row) pairs that share this KV head: column c is head c / rows,
+    // row c % rows of the group (one row per head in a plain decode step, a few in a multi-token step).
+    const int rows = p.Sq;
+    const int NC = p.G * rows;
+    const int HB = (NC + DM_HEADS - 1) / DM_HEADS;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
-    const int h0 = g * p.G + hb * DM_HEADS;
-    const int nh = min(DM_HEADS, p.G - hb * DM_HEADS);
+    const int c0 = hb * DM_HEADS;
+    const int nh = min(DM_HEADS, NC - c0);  // columns in use
+    const int cj = c0 + min(j, nh - 1);     // this lane's column
+    const int hj = g * p.G + cj / rows, rj = cj % rows;
 
     int kv_hi = p.Skv;
     if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
     if (p.kv_lens && split * p.chunk >= kv_hi && split > 0) return;  // the combine pass skips it too
+    // [lo, hi): the keys some row of the workgroup sees; [lo_j, hi_j): the keys this lane's row sees
     int lo = split * p.chunk;
     int hi = min(lo + p.chunk, kv_hi);
+    int lo_j = lo, hi_j = hi;
     if (p.analytic) {
-        if (p.causal) hi = (int)min((int64_t)hi, p.q_pos_offset + 1);
-        if (p.window > 0) lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
+        if (p.causal) {
+            hi_j = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj);
+            hi = (int)min((int64_t)hi, p.q_pos_offset + rows);  // the last row sees furthest
+        }
+        if (p.window > 0) {
+            lo_j = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj);
+            lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);  // the first row sees the earliest key
+        }
     }
 
     const uint16_t *kbase = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
     const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
     const T *mrow = nullptr;
-    if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask;
+    if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask + rj * p.ms0;
     if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const T *)p.mask + b * p.ms0;
     const float scale2 = p.scale * LOG2E;
 
@@ -505,10 +540,10 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
         if constexpr (DEPTH == 2) load_tile(base + step, set1{});
     }
 
-    // Q^T operand: head j, dims 32 kb + 8 q4 .. +8 (zero for the padding heads)
+    // Q^T operand: column j, dims 32 kb + 8 q4 .. +8 (zero for the padding columns)
     vec8 qreg[KB];
     {
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + (int64_t)(h0 + min(j, nh - 1)) * p.qs[1];
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + (int64_t)hj * p.qs[1] + (int64_t)rj * p.qs[2];
         const bool qvec = p.qs[3] == 1 && (((uintptr_t)qp) & 15) == 0;
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
@@ -548,14 +583,14 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
                 s[t] = DecMma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], s[t]);
             }
         }
-        // element (t, r) is key base + 16 t + 4 q4 + r for head j
+        // element (t, r) is key base + 16 t + 4 q4 + r for column j
         float sv[8];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int key = base + 16 * t + 4 * q4 + r;
-                const bool visible = key >= lo && key < hi;
+                const bool visible = key >= lo_j && key < hi_j;
                 float x = s[t][r] * scale2;
                 if (mrow && visible) x += to_float(mrow[(int64_t)key * p.ms1]) * LOG2E;
                 sv[4 * t + r] = visible ? x : -INFINITY;
@@ -636,14 +671,14 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
             L += wgt * src[D + 1];
             A += wgt * src[d];
         }
-        const int h = h0 + hh;
+        const int h = g * p.G + (c0 + hh) / rows, qr = (c0 + hh) % rows;
         if (p.nsplit == 1) {
             const float val = A / L;  // no visible key: 0/0 = NaN like the reference
-            const int64_t oi = b * p.os[0] + h * p.os[1] + d * p.os[3];
+            const int64_t oi = b * p.os[0] + h * p.os[1] + qr * p.os[2] + d * p.os[3];
             if (p.out_f32) ((float *)p.out)[oi] = val;
             else ((T *)p.out)[oi] = from_float<T>(val);
         } else {
-            float *ws = (float *)p.partials + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
+            float *ws = (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
             ws[d] = A;
             if (d == 0) {
                 ws[D] = M;
@@ -659,7 +694,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
 
 template <typename T, int U>
 __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
-    const int bh = blockIdx.x;
+    const int qr = blockIdx.x % p.Sq, bh = blockIdx.x / p.Sq;  // one workgroup per (batch, head, query row)
     const int h = bh % p.H, b = bh / p.H;
     const int D = p.D;
     int ns = p.nsplit;
@@ -667,8 +702,8 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
         const int len = min(p.Skv, max(p.kv_lens[b], 0));
         ns = max(1, min(ns, (len + p.chunk - 1) / p.chunk));  // split 0 is always written
     }
-    const float *ws = (const float *)p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
-    const int64_t ob = b * p.os[0] + h * p.os[1];
+    const float *ws = (const float *)p.partials + (int64_t)blockIdx.x * p.nsplit * (D + 2);
+    const int64_t ob = b * p.os[0] + h * p.os[1] + qr * p.os[2];
     // 128 dims per round (one round up to head_dim 128, two at 256)
     for (int dbase = 0; dbase < D; dbase += 128) {
         const int d0 = dbase + threadIdx.x, d1 = dbase + threadIdx.x + 64;
@@ -720,7 +755,7 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(AttnParams p) {
 template <typename T, int U>
 __global__ __launch_bounds__(256) void decode_combine4_kernel(AttnParams p) {
     __shared__ float part[4][2 + 128];
-    const int bh = blockIdx.x;
+    const int qr = blockIdx.x % p.Sq, bh = blockIdx.x / p.Sq;  // one workgroup per (batch, head, query row)
     const int h = bh % p.H, b = bh / p.H;
     const int D = p.D;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -729,8 +764,8 @@ __global__ __launch_bounds__(256) void decode_combine4_kernel(AttnParams p) {
         const int len = min(p.Skv, max(p.kv_lens[b], 0));
         ns = max(1, min(ns, (len + p.chunk - 1) / p.chunk));  // split 0 is always written
     }
-    const float *ws = (const float *)p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
-    const int64_t ob = b * p.os[0] + h * p.os[1];
+    const float *ws = (const float *)p.partials + (int64_t)blockIdx.x * p.nsplit * (D + 2);
+    const int64_t ob = b * p.os[0] + h * p.os[1] + qr * p.os[2];
     const int per = (ns + 3) / 4, s_lo = wave * per, s_hi = min(ns, s_lo + per);
     for (int dbase = 0; dbase < D; dbase += 128) {
         const int d0 = dbase + lane, d1 = dbase + lane + 64;
@@ -800,10 +835,10 @@ __global__ __launch_bounds__(256) void decode_combine4_kernel(AttnParams p) {
 
 template <typename T>
 static void launch_combine(const AttnParams &p, hipStream_t stream) {
-    const dim3 grid((unsigned)(p.B * p.H)), block(64);
+    const dim3 grid((unsigned)(p.B * p.H * p.Sq)), block(64);
     const int cus = p.cus > 0 ? p.cus : 256;
     if (p.nsplit <= 8) hipLaunchKernelGGL((decode_combine_kernel<T, 8>), grid, block, 0, stream, p);
-    else if ((long)p.B * p.H > 2L * cus) hipLaunchKernelGGL((decode_combine_kernel<T, 32>), grid, block, 0, stream, p);
+    else if ((long)p.B * p.H * p.Sq > 2L * cus) hipLaunchKernelGGL((decode_combine_kernel<T, 32>), grid, block, 0, stream, p);
     else if (p.nsplit <= 32) hipLaunchKernelGGL((decode_combine4_kernel<T, 8>), grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((decode_combine4_kernel<T, 16>), grid, dim3(256), 0, stream, p);
 }
@@ -822,8 +857,8 @@ static void launch_vec(const AttnParams &p, dim3 grid, hipStream_t stream, int g
 template <typename T>
 static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     constexpr bool F32 = sizeof(T) == 4;
-    const int gt = decode_gt(p.G, p.D, F32);
-    const int hb = (p.G + gt - 1) / gt;
+    const int gt = decode_gt(p.G * p.Sq, p.D, F32);  // columns: (query head, query row) pairs of a KV head
+    const int hb = (p.G * p.Sq + gt - 1) / gt;
     const long gy = (long)p.B * p.Hkv * hb;
     if (gy > 65535 || p.nsplit > 0x7fffffff) {
         set_error("decode: batch * kv_heads * head_blocks = %ld exceeds the grid limit 65535", gy);

@@ -153,6 +153,7 @@ def test_blocks_freed_after_capture_are_not_reused_while_the_graph_lives(device)
     buffers: a tensor freed after the capture must not be handed to a new tensor while the graph can still be
     replayed (the replay would write into the new owner's memory), and the device's workspace must neither be
     recycled nor grow inside a capture."""
+    device = device.with_new_stream()  # a stream, block cache and workspace of its own: no state from other tests
     B, H, Hkv, S, D = 2, 8, 2, 1500, 128
     q, k, v = _normal_qkv(77, B, H, Hkv, 1, S, D, 0.5)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))

@@ -1,0 +1,118 @@
+"""Multi-token decode steps (2..4 new query rows on a cache) on the split-KV decode kernels.
+
+The reference fuzzes exactly this shape (fusor-ml/core/src/composite/flash_attention.rs:807-921: q_seq_len 1..4,
+kv_seq_len = q_seq_len + 0..31, a [q_seq_len, kv_seq_len] mask tensor); kalosm-llama reaches it when a turn feeds a
+few tokens on top of a cached context, with MaskCache::get_mask(n, pos, window) as the mask
+(models/kalosm-llama/src/raw/mod.rs:618-620).  The rows ride as further columns beside the query heads that share a
+KV head, so the cache is still streamed once; every case asserts that the decode kernel is the one selected and
+compares with the CPU checker.
+"""
+import numpy as np
+import pytest
+
+import floneum_amd as fa
+import oracle
+from conftest import TOL_16, TOL_F32, assert_parity
+from test_attention_gpu import NEG_INF, _analytic_mask, _normal_qkv, _uniform, rounded
+
+pytestmark = pytest.mark.gpu
+
+
+def _tol(dtype):
+    return TOL_F32 if dtype == fa.F32 else (dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16)
+
+
+@pytest.mark.parametrize("dtype", [fa.F32, fa.F16])
+def test_reference_kv_cache_fuzz_ranges_select_the_decode_kernel(device, dtype):
+    """The reference's ranges, seeded: batch 1..2, heads 1..8, Sq 1..4, Skv = Sq + 0..31, head_dim 1..64, zero mask.
+    Head dims that are a multiple of 8 run on the decode kernel (the others have no 16-byte rows and take the general
+    kernel)."""
+    rng = np.random.default_rng(0xF111)
+    on_decode = 0
+    for it in range(60):
+        B, H, D = rng.integers(1, 3), rng.integers(1, 9), rng.integers(1, 65)
+        if it % 2:
+            D = 8 * rng.integers(1, 9)
+        Sq = rng.integers(1, 5)
+        Skv = Sq + rng.integers(0, 32)
+        q = _uniform(rng, (B, H, Sq, D))
+        k, v = _uniform(rng, (B, H, Skv, D)), _uniform(rng, (B, H, Skv, D))
+        mask = np.zeros((Sq, Skv), np.float32)
+        tq, tk, tv, tm = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v, mask))
+        sel = tq.selected_kernel(tk, tv, 0.1, mask=(tm, fa.MaskKind.QKMask))
+        if D % 8 == 0:
+            assert sel == fa.KERNEL_DECODE_SPLITKV, f"it{it} Sq{Sq} D{D}: kernel {sel}"
+            on_decode += 1
+        out = tq.flash_attention(tk, tv, 1 / np.sqrt(np.float32(D)), (tm, fa.MaskKind.QKMask)).to_numpy()
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), 1 / np.sqrt(np.float32(D)),
+                                     mask, "qk")
+        assert_parity(out, ref, _tol(dtype), f"it{it} B{B} H{H} Sq{Sq} Skv{Skv} D{D}")
+    assert on_decode >= 30
+
+
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
+@pytest.mark.parametrize("G,D,Sq,Skv", [(4, 128, 4, 3000), (4, 128, 2, 700), (1, 96, 3, 777), (8, 64, 4, 1500), (2, 128, 4, 64),
+                                        (3, 128, 3, 300), (16, 128, 2, 260), (4, 72, 4, 900), (2, 256, 2, 1500), (5, 32, 3, 5000),
+                                        (4, 128, 4, 4)])
+@pytest.mark.parametrize("case", ["causal", "window", "mask_tensor", "full"])
+def test_multi_token_step(device, dtype, G, D, Sq, Skv, case):
+    """New rows at the end of the cache: row r sits at position Skv - Sq + r and sees the keys up to its own
+    (causal among the new rows), optionally through a sliding window; the same mask as a tensor; and no mask."""
+    B, Hkv = 2, 2
+    q, k, v = _normal_qkv(41, B, Hkv * G, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    off = Skv - Sq
+    window = max(3, Skv // 3)
+    analytic, mask = {"causal": ((True, off, 0), _analytic_mask(Sq, Skv, True, off, 0)),
+                      "window": ((True, off, window), _analytic_mask(Sq, Skv, True, off, window)),
+                      "mask_tensor": (None, _analytic_mask(Sq, Skv, True, off, window)),
+                      "full": (None, None)}[case]
+    kw = {}
+    if analytic:
+        kw["analytic"] = analytic
+    elif mask is not None:
+        kw["mask"] = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    assert tq.selected_kernel(tk, tv, 0.1, **kw) == fa.KERNEL_DECODE_SPLITKV
+    m = kw.pop("mask", None)
+    out = tq.flash_attention(tk, tv, D ** -0.5, m, **kw).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                 None if mask is None else "qk")
+    assert_parity(out, ref, _tol(dtype), f"{case} G{G} D{D} Sq{Sq} Skv{Skv}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F16, fa.F32])
+def test_multi_token_step_ragged_batch_and_padding_mask(device, dtype):
+    """Per-sequence key counts and a BatchKeyMask on a multi-token step; the output written as [B, Sq, H, D]."""
+    B, H, Hkv, D, Sq, Smax = 4, 8, 2, 128, 3, 2500
+    lens = np.array([2500, 3, 1029, 640], np.int32)
+    q, k, v = _normal_qkv(43, B, H, Hkv, Sq, Smax, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    out_buf = fa.Tensor.empty(device, (B, Sq, H, D), dtype)
+    out = tq.flash_attention(tk, tv, D ** -0.5, kv_lens=fa.IntTensor(device, lens), out=out_buf.transpose(1, 2))
+    assert tq.selected_kernel(tk, tv, 0.1, kv_lens=fa.IntTensor(device, lens)) == fa.KERNEL_DECODE_SPLITKV
+    got = out_buf.to_numpy().transpose(0, 2, 1, 3)
+    bk = np.where(np.arange(Smax)[None, :] < lens[:, None], 0.0, NEG_INF).astype(np.float32)
+    got_m = tq.flash_attention(tk, tv, D ** -0.5, (fa.Tensor.from_numpy(device, bk, dtype), fa.MaskKind.BatchKeyMask)).to_numpy()
+    for b in range(B):
+        n = int(lens[b])
+        ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                     rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+        assert_parity(got[b:b + 1], ref, _tol(dtype), f"kv_lens b{b} len{n}")
+        assert_parity(got_m[b:b + 1], ref, _tol(dtype), f"batch-key mask b{b} len{n}")
+    del out
+
+
+def test_rows_fully_masked_by_their_own_limits_are_nan(device):
+    """A window so short and an offset so placed that some rows see no key: those rows are NaN (0/0) as in the
+    reference, the others are right."""
+    B, H, Hkv, D, Sq, Skv = 1, 4, 2, 64, 4, 40
+    q, k, v = _normal_qkv(44, B, H, Hkv, Sq, Skv, D)
+    mask = np.zeros((Sq, Skv), np.float32)
+    mask[1, :] = NEG_INF
+    mask[3, :] = NEG_INF
+    tq, tk, tv, tm = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v, mask))
+    assert tq.selected_kernel(tk, tv, 0.1, mask=(tm, fa.MaskKind.QKMask)) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    assert np.isnan(out[:, :, [1, 3]]).all()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5)
+    assert_parity(out[:, :, [0, 2]], ref[:, :, [0, 2]], TOL_F32, "visible rows")
