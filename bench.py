@@ -398,6 +398,49 @@ def calibration_copy(mib=256, reps=3):
         del cache
 
 
+def calibration_mfma(seconds=0.0):
+    """What the matrix cores deliver with nothing else in the way (fhip_calibration_mfma: a register-only loop of
+    the prefill kernel's matrix instruction, one wavefront per SIMD), with the clock the chip held meanwhile.  The
+    nominal 2.5 PFLOP/s is 256 CUs x 4 SIMDs x 1024 FLOP/clk at 2.4 GHz; under load the power limit sets the clock.
+    seconds > 0: keep the f16 / random-operand / 100 % case running back to back for that long (for sampling socket
+    power and clocks from outside) and report only that case."""
+    import floneum_amd as fa
+    dev = fa.Device.default()
+    L = fa.lib()
+    cus = dev.compute_units
+    nbytes = cus * (256 * 4 + 16)
+    scratch = fa.Buffer(dev, nbytes)
+    host = np.empty(nbytes, np.uint8)
+
+    def launch(dtype, rand, duty, rounds):
+        fa.check(L.fhip_calibration_mfma(dev.stream, dtype, rand, duty, rounds, ctypes.c_void_p(scratch.ptr), nbytes))
+
+    def one(dtype, rand, duty, rounds=60000, repeat=1):
+        launch(dtype, rand, duty, rounds)  # brings the clock to where this load holds it
+        dev.synchronize()
+        e0, e1 = Event(fa, dev), Event(fa, dev)
+        e0.record(dev)
+        for _ in range(repeat):
+            launch(dtype, rand, duty, rounds)
+        e1.record(dev)
+        e1.sync()
+        ms = e1.ms_since(e0)
+        fa.check(L.fhip_memcpy_d2h(dev.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(scratch.ptr), nbytes))
+        ticks = host[cus * 1024:].view(np.uint64).reshape(cus, 2).astype(np.float64)
+        ghz = ticks[:, 0] / ticks[:, 1] * 0.1
+        flops = 4.0 * cus * rounds * repeat * 32 * 32768
+        for e in (e0, e1):
+            L.fhip_event_destroy(e.h)
+        return dict(dtype={fa.F16: "f16", fa.BF16: "bf16"}[dtype], operands="random" if rand else "zero",
+                    duty_percent=duty, tflops=flops / (ms * 1e-3) / 1e12, ms=ms,
+                    sclk_ghz_median=float(np.median(ghz)), sclk_ghz_min=float(ghz.min()), sclk_ghz_max=float(ghz.max()))
+
+    if seconds > 0:
+        probe = one(fa.F16, 1, 100)
+        return [one(fa.F16, 1, 100, repeat=max(1, int(seconds * 1e3 / probe["ms"])))]
+    return [one(fa.F16, 1, 100), one(fa.F16, 1, 84), one(fa.F16, 1, 67), one(fa.F16, 0, 100), one(fa.BF16, 1, 100)]
+
+
 def record_traffic(name, fetch_csv, write_csv):
     """profiles/traffic.json entry of one configuration from the two counter CSVs (one counter per profiler run).
     The copy kernel of --calibration-copy moves 256 MiB each way; its counts give the bytes per count."""
@@ -457,6 +500,10 @@ def main():
                     help="also run a plain 256 MiB device copy (the KV-cache row copy kernel) three times, so a "
                          "rocprofv3 --pmc run of this command has a kernel of known traffic to scale FETCH_SIZE / "
                          "WRITE_SIZE with")
+    ap.add_argument("--calibration-mfma", nargs="?", type=float, const=0.0, default=None, metavar="SECONDS",
+                    help="no benchmark: run the register-only matrix-core loop (f16 random operands at 100 / 84 / 67 %% "
+                         "duty, zero operands, bf16) and print TFLOP/s and the shader clock held; with SECONDS, keep "
+                         "the f16 random 100 %% case running that long (to sample socket power from outside)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build runs on exactly one GPU (no sharding, no collectives); --gpus {a.gpus} is "
@@ -465,6 +512,9 @@ def main():
 
     if a.record_traffic:
         record_traffic(*a.record_traffic)
+        return
+    if a.calibration_mfma is not None:
+        print(json.dumps({"mfma_calibration": calibration_mfma(a.calibration_mfma), "nominal_peak_tflops": PEAK_MFMA_F16_TFLOPS}))
         return
 
     main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
@@ -489,6 +539,9 @@ def main():
                                                "frac_of_roofline", "spot_check_max_abs_err") if k in pre}
         if "cpu_baseline" in pre:
             line["prefill"]["cpu_baseline"] = pre["cpu_baseline"]
+        # beside the nominal peak the roofline is priced against: what a register-only loop of the same matrix
+        # instruction reaches on this chip under its power limit, and the clock it holds
+        line["prefill"]["mfma_calibration"] = calibration_mfma()
         # the remaining benchmark configurations, each a line of its own in miniature
         line["configs"] = {}
         for name, (steps, warmup) in (("C1", (200, 20)), ("C4", (100, 100)), ("C5", (20, 3))):

@@ -816,6 +816,25 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     return rc;
 }
 
+int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
+                          void *scratch, size_t scratch_bytes) {
+    if (!s || !scratch) {
+        set_error("calibration: NULL stream or scratch");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (duty_percent < 40 || duty_percent > 100 || rounds < 1) {
+        set_error("calibration: duty_percent %d must be in 40..100 and rounds %d positive", duty_percent, rounds);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const int cus = s->dev->prop.multiProcessorCount;
+    if (scratch_bytes < calibration_mfma_bytes(cus) || ((uintptr_t)scratch & 15) != 0) {
+        set_error("calibration: scratch of %zu bytes, 16-byte aligned, needed (got %zu)", calibration_mfma_bytes(cus), scratch_bytes);
+        return FHIP_ERR_WORKSPACE;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return launch_calibration_mfma(dtype, cus, duty_percent, rounds, random_operands ? 1 : 0, scratch, s->s);
+}
+
 // The same call on the library's own workspace (see `scratch` above): no hipMalloc / hipFree here or in anything
 // this calls, and none needed from the caller beyond the tensors.
 int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args) {

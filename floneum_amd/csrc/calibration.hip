@@ -1,0 +1,113 @@
+// Calibration kernels for the benchmark: what the matrix cores deliver with nothing else in the way.
+//
+// mfma_burn_kernel: one wavefront per SIMD of every compute unit runs rounds of 32 independent-accumulator
+// v_mfma_f32_32x32x16 instructions on operands held in registers (no LDS, no memory traffic, no vector work), the
+// instruction and the per-tile count of the prefill kernel's matrix phase.  Between rounds the wavefront may sleep so
+// that the matrix pipe is busy only a given share of the time.  Operands are pseudo-random f16/bf16 values in
+// (-2, 2), or all zero.  Every workgroup reports its shader-clock cycles and the 100 MHz wall-clock ticks it ran:
+// the ratio is the clock the chip held under that load.  The figure bounds from above what ANY f16 kernel can reach
+// on the same data; it has no counterpart in the reference.
+#include "common.h"
+#include "device_utils.h"
+
+namespace fhip {
+
+template <typename T>
+struct BurnMma;
+template <>
+struct BurnMma<half_t> {
+    typedef half8_t vec8;
+    static __device__ __forceinline__ float16_t mfma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ half_t from(float x) { return (half_t)x; }
+};
+template <>
+struct BurnMma<bf16_t> {
+    typedef bf16x8_t vec8;
+    static __device__ __forceinline__ float16_t mfma(vec8 a, vec8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ __bf16 from(float x) { return (__bf16)x; }
+};
+
+// SLEEP: s_sleep units (64 cycles each) after every round of 32 MFMAs (1024 matrix-pipe cycles)
+template <typename T, int SLEEP>
+__global__ __launch_bounds__(256) void mfma_burn_kernel(float *sink, uint64_t *ticks, int rounds, int random_operands) {
+    typedef typename BurnMma<T>::vec8 vec8;
+    const uint64_t c0 = clock64(), w0 = wall_clock64();
+    vec8 av[8], bv[4];
+    uint32_t s = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            s = s * 1664525u + 1013904223u;
+            const float x = ((s >> 8) & 0xffff) / 65536.0f - 0.5f;
+            s = s * 1664525u + 1013904223u;
+            const float y = ((s >> 8) & 0xffff) / 65536.0f - 0.5f;
+            av[j][i] = BurnMma<T>::from(random_operands ? x * 4.0f : 0.0f);
+            bv[j & 3][i] = BurnMma<T>::from(random_operands ? y * 4.0f : 0.0f);
+        }
+    float16_t acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = 0.0f;
+    for (int it = 0; it < rounds; it++) {
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] = BurnMma<T>::mfma(av[u], bv[c], acc[c]);
+        if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+    }
+    float res = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) res += acc[c][r];
+    const uint64_t c1 = clock64(), w1 = wall_clock64();
+    sink[blockIdx.x * 256 + threadIdx.x] = res;
+    if (threadIdx.x == 0) {
+        ticks[2 * blockIdx.x] = c1 - c0;
+        ticks[2 * blockIdx.x + 1] = w1 - w0;
+    }
+}
+
+// s_sleep units per round that leave the matrix pipe busy about `duty` percent of the time
+static int sleep_units(int duty) {
+    if (duty >= 100) return 0;
+    const int idle_cycles = 1024 * (100 - duty) / duty;
+    int units = (idle_cycles + 32) / 64;
+    return units < 1 ? 1 : units > 15 ? 15 : units;
+}
+
+template <typename T>
+static int launch_burn_t(int units, dim3 grid, hipStream_t stream, float *sink, uint64_t *ticks, int rounds, int random_operands) {
+#define FHIP_BURN(U) \
+    case U: hipLaunchKernelGGL((mfma_burn_kernel<T, U>), grid, dim3(256), 0, stream, sink, ticks, rounds, random_operands); break
+    switch (units) {
+        FHIP_BURN(0); FHIP_BURN(1); FHIP_BURN(2); FHIP_BURN(3); FHIP_BURN(4); FHIP_BURN(5); FHIP_BURN(6); FHIP_BURN(7);
+        FHIP_BURN(8); FHIP_BURN(9); FHIP_BURN(10); FHIP_BURN(11); FHIP_BURN(12); FHIP_BURN(13); FHIP_BURN(14); FHIP_BURN(15);
+        default: set_error("calibration: bad sleep count %d", units); return FHIP_ERR_INVALID_ARG;
+    }
+#undef FHIP_BURN
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+size_t calibration_mfma_bytes(int compute_units) { return (size_t)compute_units * (256 * sizeof(float) + 2 * sizeof(uint64_t)); }
+
+int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,
+                            hipStream_t stream) {
+    float *sink = (float *)scratch;
+    uint64_t *ticks = (uint64_t *)((char *)scratch + (size_t)compute_units * 256 * sizeof(float));
+    const int units = sleep_units(duty_percent);
+    const dim3 grid((unsigned)compute_units);
+    if (dtype == FHIP_F16) return launch_burn_t<half_t>(units, grid, stream, sink, ticks, rounds, random_operands);
+    if (dtype == FHIP_BF16) return launch_burn_t<bf16_t>(units, grid, stream, sink, ticks, rounds, random_operands);
+    set_error("calibration: the matrix-core loop takes f16 or bf16");
+    return FHIP_ERR_UNSUPPORTED;
+}
+
+}  // namespace fhip

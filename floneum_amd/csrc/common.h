@@ -111,6 +111,11 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
                  int *nsplit);
 size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 
+// calibration (calibration.hip): the register-only matrix-core loop and the scratch it reports into
+size_t calibration_mfma_bytes(int compute_units);
+int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,
+                            hipStream_t stream);
+
 // KV cache copies
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream);

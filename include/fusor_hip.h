@@ -241,6 +241,18 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
 #define FHIP_NOALLOC_WORKSPACE_BYTES (32u << 20)
 int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
 
+/* Calibration for benchmarks (no counterpart in the reference): what the matrix cores deliver with nothing else
+ * in the way.  One wavefront per SIMD of every compute unit runs `rounds` rounds of 32 v_mfma_f32_32x32x16
+ * instructions (the instruction and per-tile count of the prefill kernel's matrix phase) on operands held in
+ * registers: no LDS, no memory traffic, no vector work.  `random_operands` != 0: pseudo-random values in (-2, 2);
+ * 0: all zero (no data toggling).  `duty_percent` (40..100): the share of the time the matrix pipe is kept busy
+ * (the wavefront sleeps in between).  FLOPs per launch = 4 * compute_units * rounds * 32 * 32768.  `scratch`
+ * (device, 16-byte aligned, compute_units * 1040 bytes) receives compute_units * 256 floats nobody needs and then,
+ * per compute unit, two uint64: the shader-clock cycles and the 100 MHz wall-clock ticks its workgroup ran (their
+ * ratio * 0.1 = the clock in GHz the chip held under this load).  Asynchronous on `s`. */
+int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
+                          void *scratch, size_t scratch_bytes);
+
 /* ---- masks: host builders, bit-exact with the reference ---------------------------------------
  * `out` is host memory of the given dtype (f32: 0x00000000 / 0xFF800000; f16: 0x0000 / 0xFC00;
  * bf16: 0x0000 / 0xFF80), row-major contiguous. */

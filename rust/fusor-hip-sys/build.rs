@@ -19,6 +19,7 @@ const SOURCES: &[&str] = &[
     "kv_cache.hip",
     "mask_intervals.hip",
     "rope.hip",
+    "calibration.hip",
 ];
 
 // the flags floneum_amd/build.py uses; packed-f32 VALU forms are kept out of the generated code on purpose

@@ -202,6 +202,17 @@ unsafe extern "C" {
     pub fn fhip_flash_attention(s: *mut fhip_stream, args: *const fhip_attn_args) -> c_int;
     pub fn fhip_flash_attention_noalloc(s: *mut fhip_stream, args: *const fhip_attn_args) -> c_int;
 
+    // calibration for benchmarks: the register-only matrix-core loop
+    pub fn fhip_calibration_mfma(
+        s: *mut fhip_stream,
+        dtype: fhip_dtype,
+        random_operands: i32,
+        duty_percent: i32,
+        rounds: i32,
+        scratch: *mut c_void,
+        scratch_bytes: usize,
+    ) -> c_int;
+
     // masks
     pub fn fhip_mask_causal(dtype: fhip_dtype, seq_len: u32, out: *mut c_void) -> c_int;
     pub fn fhip_mask_sliding_window(dtype: fhip_dtype, seq_len: u32, window: u64, out: *mut c_void) -> c_int;
