@@ -441,6 +441,34 @@ def calibration_mfma(seconds=0.0):
     return [one(fa.F16, 1, 100), one(fa.F16, 1, 84), one(fa.F16, 1, 67), one(fa.F16, 0, 100), one(fa.BF16, 1, 100)]
 
 
+def calibration_read(mib=256, slices=5, launches=60):
+    """What a kernel that only reads reaches (fhip_calibration_read: 16-byte non-temporal loads, eight in flight per
+    lane, no arithmetic, no output): `mib` MiB per launch, the launches rotating over `slices` distinct slices so that
+    the 256 MB Infinity Cache cannot serve them, back to back.  The size is C2's KV bytes per call."""
+    import floneum_amd as fa
+    dev = fa.Device.default()
+    L = fa.lib()
+    nbytes = mib << 20
+    buf = fa.Buffer(dev, nbytes * slices)
+    sink = fa.Buffer(dev, dev.compute_units * 32)
+    fa.check(L.fhip_memset(dev.stream, ctypes.c_void_p(buf.ptr), 0x3c, nbytes * slices))
+
+    def launch(i):
+        fa.check(L.fhip_calibration_read(dev.stream, ctypes.c_void_p(buf.ptr + (i % slices) * nbytes), nbytes,
+                                         ctypes.c_void_p(sink.ptr), dev.compute_units * 32))
+
+    for i in range(10):
+        launch(i)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for i in range(launches):
+        launch(i)
+    dev.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / launches
+    return dict(mib_per_launch=mib, slices_rotated=slices, launches=launches, us_per_launch=us,
+                gbps=nbytes / us / 1e3, frac_of_peak=nbytes / us / 1e3 / PEAK_HBM_GBS)
+
+
 def record_traffic(name, fetch_csv, write_csv):
     """profiles/traffic.json entry of one configuration from the two counter CSVs (one counter per profiler run).
     The copy kernel of --calibration-copy moves 256 MiB each way; its counts give the bytes per count."""
@@ -500,6 +528,8 @@ def main():
                     help="also run a plain 256 MiB device copy (the KV-cache row copy kernel) three times, so a "
                          "rocprofv3 --pmc run of this command has a kernel of known traffic to scale FETCH_SIZE / "
                          "WRITE_SIZE with")
+    ap.add_argument("--calibration-read", action="store_true",
+                    help="no benchmark: run the read-only streaming kernel over 256 MiB slices and print GB/s")
     ap.add_argument("--calibration-mfma", nargs="?", type=float, const=0.0, default=None, metavar="SECONDS",
                     help="no benchmark: run the register-only matrix-core loop (f16 random operands at 100 / 84 / 67 %% "
                          "duty, zero operands, bf16) and print TFLOP/s and the shader clock held; with SECONDS, keep "
@@ -512,6 +542,9 @@ def main():
 
     if a.record_traffic:
         record_traffic(*a.record_traffic)
+        return
+    if a.calibration_read:
+        print(json.dumps({"read_calibration": calibration_read(), "nominal_peak_gbps": PEAK_HBM_GBS}))
         return
     if a.calibration_mfma is not None:
         print(json.dumps({"mfma_calibration": calibration_mfma(a.calibration_mfma), "nominal_peak_tflops": PEAK_MFMA_F16_TFLOPS}))
@@ -531,6 +564,9 @@ def main():
     if "imbalance" in main_res:
         line["imbalance"] = main_res["imbalance"]
     if not a.no_extra and a.config == "C2":
+        # beside the nominal 8 TB/s the roofline is priced against: what a kernel that only reads the same number of
+        # bytes per launch reaches on this chip
+        line["roofline"]["read_calibration"] = calibration_read()
         # the other half of the metric: C3 prefill on the matrix cores
         # the shader clock needs some tens of milliseconds of matrix load to settle: warm the prefill
         # leg up for longer than the (much shorter) decode steps need

@@ -835,6 +835,20 @@ int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_opera
     return launch_calibration_mfma(dtype, cus, duty_percent, rounds, random_operands ? 1 : 0, scratch, s->s);
 }
 
+int fhip_calibration_read(fhip_stream *s, const void *src, size_t bytes, void *scratch, size_t scratch_bytes) {
+    if (!s || !src || !scratch) {
+        set_error("calibration: NULL stream, source or scratch");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const int cus = s->dev->prop.multiProcessorCount;
+    if (((uintptr_t)src & 15) != 0 || scratch_bytes < (size_t)cus * 8 * sizeof(uint32_t)) {
+        set_error("calibration: the source must be 16-byte aligned and the scratch hold %zu bytes", (size_t)cus * 8 * sizeof(uint32_t));
+        return FHIP_ERR_WORKSPACE;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return launch_calibration_read(src, bytes, cus, scratch, s->s);
+}
+
 // The same call on the library's own workspace (see `scratch` above): no hipMalloc / hipFree here or in anything
 // this calls, and none needed from the caller beyond the tensors.
 int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args) {

@@ -96,6 +96,36 @@ static int launch_burn_t(int units, dim3 grid, hipStream_t stream, float *sink, 
     return FHIP_OK;
 }
 
+// read_burn_kernel: nothing but the loads of a streaming kernel.  Every workgroup reads its contiguous share of the
+// buffer with 16-byte non-temporal loads, eight in flight per lane (a wavefront load instruction covers 1 KB, as in the
+// decode kernels), folds what it read into one word and writes that word only if it has a value no fold produces.
+__global__ __launch_bounds__(256) void read_burn_kernel(const uint4_t *src, size_t n16, uint32_t *sink) {
+    const size_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t lo = (size_t)blockIdx.x * per_wg, hi = lo + per_wg < n16 ? lo + per_wg : n16;
+    uint32_t acc = 0;
+    constexpr int U = 8;
+    for (size_t base = lo + threadIdx.x; base < hi; base += (size_t)U * 256) {
+        uint4_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256;
+            v[u] = __builtin_nontemporal_load(src + (i < hi ? i : hi - 1));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) acc ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+    }
+    if (acc == 0x9e3779b9u && lo == hi) sink[blockIdx.x] = acc;  // never true (lo < hi whenever something was read)
+}
+
+int launch_calibration_read(const void *src, size_t bytes, int compute_units, void *sink, hipStream_t stream) {
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return FHIP_OK;
+    const unsigned wgs = (unsigned)compute_units * 8;  // two rounds of four resident workgroups per CU
+    hipLaunchKernelGGL(read_burn_kernel, dim3(wgs), dim3(256), 0, stream, (const uint4_t *)src, n16, (uint32_t *)sink);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
 size_t calibration_mfma_bytes(int compute_units) { return (size_t)compute_units * (256 * sizeof(float) + 2 * sizeof(uint64_t)); }
 
 int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,

@@ -116,6 +116,8 @@ size_t calibration_mfma_bytes(int compute_units);
 int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,
                             hipStream_t stream);
 
+int launch_calibration_read(const void *src, size_t bytes, int compute_units, void *sink, hipStream_t stream);
+
 // KV cache copies
 int launch_copy_rows(const void *src, const int64_t sstride[4], void *dst, const int64_t dstride[4],
                      const uint32_t shape[4], int elem_bytes, hipStream_t stream);

@@ -253,6 +253,12 @@ int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
 int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
                           void *scratch, size_t scratch_bytes);
 
+/* Calibration for benchmarks (no counterpart in the reference): a kernel that does nothing but read `bytes` of
+ * device memory at `src` (16-byte aligned) once, with 16-byte non-temporal loads, eight in flight per lane: the
+ * rate a streaming kernel of this shape can reach at most.  `scratch`: device memory of at least
+ * compute_units * 32 bytes (nothing of interest is written there).  Asynchronous on `s`. */
+int fhip_calibration_read(fhip_stream *s, const void *src, size_t bytes, void *scratch, size_t scratch_bytes);
+
 /* ---- masks: host builders, bit-exact with the reference ---------------------------------------
  * `out` is host memory of the given dtype (f32: 0x00000000 / 0xFF800000; f16: 0x0000 / 0xFC00;
  * bf16: 0x0000 / 0xFF80), row-major contiguous. */

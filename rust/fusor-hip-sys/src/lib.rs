@@ -213,6 +213,14 @@ unsafe extern "C" {
         scratch_bytes: usize,
     ) -> c_int;
 
+    pub fn fhip_calibration_read(
+        s: *mut fhip_stream,
+        src: *const c_void,
+        bytes: usize,
+        scratch: *mut c_void,
+        scratch_bytes: usize,
+    ) -> c_int;
+
     // masks
     pub fn fhip_mask_causal(dtype: fhip_dtype, seq_len: u32, out: *mut c_void) -> c_int;
     pub fn fhip_mask_sliding_window(dtype: fhip_dtype, seq_len: u32, window: u64, out: *mut c_void) -> c_int;

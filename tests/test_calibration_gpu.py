@@ -39,3 +39,18 @@ def test_mfma_calibration_rejects_bad_arguments(device):
     assert L.fhip_calibration_mfma(device.stream, fa.F16, 1, 100, 0, p, nbytes) == fa.ERR_INVALID_ARG
     assert L.fhip_calibration_mfma(device.stream, fa.F16, 1, 100, 10, p, nbytes - 16) == fa.ERR_WORKSPACE
     assert L.fhip_calibration_mfma(device.stream, fa.F16, 1, 100, 10, None, nbytes) == fa.ERR_INVALID_ARG
+
+
+def test_read_calibration_runs_and_rejects_bad_arguments(device):
+    L = fa.lib()
+    n = 8 << 20
+    buf, sink = fa.Buffer(device, n), fa.Buffer(device, device.compute_units * 32)
+    fa.check(L.fhip_memset(device.stream, ctypes.c_void_p(buf.ptr), 1, n))
+    for nbytes in (n, n - 4096 + 16, 16, 0):
+        fa.check(L.fhip_calibration_read(device.stream, ctypes.c_void_p(buf.ptr), nbytes, ctypes.c_void_p(sink.ptr),
+                                         device.compute_units * 32))
+    device.synchronize()
+    assert L.fhip_calibration_read(device.stream, ctypes.c_void_p(buf.ptr + 8), n - 16, ctypes.c_void_p(sink.ptr),
+                                   device.compute_units * 32) == fa.ERR_WORKSPACE
+    assert L.fhip_calibration_read(device.stream, ctypes.c_void_p(buf.ptr), n, ctypes.c_void_p(sink.ptr), 16) == fa.ERR_WORKSPACE
+    assert L.fhip_calibration_read(device.stream, None, n, ctypes.c_void_p(sink.ptr), 1 << 20) == fa.ERR_INVALID_ARG
