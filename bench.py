@@ -88,6 +88,10 @@ def configs():
         "S1": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
         "S2": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
         "S3": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=32768, D=128, dtype="f16", std=0.5, causal=False),
+        # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the vector variant of
+        # the decode kernel; and a 16-bit cache with Gemma-3's key length 256, which the vector variant serves too
+        "F2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
+        "W2": dict(kind="decode", B=16, H=16, Hkv=4, Sq=1, Skv=4096, D=256, dtype="f16", std=0.5, causal=False),
         # a multi-token decode step: C2's batch with four new rows per sequence at the end of the cache, causal among
         # themselves (a draft being verified); the rows ride beside the heads of a GQA group, the cache is read once
         "M1": dict(kind="decode", B=16, H=32, Hkv=8, Sq=4, Skv=4096, D=128, dtype="f16", std=0.5, causal=True),

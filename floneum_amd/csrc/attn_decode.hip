@@ -31,9 +31,11 @@ constexpr int DEC_WAVES = 4;
 constexpr int DEC_UNROLL = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 
-// the matrix-core variant takes 16-bit tensors; f32 tensors run on the vector variant
+// the matrix-core variants: 16-bit tensors on the 16-bit instruction, f32 tensors on the f32 one; other head dims
+// run on the vector variant
 static bool decode_use_mfma(int D, bool f32) {
-    return !f32 && (D == 32 || D == 64 || D == 96 || D == 128);
+    (void)f32;
+    return D == 32 || D == 64 || D == 96 || D == 128;
 }
 
 // query heads handled by one workgroup
@@ -60,7 +62,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // variant is quicker unsplit than with a second launch to merge two splits (measured 6.6 vs 8.6 us).
     // (the vector variant's step is 16 rows of 64 / LPK keys: 64 keys at head_dim 128 in f32, where one step
     // per workgroup is one memory round trip less than two)
-    int step_keys = 128;
+    int step_keys = f32 ? 64 : 128;  // matrix-core variants: four wavefronts of 16 (f32) or 32 keys
     if (!decode_use_mfma(D, f32)) {
         const int lpk = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
         step_keys = 16 * (64 / lpk);
@@ -688,6 +690,245 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
     }
 }
 
+// ---- pass 1, matrix-core variant for f32 tensors -------------------------------------------------------
+// The cache type kalosm-llama keeps (models/kalosm-llama/src/raw/attention_layer.rs:400-403).  Same structure as
+// decode_mfma_kernel on v_mfma_f32_16x16x4_f32 (full f32 products): a wavefront step is 16 consecutive keys, parked
+// in a wavefront-private LDS tile.
+//   S^T[key][col] = K . Q^T : lane (j, q4) reads K[key j][16 c + 4 q4 .. +4] with one 128-bit LDS read per chunk c and
+//     feeds its four values to four matrix steps (contraction slot (c, i, q4) = dim 16 c + 4 q4 + i on both operands);
+//     the lane ends up with the scores of keys 4 q4 + r (r = 0..3) for column j.
+//   O^T[dim][col] += V^T . P^T : contraction slot (ks, q4) is key 4 q4 + ks, so the B operand of step ks is the lane's
+//     own probability r = ks (nothing changes lanes).  Lane (i, q4) reads VW consecutive dims of V[key 4 q4 + ks] with
+//     one LDS read and feeds VW matrix steps: row i of output block (hb, e) is dim 16 VW hb + VW i + e.  The lane
+//     therefore holds, for its column, the 4 VW consecutive dims starting at 16 VW hb + 4 VW q4 of every block hb.
+// The vector variant spends most of its instructions on a softmax that every lane of a key's group repeats; here
+// the softmax of a column is computed once, by the four lanes that hold its 16 scores.
+constexpr int DF_KEYS = 16;  // keys per wavefront step
+
+template <int D>
+__global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_f32_kernel(AttnParams p) {
+    constexpr int KP = D * 4 + 16;             // tile row pitch (bytes): rows 4 banks apart
+    constexpr int K_BYTES = DF_KEYS * KP;
+    constexpr int WAVE_BYTES = 2 * K_BYTES;    // K tile, V tile
+    constexpr int CPR = D / 4;                 // 16-byte chunks per row
+    constexpr int NLD = DF_KEYS * CPR / 64;    // 16-byte loads per lane per tile
+    static_assert(DF_KEYS * CPR % 64 == 0, "a tile is a whole number of wavefront loads");
+    constexpr int KC = D / 16;                 // 16-dim chunks of the contraction of K . Q^T
+    constexpr int VW = (D % 64 == 0) ? 4 : 2;  // dims per V read
+    constexpr int NBLK = D / (16 * VW);        // output blocks of 16 VW dims
+    constexpr int MERGE_BYTES = DEC_WAVES * DM_HEADS * (D + 2) * 4;
+    constexpr int LDS_BYTES = DEC_WAVES * WAVE_BYTES > MERGE_BYTES ? DEC_WAVES * WAVE_BYTES : MERGE_BYTES;
+    __shared__ __attribute__((aligned(16))) char smem[LDS_BYTES];
+
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 15;  // column of this lane
+    const int q4 = lane >> 4; // key group
+    auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
+
+    const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
+    const int rows = p.Sq;  // columns are (query head, query row) pairs, see decode_mfma_kernel
+    const int NC = p.G * rows;
+    const int HB = (NC + DM_HEADS - 1) / DM_HEADS;
+    const int hb = blockIdx.y % HB;
+    const int bg = blockIdx.y / HB;
+    const int g = bg % p.Hkv;
+    const int b = bg / p.Hkv;
+    const int c0 = hb * DM_HEADS;
+    const int nh = min(DM_HEADS, NC - c0);
+    const int cj = c0 + min(j, nh - 1);
+    const int hj = g * p.G + cj / rows, rj = cj % rows;
+
+    int kv_hi = p.Skv;
+    if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
+    if (p.kv_lens && split * p.chunk >= kv_hi && split > 0) return;  // the combine pass skips it too
+    int lo = split * p.chunk;
+    int hi = min(lo + p.chunk, kv_hi);
+    int lo_j = lo, hi_j = hi;
+    if (p.analytic) {
+        if (p.causal) {
+            hi_j = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj);
+            hi = (int)min((int64_t)hi, p.q_pos_offset + rows);
+        }
+        if (p.window > 0) {
+            lo_j = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj);
+            lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
+        }
+    }
+
+    const float *kbase = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
+    const float *vbase = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
+    const float *mrow = nullptr;
+    if (p.mask_kind == FHIP_MASK_QK) mrow = (const float *)p.mask + rj * p.ms0;
+    if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const float *)p.mask + b * p.ms0;
+    const float scale2 = p.scale * LOG2E;
+
+    float4_t o[NBLK][VW];
+#pragma unroll
+    for (int nb = 0; nb < NBLK; nb++)
+#pragma unroll
+        for (int e = 0; e < VW; e++) o[nb][e] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.0f;
+
+    // one wavefront step = 16 consecutive keys; the four wavefronts interleave their steps.  Every lane always loads
+    // (rows outside [lo, hi) are replaced by the nearest one inside; their scores are masked below).
+    const int lo_al = lo - (lo % DF_KEYS);
+    const int step = DEC_WAVES * DF_KEYS;
+    float4_t kst[NLD], vst[NLD];
+    auto load_tile = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = lane + 64 * u;
+            const int row = cid / CPR, col = cid % CPR;
+            const int key = min(max(base + row, lo), hi - 1);
+            kst[u] = __builtin_nontemporal_load((const float4_t *)(kbase + (int64_t)key * p.ks[2] + col * 4));
+            vst[u] = __builtin_nontemporal_load((const float4_t *)(vbase + (int64_t)key * p.vs[2] + col * 4));
+        }
+    };
+    auto store_tile = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = lane + 64 * u;
+            const int row = cid / CPR, col = cid % CPR;
+            *DLDS_PTR(float4_t, row * KP + col * 16) = kst[u];
+            *DLDS_PTR(float4_t, K_BYTES + row * KP + col * 16) = vst[u];
+        }
+    };
+
+    int base = lo_al + wave * DF_KEYS;
+    if (base < hi) load_tile(base);  // issued first so the Q fetch below overlaps it
+
+    // Q^T operand: column j, dims 16 c + 4 q4 .. +4 (zero for the padding columns)
+    float4_t qreg[KC];
+    {
+        const float *qp = (const float *)p.q + b * p.qs[0] + (int64_t)hj * p.qs[1] + (int64_t)rj * p.qs[2];
+        const bool qvec = p.qs[3] == 1 && (((uintptr_t)qp) & 15) == 0;
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (j < nh) {
+                if (qvec) {
+                    v = *(const float4_t *)(qp + 16 * c + 4 * q4);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = qp[(int64_t)(16 * c + 4 * q4 + e) * p.qs[3]];
+                }
+            }
+            qreg[c] = v;
+        }
+    }
+
+    for (; base < hi; base += step) {
+        wave_lds_sync();  // the previous step's LDS reads precede these writes
+        store_tile();
+        wave_lds_sync();
+        load_tile(base + step);  // in flight during the math below (beyond the end: a row read again)
+
+        // ---- S^T[key][col] = K . Q^T ---------------------------------------------------------------------
+        float4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+            const float4_t a = *DLDS_PTR(float4_t, j * KP + (16 * c + 4 * q4) * 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], qreg[c][i], s, 0, 0, 0);
+        }
+        // element r is key base + 4 q4 + r for column j
+        float sv[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int key = base + 4 * q4 + r;
+            const bool visible = key >= lo_j && key < hi_j;
+            float x = s[r] * scale2;
+            if (mrow && visible) x += mrow[(int64_t)key * p.ms1] * LOG2E;
+            sv[r] = visible ? x : -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+        mx = quad_rows_max(mx);
+        const float m_new = fmaxf(m, mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
+        m = m_new;
+        float pe[4], psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            pe[r] = __builtin_amdgcn_exp2f(sv[r] - m_safe);
+            psum += pe[r];
+        }
+        l = l * corr + psum;
+#pragma unroll
+        for (int nb = 0; nb < NBLK; nb++)
+#pragma unroll
+            for (int e = 0; e < VW; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[nb][e][r] *= corr;
+
+        // ---- O^T[dim][col] += V^T . P^T : step ks contracts the keys 4 q4 + ks ----------------------------
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+            for (int nb = 0; nb < NBLK; nb++) {
+                const int voff = K_BYTES + (4 * q4 + ks) * KP + (16 * VW * nb + VW * j) * 4;
+                if constexpr (VW == 4) {
+                    const float4_t a = *DLDS_PTR(float4_t, voff);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[ks], o[nb][e], 0, 0, 0);
+                } else {
+                    typedef float float2v_t __attribute__((ext_vector_type(2)));
+                    const float2v_t a = *DLDS_PTR(float2v_t, voff);
+#pragma unroll
+                    for (int e = 0; e < 2; e++) o[nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[ks], o[nb][e], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- merge: key groups -> wavefront -> workgroup ------------------------------------------------
+    l = quad_rows_sum(l);
+    __syncthreads();  // every wavefront is done with its K/V tile; the LDS is reused for the merge
+    float *macc = (float *)smem;  // [wave][column][D + 2]
+    if (j < nh) {
+        float *dst = macc + ((wave * DM_HEADS + j) * (D + 2));
+        // element (nb, e, r) of this lane is dim 16 VW nb + VW (4 q4 + r) + e
+#pragma unroll
+        for (int nb = 0; nb < NBLK; nb++)
+#pragma unroll
+            for (int e = 0; e < VW; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) dst[16 * VW * nb + VW * (4 * q4 + r) + e] = o[nb][e][r];
+        if (q4 == 0) {
+            dst[D] = m;
+            dst[D + 1] = l;
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nh * D; idx += 64 * DEC_WAVES) {
+        const int hh = idx / D, d = idx % D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
+        const float Ms = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) {
+            const float *src = macc + (w * DM_HEADS + hh) * (D + 2);
+            const float wgt = __builtin_amdgcn_exp2f(src[D] - Ms);
+            L += wgt * src[D + 1];
+            A += wgt * src[d];
+        }
+        const int h = g * p.G + (c0 + hh) / rows, qr = (c0 + hh) % rows;
+        if (p.nsplit == 1) {
+            ((float *)p.out)[b * p.os[0] + h * p.os[1] + qr * p.os[2] + d * p.os[3]] = A / L;  // no visible key: 0/0 = NaN
+        } else {
+            float *ws = (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
+            ws[d] = A;
+            if (d == 0) {
+                ws[D] = M;
+                ws[D + 1] = L;
+            }
+        }
+    }
+}
+
 // ---- pass 2 -------------------------------------------------------------------------------------
 // One 64-lane wavefront per (batch, head); up to U partials are fetched in one round of loads (a round costs
 // one memory latency, so calls with many splits take the wide form).
@@ -865,6 +1106,23 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     dim3 grid((unsigned)p.nsplit, (unsigned)gy), block(64 * DEC_WAVES);
+    if constexpr (F32) {
+        if (decode_use_mfma(p.D, true)) {
+            switch (p.D) {
+                case 32: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<32>), grid, block, stream, p, p); break;
+                case 64: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<64>), grid, block, stream, p, p); break;
+                case 96: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<96>), grid, block, stream, p, p); break;
+                default: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128>), grid, block, stream, p, p); break;
+            }
+            FHIP_HIP_CHECK(hipGetLastError());
+            FHIP_MARK_MAIN_DONE(p, stream);
+            if (p.nsplit > 1) {
+                launch_combine<T>(p, stream);
+                FHIP_HIP_CHECK(hipGetLastError());
+            }
+            return FHIP_OK;
+        }
+    }
     if constexpr (!F32) {
         if (decode_use_mfma(p.D, false)) {
             switch (p.D) {
