@@ -690,11 +690,11 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
         if (part) *bytes = f32_partials_offset(args) + part;
     }
     if (id == FHIP_KERNEL_DECODE_SPLITKV) {
-        int chunk, nsplit;
+        int chunk, nsplit, waves;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
         const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2], rows = (int)args->q.shape[2];
         decode_plan(B, Hkv, H / Hkv * rows, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr,
-                    args->dtype == FHIP_F32, &chunk, &nsplit);
+                    args->dtype == FHIP_F32, &chunk, &nsplit, &waves);
         *bytes = decode_workspace_bytes(B, H * rows, Hkv, D, nsplit);
     }
     return FHIP_OK;
@@ -794,7 +794,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
             decode_plan(p.B, p.Hkv, p.G * p.Sq, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr,
-                        args->dtype == FHIP_F32, &p.chunk, &p.nsplit);
+                        args->dtype == FHIP_F32, &p.chunk, &p.nsplit, &p.dec_waves);
             const size_t need = decode_workspace_bytes(p.B, p.H * p.Sq, p.Hkv, p.D, p.nsplit);
             if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
                 set_error("decode needs a workspace of %zu bytes, got %zu", need,

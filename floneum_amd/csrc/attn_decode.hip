@@ -45,10 +45,18 @@ static int decode_gt(int G, int D, bool f32) {
 }
 
 void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, bool f32, int *chunk,
-                 int *nsplit) {
+                 int *nsplit, int *waves) {
     const int gt = decode_gt(G, D, f32);
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
+    *waves = DEC_WAVES;
+    if (decode_use_mfma(D, f32) && !f32 && units >= compute_units && Skv > 2048) {
+        // the 8-wavefront form of the 16-bit matrix-core variant: whole units for every CU, chunks of 2048 keys
+        *waves = 8;
+        *chunk = 2048;
+        *nsplit = (Skv + 2047) / 2048;
+        return;
+    }
     // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more; f32 rows carry
     // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at
     // batch 1 with 32768 keys)
@@ -436,8 +444,12 @@ constexpr int DM_DEPTH = 1;  // tiles in flight per wavefront beside the one in 
                              // is not latency-bound with eight wavefronts per CU)
 constexpr int DM_HEADS = 16; // query heads per workgroup (MFMA N dimension)
 
-template <typename T, int D>
-__global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnParams p) {
+// WAVES = 4: two workgroups per CU.  WAVES = 8: one workgroup per CU with chunks of up to 2048 keys, for calls with at
+// least one (batch, kv head) unit per CU: a workgroup's first tile takes several microseconds to arrive while the
+// memory system is loaded, so with work enough to keep every CU busy anyway, fewer and longer workgroups stream
+// better (32 ragged sequences of up to 32768 keys: 6.45 -> 6.83 TB/s).
+template <typename T, int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void decode_mfma_kernel(AttnParams p) {
     typedef typename DecMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;          // K tile row pitch (bytes): rows 4 banks apart
     constexpr int VP = D * 2 + 32;          // V tile row pitch (bytes): rows 8 banks apart
@@ -448,8 +460,8 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
     constexpr int NLD = DM_KEYS * CPR / 64; // 16-byte loads per lane per tile
     constexpr int KB = D / 32;              // contraction blocks of QK^T
     constexpr int NB = D / 16;              // 16-dim blocks of the output
-    constexpr int MERGE_BYTES = DEC_WAVES * DM_HEADS * (D + 2) * 4;
-    constexpr int LDS_BYTES = DEC_WAVES * WAVE_BYTES > MERGE_BYTES ? DEC_WAVES * WAVE_BYTES : MERGE_BYTES;
+    constexpr int MERGE_BYTES = WAVES * DM_HEADS * (D + 2) * 4;
+    constexpr int LDS_BYTES = WAVES * WAVE_BYTES > MERGE_BYTES ? WAVES * WAVE_BYTES : MERGE_BYTES;
     __shared__ __attribute__((aligned(16))) char smem[LDS_BYTES];
 
     const int wave = threadIdx.x >> 6;
@@ -505,7 +517,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
 
     // one wavefront step = 32 consecutive keys; the four wavefronts interleave their steps
     const int lo_al = lo - (lo % DM_KEYS);
-    const int step = DEC_WAVES * DM_KEYS;
+    const int step = WAVES * DM_KEYS;
     // Staging registers of the tiles in flight: DEPTH tiles per wavefront.
     // Every lane always loads: a row outside [lo, hi) is replaced by the nearest one inside (its score is set to
     // -inf below, so what it holds never counts).  Without branches around the loads the compiler can count them,
@@ -659,15 +671,15 @@ __global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_kernel(AttnPara
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < nh * D; idx += 64 * DEC_WAVES) {
+    for (int idx = threadIdx.x; idx < nh * D; idx += 64 * WAVES) {
         const int hh = idx / D, d = idx % D;
         float M = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
+        for (int w = 0; w < WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
         const float Ms = (M == -INFINITY) ? 0.0f : M;
         float L = 0.0f, A = 0.0f;
 #pragma unroll
-        for (int w = 0; w < DEC_WAVES; w++) {
+        for (int w = 0; w < WAVES; w++) {
             const float *src = macc + (w * DM_HEADS + hh) * (D + 2);
             const float wgt = __builtin_amdgcn_exp2f(src[D] - Ms);
             L += wgt * src[D + 1];
@@ -1125,11 +1137,21 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     }
     if constexpr (!F32) {
         if (decode_use_mfma(p.D, false)) {
-            switch (p.D) {
-                case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32>), grid, block, stream, p, p); break;
-                case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64>), grid, block, stream, p, p); break;
-                case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96>), grid, block, stream, p, p); break;
-                default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128>), grid, block, stream, p, p); break;
+            if (p.dec_waves == 8) {
+                const dim3 block8(64 * 8);
+                switch (p.D) {
+                    case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, 8>), grid, block8, stream, p, p); break;
+                    case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, 8>), grid, block8, stream, p, p); break;
+                    case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, 8>), grid, block8, stream, p, p); break;
+                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, 8>), grid, block8, stream, p, p); break;
+                }
+            } else {
+                switch (p.D) {
+                    case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, DEC_WAVES>), grid, block, stream, p, p); break;
+                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, DEC_WAVES>), grid, block, stream, p, p); break;
+                }
             }
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);

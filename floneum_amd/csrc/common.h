@@ -28,6 +28,7 @@ struct AttnParams {
     float *partials;        // [B, H, nsplit, D + 2] per-split (acc, m, l)
     int32_t chunk;          // keys per split
     int32_t nsplit;         // splits per (batch, kv head) over Skv
+    int32_t dec_waves;      // wavefronts per workgroup of the 16-bit matrix-core decode variant (4 or 8)
     // host-side only (profiling hook).  Both set: the dispatch of the main kernel carries the two events, which then
     // hold its own begin and end timestamps.  Only main_done: recorded on the stream after the main kernel.
     hipEvent_t main_start, main_done;
@@ -108,7 +109,7 @@ int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream
 // decode planning (host): keys per split and number of splits; `ragged`: per-batch key counts are given;
 // `f32`: the tensors are f32 (vector variant) rather than 16-bit
 void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool ragged, bool f32, int *chunk,
-                 int *nsplit);
+                 int *nsplit, int *waves);
 size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 
 // calibration (calibration.hip): the register-only matrix-core loop and the scratch it reports into

@@ -624,3 +624,34 @@ def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
     args = tq._attn_args(tk, tv, D ** -0.5, mt, analytic, lens_t, None, fa.KERNEL_AUTO, out_t)
     fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
     assert_parity(out_t.to_numpy(), ref, tol, f"unsplit, {case} D{D}")
+
+
+@pytest.mark.parametrize("dtype,D,Sq", [(fa.F16, 96, 1), (fa.BF16, 128, 1), (fa.F16, 64, 2), (fa.F16, 32, 1)])
+def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype, D, Sq):
+    """At least one (batch, kv head) unit per CU and more than 2048 keys: the 16-bit matrix-core variant runs with eight
+    wavefronts per workgroup on chunks of 2048 keys (fewer, longer workgroups).  All keys, then ragged lengths."""
+    B, H, Hkv, Skv = 9, 32, 32, 4500
+    assert B * Hkv >= device.compute_units
+    q, k, v = _normal_qkv(47, B, H, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
+    # three splits of 2048 keys per (batch, head, row): that is what the workspace is sized for
+    need = ctypes.c_size_t()
+    args = tq._attn_args(tk, tv, 0.1, None, None, None, None, fa.KERNEL_AUTO, None)
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+    assert need.value == B * H * Sq * 3 * (D + 2) * 4
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16)
+    analytic = (True, Skv - Sq, 0) if Sq > 1 else None
+    mask = _analytic_mask(Sq, Skv, True, Skv - Sq, 0) if Sq > 1 else None
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                 None if mask is None else "qk")
+    assert_parity(out, ref, tol, "all keys")
+    if Sq == 1:
+        lens = np.array([4500, 1, 2048, 2049, 4096, 300, 4097, 2047, 3333], np.int32)
+        out = tq.flash_attention(tk, tv, D ** -0.5, kv_lens=fa.IntTensor(device, lens)).to_numpy()
+        for b in range(B):
+            n = int(lens[b])
+            ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                         rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+            assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
