@@ -46,6 +46,12 @@ constexpr int PF_BM = 32 * PF_WAVES;  // query rows per workgroup
 constexpr int PF_BN = 64;             // key rows per tile
 constexpr float PF_LOG2E = 1.4426950408889634f;
 
+// Sensitivity switches for measurements only; never defined in a shipped build (`FHIP_EXTRA_FLAGS=-D... python -m
+// floneum_amd.build`).  Both give WRONG RESULTS on purpose: they take away half of one kind of work while the matrix
+// instructions stay the same, to see how much of the run time (i.e. of the power budget) that work costs.
+//   FHIP_EXP_HALF_LDS  every second LDS operand read is skipped (the registers keep what they held)
+//   FHIP_EXP_HALF_EXP  every second exponential is skipped
+
 #define LDS_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
 
 template <typename T>
@@ -341,6 +347,12 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         auto read_v = [&](int gq, uint4_t (&a)[NDB]) {  // gq = 2 t + kk: rows 32 t + 16 kk (+8)
 #pragma unroll
             for (int db = 0; db < NDB; db++) {
+#ifdef FHIP_EXP_HALF_LDS
+                if (db & 1) {
+                    a[db] = a[db - 1];
+                    continue;
+                }
+#endif
                 const int addr = vbase + gq * C::ROWB + db * 64;
                 short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr));
                 short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VG));
@@ -356,6 +368,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             for (int db = 0; db < NDB; db++) o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, a[db]), bop, o[db]);
         };
         auto read_k = [&](int kb, uint4_t (&a)[2]) {
+#ifdef FHIP_EXP_HALF_LDS
+            if (kb & 1) return;
+#endif
 #pragma unroll
             for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
         };
@@ -444,7 +459,11 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(s[t][r]);
+#ifdef FHIP_EXP_HALF_EXP
+                const float p1 = p0;
+#else
                 const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
+#endif
                 pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
                 l += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
             }
