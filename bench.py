@@ -7,8 +7,9 @@ A step is one attention call through the C ABI on synthetic, seeded inputs that 
 HBM before the timed region.  The default workload is C2 (Llama-3-8B-shaped decode, batch 16, 4096
 f16 KV tokens per sequence): `value` is its KV-streaming rate in GB/s (algorithmic bytes per call /
 time per call, combine pass included).  The same JSON line also carries the C3 prefill figure
-(TFLOP/s, MFMA roofline) under "prefill" and the other three benchmark configurations under
-"configs" (C1, C4, C5), each with the HBM/MFMA roofline of its dominant kernel (the kernel's own
+(TFLOP/s, MFMA roofline) under "prefill" and, under "configs", the other three benchmark configurations
+(C1, C4, C5) plus two decode workloads beside C2 (F2: the same batch with an f32 cache, M1: four new rows per
+sequence), each with the HBM/MFMA roofline of its dominant kernel (the kernel's own
 duration from HIP events carried by its dispatch on the launch stream) and the CPU checker timed on
 the host cores ("cpu_baseline").
 """
@@ -88,6 +89,10 @@ def configs():
         "S1": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
         "S2": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
         "S3": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=32768, D=128, dtype="f16", std=0.5, causal=False),
+        # C1 as kalosm-llama really calls it: the mask comes as the [512, 512] tensor MaskCache::get_mask builds, not as
+        # a formula (interval scan + tiled kernel + the kernel for masks that are not intervals, which exits at once)
+        "C1M": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True,
+                    mask_tensor=True),
         # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the vector variant of
         # the decode kernel; and a 16-bit cache with Gemma-3's key length 256, which the vector variant serves too
         "F2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
@@ -180,11 +185,17 @@ def prepare(fa, dev, c, sets, lens_t):
     """Argument blocks (one per input set) with output and workspace bound once, outside the timed region."""
     L = fa.lib()
     blocks = []
+    mask = None
+    if c.get("mask_tensor"):
+        # the tensor the reference's MaskCache builds for this call, written on the device
+        dt = {"f32": fa.F32, "f16": fa.F16}[c["dtype"]]
+        off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
+        mask = (fa.MaskCache(dt).get_mask_on_device(c["Sq"], off, c.get("window") or None, dev).mask(), fa.MaskKind.QKMask)
     for (q, k, v) in sets:
         analytic = None
-        if c["causal"]:
+        if c["causal"] and mask is None:
             analytic = (True, c.get("q_pos_offset", c["Skv"] - c["Sq"]), c.get("window", 0))
-        args = q._attn_args(k, v, c["D"] ** -0.5, None, analytic, lens_t, None, fa.KERNEL_AUTO, None)
+        args = q._attn_args(k, v, c["D"] ** -0.5, mask, analytic, lens_t, None, fa.KERNEL_AUTO, None)
         need = ctypes.c_size_t()
         fa.check(L.fhip_flash_attention_workspace_bytes(ctypes.byref(args), dev.compute_units, ctypes.byref(need)))
         if need.value:
@@ -584,7 +595,9 @@ def main():
         line["prefill"]["mfma_calibration"] = calibration_mfma()
         # the remaining benchmark configurations, each a line of its own in miniature
         line["configs"] = {}
-        for name, (steps, warmup) in (("C1", (200, 20)), ("C4", (100, 100)), ("C5", (20, 3))):
+        # (F2: C2's batch with the f32 cache kalosm-llama keeps; M1: C2's batch with four new rows per sequence)
+        for name, (steps, warmup) in (("C1", (200, 20)), ("C4", (100, 100)), ("C5", (20, 3)), ("F2", (100, 10)),
+                                      ("M1", (100, 10))):
             r = run_config(name, steps, warmup, with_cpu=not a.no_cpu)
             r["steps"], r["warmup"] = steps, warmup
             line["configs"][name] = r
