@@ -221,6 +221,52 @@ static void test_capture(const Device &d) {  // a recorded rope call replays on 
            h[4], h[5], h[6], h[7]);
 }
 
+// A multi-token decode step through the cache, as a turn that feeds three tokens on top of a cached context does
+// (models/kalosm-llama/src/raw/mod.rs:618-620: the mask is get_mask(3, pos, None)).  With all keys equal every
+// visible key weighs the same, and with V[j][d] = j the output of row r is the mean of 0 .. n_r - 1, n_r = pos + r + 1.
+static void test_multi_token_step_on_a_cache(const Device &d) {
+    const uint32_t H = 4, Hkv = 2, D = 64, pos = 700, n = 3;
+    KvCache cache(d, 2, 4096);
+    std::vector<float> k(Hkv * pos * D, 0.25f), v(Hkv * pos * D);
+    for (uint32_t g = 0; g < Hkv; g++)
+        for (uint32_t j = 0; j < pos; j++)
+            for (uint32_t e = 0; e < D; e++) v[(g * pos + j) * D + e] = (float)j;
+    cache.append(d, t4(d, k, 1, Hkv, pos, D), t4(d, v, 1, Hkv, pos, D));
+    std::vector<float> kn(Hkv * n * D, 0.25f), vn(Hkv * n * D);
+    for (uint32_t g = 0; g < Hkv; g++)
+        for (uint32_t j = 0; j < n; j++)
+            for (uint32_t e = 0; e < D; e++) vn[(g * n + j) * D + e] = (float)(pos + j);
+    auto all = cache.append(d, t4(d, kn, 1, Hkv, n, D), t4(d, vn, 1, Hkv, n, D));
+    EXPECT(all.first.shape()[2] == pos + n, "cache holds the context and the new rows");
+    std::vector<float> q(H * n * D, 0.5f);
+    auto tq = t4(d, q, 1, H, n, D);
+    MaskCache masks;
+    auto am = masks.get_mask(n, pos, std::nullopt, d);
+    EXPECT(am.mask().shape()[0] == n && am.mask().shape()[1] == pos + n, "mask [3, pos + 3]");
+    auto out_t = tq.flash_attention(all.first, all.second, 0.125f, std::make_pair(&am.mask(), MaskKind::QKMask));
+    auto out = host(out_t);
+    auto out_a = host(tq.flash_attention(all.first, all.second, 0.125f, std::nullopt, &*am.analytic()));
+    for (uint32_t h = 0; h < H; h++)
+        for (uint32_t r = 0; r < n; r++) {
+            const float want = 0.5f * (float)(pos + r);  // mean of 0 .. pos + r
+            const float got = out[(h * n + r) * D + 7], got_a = out_a[(h * n + r) * D + 7];
+            EXPECT(std::fabs(got - want) < 1e-3f * want, "head %u row %u: %f, want %f", h, r, got, want);
+            EXPECT(got == got_a, "mask tensor and analytic descriptor differ: %f vs %f", got, got_a);
+        }
+}
+
+// the benchmark's calibration entry points, called through the C header
+static void test_calibrations(const Device &d) {
+    const size_t cus = (size_t)d.info().compute_units;
+    Buffer scratch(d, cus * 1040), data(d, 1 << 20);
+    check(fhip_memset(d.stream(), data.ptr(), 0, 1 << 20));
+    check(fhip_calibration_read(d.stream(), data.ptr(), 1 << 20, scratch.ptr(), cus * 1040));
+    check(fhip_calibration_mfma(d.stream(), FHIP_F16, 1, 100, 50, scratch.ptr(), cus * 1040));
+    check(fhip_stream_synchronize(d.stream()));
+    EXPECT(fhip_calibration_mfma(d.stream(), FHIP_F32, 1, 100, 50, scratch.ptr(), cus * 1040) == FHIP_ERR_UNSUPPORTED,
+           "the matrix-core loop takes 16-bit types");
+}
+
 int main() {
     try {
         Device d(0);
@@ -234,6 +280,8 @@ int main() {
         test_rope(d);
         test_rms_norm(d);
         test_capture(d);
+        test_multi_token_step_on_a_cache(d);
+        test_calibrations(d);
     } catch (const std::exception &e) {
         printf("exception: %s\n", e.what());
         return 2;
