@@ -196,8 +196,14 @@ static bool rows_vectorizable(const fhip_tensor4 &t, int eb, int bytes = 16) {
 constexpr uint32_t DECODE_MAX_ROWS = 4;
 
 static bool decode_eligible(const fhip_attn_args *a) {
-    const uint32_t D = a->q.shape[3];
-    if (a->q.shape[2] < 1 || a->q.shape[2] > DECODE_MAX_ROWS) return false;
+    const uint32_t D = a->q.shape[3], rows = a->q.shape[2];
+    if (rows < 1) return false;
+    if (rows > DECODE_MAX_ROWS) {
+        // more rows (a longer draft) still ride along while rows x group fit the 16 columns of one matrix-core block
+        const uint32_t Hkv = a->k.shape[1], G = Hkv ? a->q.shape[1] / Hkv : 0;
+        const bool matrix_variant = D == 32 || D == 64 || D == 96 || D == 128;
+        if (!matrix_variant || G == 0 || rows * G > 16) return false;
+    }
     if (D % 8 != 0 || D < 8 || D > 256) return false;
     const int eb = a->dtype == FHIP_F32 ? 4 : 2;
     if (!rows_vectorizable(a->k, eb) || !rows_vectorizable(a->v, eb)) return false;

@@ -141,9 +141,11 @@ typedef enum {
     FHIP_KERNEL_PREFILL_F32 = 3, /* f32 arithmetic on the f32 MFMA, LDS-tiled: f32 tensors, and 16-bit tensors
                                     (widened on load) the kernel above does not take; head_dim multiple of
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */
-    FHIP_KERNEL_DECODE_SPLITKV = 4 /* Sq == 1, head_dim multiple of 8 up to 256: split-KV streaming + LSE
-                                      combine (matrix cores for f16/bf16 at head_dim 32/64/96/128, vector
-                                      units otherwise)                                                 */
+    FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence (up to 16 while rows x GQA group <= 16 at
+                                      head_dim 32/64/96/128), head_dim multiple of 8 up to 256: split-KV
+                                      streaming + LSE combine (matrix cores at head_dim 32/64/96/128, on the
+                                      16-bit or the f32 instruction by the tensors' type; vector units
+                                      otherwise)                                                       */
 } fhip_kernel_id;
 
 

@@ -116,3 +116,28 @@ def test_rows_fully_masked_by_their_own_limits_are_nan(device):
     assert np.isnan(out[:, :, [1, 3]]).all()
     ref = oracle.flash_attention(q, k, v, D ** -0.5)
     assert_parity(out[:, :, [0, 2]], ref[:, :, [0, 2]], TOL_F32, "visible rows")
+
+
+@pytest.mark.parametrize("dtype,G,Sq,D", [(fa.F16, 1, 16, 128), (fa.F32, 2, 8, 64), (fa.BF16, 1, 9, 96), (fa.F16, 4, 4, 128)])
+def test_longer_drafts_while_rows_times_group_fit_one_block(device, dtype, G, Sq, D):
+    """Up to 16 rows when rows x GQA group fit the 16 columns of one matrix-core block (a 16-token draft on an MHA model);
+    one row more, or a head_dim the matrix-core variants do not take, and the call is a prefill call again."""
+    B, Hkv, Skv = 2, 2, 2100
+    q, k, v = _normal_qkv(45, B, Hkv * G, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    analytic = (True, Skv - Sq, 0)
+    assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 _analytic_mask(Sq, Skv, True, Skv - Sq, 0), "qk")
+    assert_parity(out, ref, _tol(dtype), f"G{G} Sq{Sq} D{D}")
+    if Sq * G == 16:
+        q2 = np.concatenate([q, q[:, :, :1]], 2)
+        t2 = fa.Tensor.from_numpy(device, q2, dtype)
+        assert t2.selected_kernel(tk, tv, 0.1, analytic=(True, Skv - Sq - 1, 0)) != fa.KERNEL_DECODE_SPLITKV
+
+
+def test_five_rows_at_a_head_dim_of_the_vector_variant_is_a_prefill_call(device):
+    q, k, v = _normal_qkv(46, 1, 2, 2, 5, 300, 80)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
+    assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_PREFILL_F32
