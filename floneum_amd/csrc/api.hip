@@ -254,6 +254,10 @@ static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
 // The f32 tiled kernel can add a mask tensor element by element (no scratch, no interval form) up to head_dim 128.
 static bool f32_adds_masks(const fhip_attn_args *a) { return a->q.shape[3] <= 128; }
 
+// At head_dim <= 64 the f32 tiled kernel holds both mask forms: it reads what the scan found and no hand-over kernel
+// is queued behind it.
+static bool f32_serves_both_mask_forms(const fhip_attn_args *a) { return a->q.shape[3] <= 64; }
+
 // Key split of a call the f32-arithmetic tiled kernel serves (few query rows on a long cache), and where its
 // partial results go in the workspace: behind the mask scratch, 256-byte aligned.
 static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
@@ -764,8 +768,9 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     }
     if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && args->mask_kind != FHIP_MASK_NONE) {
         // dense mask: reduce it to one visible interval per row on the device; the tiled kernel skips the
-        // masked tiles if every row is of that form.  If not, the kernel queued right behind it takes the
-        // call: the f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
+        // masked tiles if every row is of that form.  If not, the f32-arithmetic kernel at head_dim <= 64 adds the
+        // mask values itself; otherwise the kernel queued right behind the tiled one takes the call: the
+        // f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
         do p.bad_tag = (int32_t)s->dev->next_tag.fetch_add(1, std::memory_order_relaxed);
@@ -784,9 +789,12 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         AttnParams pt = p;
         pt.iv = iv;
         pt.iv_bad = bad;
+        const bool both_forms = id == FHIP_KERNEL_PREFILL_F32 && f32_serves_both_mask_forms(args);
+        pt.iv_either = both_forms ? 1 : 0;
         rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, args->dtype, s->s);
         if (rc) return rc;
         FHIP_MARK_MAIN_DONE(p, s->s);
+        if (both_forms) return FHIP_OK;
         AttnParams pg = p;
         pg.only_if_bad = bad;
         pg.main_start = pg.main_done = nullptr;  // the hook times the tiled kernel

@@ -9,6 +9,7 @@
 // that need no element test).
 #pragma once
 #include "common.h"
+#include "device_utils.h"
 
 namespace fhip {
 
@@ -20,18 +21,18 @@ struct RowBounds {
 };
 
 // q0: first row of the workgroup, bm: rows per workgroup, qw0: first row of the wavefront (32 rows,
-// lane ln = lane % 32 owns row qw0 + ln)
-__device__ __forceinline__ RowBounds row_bounds(const AttnParams &p, int b, int q0, int bm, int qw0, int lane) {
+// lane ln = lane % 32 owns row qw0 + ln).  iv: the interval form of the mask tensor, or NULL.
+__device__ __forceinline__ RowBounds row_bounds(const AttnParams &p, const int2 *iv, int b, int q0, int bm, int qw0, int lane) {
     const int ln = lane & 31;
     int kv_lo = 0, kv_hi = p.Skv;
     if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
-    if (p.iv && p.mask_kind == FHIP_MASK_BATCH_KEY) {
-        const int2 t = p.iv[b];
+    if (iv && p.mask_kind == FHIP_MASK_BATCH_KEY) {
+        const int2 t = iv[b];
         kv_lo = max(kv_lo, t.x);
         kv_hi = min(kv_hi, t.y);
     }
     RowBounds r;
-    if (!(p.iv && p.mask_kind == FHIP_MASK_QK)) {
+    if (!(iv && p.mask_kind == FHIP_MASK_QK)) {
         const int64_t off = p.q_pos_offset;
         auto row_lo = [&](int q) __attribute__((always_inline)) -> int {
             return (p.analytic && p.window > 0) ? (int)max((int64_t)kv_lo, (int64_t)q + off - p.window + 1) : kv_lo;
@@ -52,20 +53,16 @@ __device__ __forceinline__ RowBounds row_bounds(const AttnParams &p, int b, int 
     }
     constexpr int NONE = 0x7fffffff;
     auto load_row = [&](int q, int &lo, int &hi) __attribute__((always_inline)) {
-        const int2 t = p.iv[min(q, p.Sq - 1)];
+        const int2 t = iv[min(q, p.Sq - 1)];
         lo = max(kv_lo, t.x);
         hi = min(kv_hi, t.y);
         if (hi <= lo) lo = hi = 0;  // nothing visible
     };
     auto wave_min = [&](int x) __attribute__((always_inline)) -> int {
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) x = min(x, __shfl_xor(x, o, 64));
-        return __builtin_amdgcn_readfirstlane(x);
+        return __builtin_amdgcn_readfirstlane(wave_reduce_i(x, [](int a, int b) { return min(a, b); }));
     };
     auto wave_max = [&](int x) __attribute__((always_inline)) -> int {
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) x = max(x, __shfl_xor(x, o, 64));
-        return __builtin_amdgcn_readfirstlane(x);
+        return __builtin_amdgcn_readfirstlane(wave_reduce_i(x, [](int a, int b) { return max(a, b); }));
     };
     load_row(qw0 + ln, r.klo, r.khi);
     const bool empty = r.khi == 0;
@@ -85,6 +82,10 @@ __device__ __forceinline__ RowBounds row_bounds(const AttnParams &p, int b, int 
     r.hi_wg = wave_max(hi_u);
     if (r.hi_wg <= r.lo_wg) r.lo_wg = r.hi_wg = 0;
     return r;
+}
+
+__device__ __forceinline__ RowBounds row_bounds(const AttnParams &p, int b, int q0, int bm, int qw0, int lane) {
+    return row_bounds(p, p.iv, b, q0, bm, qw0, lane);
 }
 
 }  // namespace fhip

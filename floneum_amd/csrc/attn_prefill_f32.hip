@@ -70,11 +70,19 @@ __device__ __forceinline__ float half_swap_sum32(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// BIAS: the additive mask tensor is applied as it is, element by element (p.mask, no interval form): finite
-// biases, several visible runs per row, NaN or +inf entries.  Score = (q.k * scale) + mask as in the reference
-// (fusor flash_attention.rs:145,177), every key tile is visited.
-template <typename T, int D, int S, bool BIAS>
+// How a mask tensor is applied (MODE):
+//   PF32_INTERVALS  by interval: analytic description, key counts, or the interval form a scan launch left in p.iv
+//   PF32_BIAS       the tensor is added as it is, element by element (p.mask, no interval form): finite biases,
+//                   several visible runs per row, NaN or +inf entries.  Score = (q.k * scale) + mask as in the
+//                   reference (fusor flash_attention.rs:145,177), every key tile is visited.
+//   PF32_EITHER     decided when the kernel starts, from the word the scan launch in front of it left in *p.iv_bad:
+//                   by interval (p.iv) if every row of the mask is one, else the values are added.  No hand-over
+//                   launch behind the tiled kernel; head_dim <= 64 (the register budget of both forms in one kernel).
+constexpr int PF32_INTERVALS = 0, PF32_BIAS = 1, PF32_EITHER = 2;
+
+template <typename T, int D, int S, int MODE>
 __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnParams p, int nqb) {
+    constexpr bool BIAS = MODE != PF32_INTERVALS;  // the mask-adding code is in the kernel
     constexpr int WPG = PF32_WAVES / S;   // wavefronts per key-split group
     constexpr int BM = 32 * WPG;          // query rows per workgroup
     // Which head dims a 32-row block of O^T holds.  With 2 or 4 blocks, row i of block db is dim NDB i + db: the
@@ -98,9 +106,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     __shared__ __attribute__((aligned(16))) char smem[S * G_BYTES];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
-    if constexpr (BIAS) {
+    if constexpr (MODE == PF32_BIAS) {
         if (p.only_if_bad && *p.only_if_bad != p.bad_tag) return;  // the interval form of the mask has served the call
-    } else {
+    } else if constexpr (MODE == PF32_INTERVALS) {
         if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the BIAS form takes the call
     }
     const int tid = threadIdx.x;
@@ -127,7 +135,24 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int q0 = qb * BM;
     const int qw0 = q0 + 32 * wig;
     const int query = qw0 + ln;
-    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    // Q operand: Q[query][8 kc + 4 h2 .. +4]; requested before the bounds, whose table reads (mask tensors) would
+    // otherwise delay these loads by a memory latency
+    float4_t qreg[D / 8];
+    {
+        const int qrow = min(query, p.Sq - 1);
+        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
+#pragma unroll
+        for (int kc = 0; kc < D / 8; kc++)
+            qreg[kc] = 8 * kc + 4 * h2 < p.D ? load4(qp + 8 * kc + 4 * h2) : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    // uniform over the launch
+    const bool bias_on = MODE == PF32_BIAS || (MODE == PF32_EITHER && *p.iv_bad == p.bad_tag);
+    RowBounds rb = row_bounds(p, MODE == PF32_BIAS ? nullptr : p.iv, b, q0, BM, qw0, lane);
+    if constexpr (MODE == PF32_EITHER) {
+        // the table was read whatever the scan found (its loads need not wait for that word); without the interval
+        // form the bounds are those of a call whose mask is added
+        if (bias_on) rb = row_bounds(p, nullptr, b, q0, BM, qw0, lane);
+    }
     if (nks > 1) {  // this workgroup's share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -138,15 +163,6 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int lo_wg = rb.lo_wg, hi_wg = rb.hi_wg, lo_w = rb.lo_w, hi_w = rb.hi_w;
     const bool wave_has_rows = qw0 < p.Sq;
 
-    // Q operand: Q[query][8 kc + 4 h2 .. +4]
-    float4_t qreg[D / 8];
-    {
-        const int qrow = min(query, p.Sq - 1);
-        const T *qp = (const T *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
-#pragma unroll
-        for (int kc = 0; kc < D / 8; kc++)
-            qreg[kc] = 8 * kc + 4 * h2 < p.D ? load4(qp + 8 * kc + 4 * h2) : float4_t{0.f, 0.f, 0.f, 0.f};
-    }
     const T *kg = (const T *)p.k + b * p.ks[0] + g * p.ks[1];
     const T *vg = (const T *)p.v + b * p.vs[0] + g * p.vs[1];
 
@@ -158,7 +174,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     float m = -INFINITY, l = 0.0f;
     // scores reach the softmax in the base-2 domain: raw dot products times scale * log2(e); with BIAS they are
     // scaled, biased, and then only multiplied by log2(e)
-    const float scale2 = BIAS ? PF32_LOG2E : p.scale * PF32_LOG2E;
+    const float scale2 = bias_on ? PF32_LOG2E : p.scale * PF32_LOG2E;
     const T *mrow = nullptr;
     if constexpr (BIAS)
         mrow = (const T *)p.mask + (int64_t)(p.mask_kind == FHIP_MASK_QK ? min(query, p.Sq - 1) : b) * p.ms0;
@@ -175,10 +191,12 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     auto tile_math = [&](int j0, int voff, auto &&between) __attribute__((always_inline)) {
         float bias[BIAS ? 16 : 1];
         if constexpr (BIAS) {  // requested before the matrix work that hides their latency
+            if (bias_on) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                bias[r] = key < p.Skv ? to_float(mrow[(int64_t)key * p.ms1]) : 0.0f;
+                for (int r = 0; r < 16; r++) {
+                    const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                    bias[r] = key < p.Skv ? to_float(mrow[(int64_t)key * p.ms1]) : 0.0f;
+                }
             }
         }
 
@@ -203,8 +221,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         }
 
         if constexpr (BIAS) {
+            if (bias_on) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[r] = s[r] * p.scale + bias[r];
+                for (int r = 0; r < 16; r++) s[r] = s[r] * p.scale + bias[r];
+            }
         }
 
         float mx = s[0];
@@ -425,8 +445,9 @@ __global__ __launch_bounds__(256) void prefill_f32_merge_kernel(AttnParams p) {
     const int lane = threadIdx.x & 63;
     const int64_t rows = (int64_t)p.B * p.H * p.Sq;
     if (row >= rows) return;
-    // the same hand-over between the interval form and the mask-adding form as in the main kernel
-    if ((p.iv_bad && *p.iv_bad == p.bad_tag) || (p.only_if_bad && *p.only_if_bad != p.bad_tag)) return;
+    // the same hand-over between the interval form and the mask-adding form as in the main kernel (none when the
+    // main kernel held both forms)
+    if (!p.iv_either && ((p.iv_bad && *p.iv_bad == p.bad_tag) || (p.only_if_bad && *p.only_if_bad != p.bad_tag))) return;
     const int query = (int)(row % p.Sq);
     const int h = (int)((row / p.Sq) % p.H), b = (int)(row / p.Sq / p.H);
     const int D = p.D, ns = p.pf_nsplit, pitch = p.pf_pitch;
@@ -710,8 +731,9 @@ int launch_prefill_merge(const AttnParams &p, fhip_dtype dtype, hipStream_t stre
     return launch_merge_t<float>(p, stream);
 }
 
-template <typename T, int S, bool BIAS>
+template <typename T, int S, int MODE>
 static int launch_split(const AttnParams &p, hipStream_t stream) {
+    constexpr bool BIAS = MODE != PF32_INTERVALS;
     constexpr int BM = 32 * (PF32_WAVES / S);
     const int nqb = (p.Sq + BM - 1) / BM;
     const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
@@ -721,13 +743,15 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)blocks), block(64 * PF32_WAVES);
     switch ((p.D + 31) / 32 * 32) {  // the kernel's D is head_dim rounded up to a multiple of 32
-        case 32: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 32, S, BIAS>), grid, block, stream, p, p, nqb); break;
-        case 64: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 64, S, BIAS>), grid, block, stream, p, p, nqb); break;
+        case 32: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 32, S, MODE>), grid, block, stream, p, p, nqb); break;
+        case 64: FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 64, S, MODE>), grid, block, stream, p, p, nqb); break;
         case 96:
-            if constexpr (S <= (BIAS ? 1 : 4)) FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 96, S, BIAS>), grid, block, stream, p, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4) && MODE != PF32_EITHER)
+                FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 96, S, MODE>), grid, block, stream, p, p, nqb);
             break;
         case 128:
-            if constexpr (S <= (BIAS ? 1 : 4)) FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 128, S, BIAS>), grid, block, stream, p, p, nqb);
+            if constexpr (S <= (BIAS ? 1 : 4) && MODE != PF32_EITHER)
+                FHIP_LAUNCH_MAIN((prefill_f32_kernel<T, 128, S, MODE>), grid, block, stream, p, p, nqb);
             break;
         default: set_error("prefill f32 kernel: head_dim %d is not a multiple of 4 up to 128", p.D); return FHIP_ERR_UNSUPPORTED;
     }
@@ -781,6 +805,11 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
     if (sizeof(T) != 4) split = 1;
     // a mask tensor without its interval form is added element by element (the 16 bias registers leave no
     // room for the key-split form at head_dim 96 / 128)
+    const bool either = p.mask && p.iv && p.iv_either;  // the kernel reads the scan's verdict itself
+    if (either && !small_dim) {
+        set_error("internal: the two-form f32 kernel takes head_dim <= 64");
+        return FHIP_ERR_UNSUPPORTED;
+    }
     const bool add_mask = p.mask && !p.iv;
     if (add_mask && !small_dim) split = 1;
     AttnParams ps = p;
@@ -788,18 +817,25 @@ static int launch_prefill_f32_t(const AttnParams &p, hipStream_t stream) {
         const long blocks = bh * ((p.Sq + 128 / split - 1) / (128 / split));
         ps.snake_cus = (blocks > cus && blocks <= 2L * cus) ? cus : 0;
     }
+    if (either) {
+        if constexpr (sizeof(T) == 4) {
+            if (split == 4) return launch_split<T, 4, PF32_EITHER>(ps, stream);
+            if (split == 2) return launch_split<T, 2, PF32_EITHER>(ps, stream);
+        }
+        return launch_split<T, 1, PF32_EITHER>(ps, stream);
+    }
     if (add_mask) {
         if constexpr (sizeof(T) == 4) {
-            if (split == 4) return launch_split<T, 4, true>(ps, stream);
-            if (split == 2) return launch_split<T, 2, true>(ps, stream);
+            if (split == 4) return launch_split<T, 4, PF32_BIAS>(ps, stream);
+            if (split == 2) return launch_split<T, 2, PF32_BIAS>(ps, stream);
         }
-        return launch_split<T, 1, true>(ps, stream);
+        return launch_split<T, 1, PF32_BIAS>(ps, stream);
     }
     if constexpr (sizeof(T) == 4) {
-        if (split == 4) return launch_split<T, 4, false>(ps, stream);
-        if (split == 2) return launch_split<T, 2, false>(ps, stream);
+        if (split == 4) return launch_split<T, 4, PF32_INTERVALS>(ps, stream);
+        if (split == 2) return launch_split<T, 2, PF32_INTERVALS>(ps, stream);
     }
-    return launch_split<T, 1, false>(ps, stream);
+    return launch_split<T, 1, PF32_INTERVALS>(ps, stream);
 }
 
 int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {

@@ -38,6 +38,9 @@ struct AttnParams {
     // `iv` does nothing when *iv_bad == bad_tag; the kernel given `only_if_bad` does nothing when
     // *only_if_bad != bad_tag: exactly one of the two computes the result.
     const int2 *iv;
+    // With iv_either set the f32-arithmetic tiled kernel (head_dim <= 64) serves the call whatever the scan found: it
+    // masks by interval when *iv_bad != bad_tag and adds the mask values otherwise, and no second kernel is queued.
+    int32_t iv_either;
     const int32_t *iv_bad;
     const int32_t *only_if_bad;
     // What the scan writes to *iv_bad when a row is not of that form: a value unique to the call, so that the word

@@ -113,4 +113,22 @@ __device__ __forceinline__ float group_sum32(float x) {
     return x;
 }
 
+template <int ctrl>
+__device__ __forceinline__ int dpp_mov_i(int x) {
+    return (int)__builtin_amdgcn_update_dpp(0u, (uint32_t)x, ctrl, 0xf, 0xf, true);
+}
+// reduction over the 64 lanes of a wavefront, result in every lane: four DPP steps inside the rows of 16 lanes, two
+// swaps across them (no LDS traffic, unlike __shfl_xor)
+template <typename OP>
+__device__ __forceinline__ int wave_reduce_i(int x, OP op) {
+    x = op(x, dpp_mov_i<DPP_QUAD_XOR1>(x));
+    x = op(x, dpp_mov_i<DPP_QUAD_XOR2>(x));
+    x = op(x, dpp_mov_i<DPP_ROW_HALF_MIRROR>(x));
+    x = op(x, dpp_mov_i<DPP_ROW_MIRROR>(x));
+    auto a = __builtin_amdgcn_permlane16_swap((uint32_t)x, (uint32_t)x, false, false);
+    x = op((int)a[0], (int)a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap((uint32_t)x, (uint32_t)x, false, false);
+    return op((int)b[0], (int)b[1]);
+}
+
 }  // namespace fhip

@@ -90,13 +90,10 @@ __global__ __launch_bounds__(64 * MI_WAVES) void mask_intervals_kernel(const cha
             take(j, bits);
         }
     }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-        lo = min(lo, __shfl_xor(lo, o, 64));
-        hi = max(hi, __shfl_xor(hi, o, 64));
-        zeros += __shfl_xor(zeros, o, 64);
-        others += __shfl_xor(others, o, 64);
-    }
+    lo = wave_reduce_i(lo, [](int a, int b) { return min(a, b); });
+    hi = wave_reduce_i(hi, [](int a, int b) { return max(a, b); });
+    zeros = wave_reduce_i(zeros, [](int a, int b) { return a + b; });
+    others = __builtin_amdgcn_ballot_w64(others != 0) != 0 ? 1 : 0;
     if (lane == 0) {
         if (hi == 0) lo = 0;  // no visible key at all: the empty interval
         const bool ok = others == 0 && zeros == hi - lo;  // only zeros and -inf, and the zeros are one run

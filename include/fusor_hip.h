@@ -213,7 +213,8 @@ int fhip_flash_attention_validate(const fhip_attn_args *args);
  * with a mask tensor and a sufficient workspace in `args` this names the tiled kernel, which runs if
  * the mask turns out to be made of intervals (decided on the device) and otherwise hands over, inside
  * the same call, to the kernel that adds the mask values one by one (the mask-adding form of the
- * f32-arithmetic tiled kernel up to head_dim 128, the general kernel above); without the workspace it
+ * f32-arithmetic tiled kernel up to head_dim 128, the general kernel above; at head_dim <= 64 the
+ * f32-arithmetic tiled kernel holds both forms and nothing is handed over); without the workspace it
  * names that kernel.  The answer does not depend on the device: how a kernel splits its work over the
  * compute units is planned inside the call, and fhip_flash_attention_workspace_bytes takes their number
  * because the scratch for those splits does. */

@@ -239,3 +239,88 @@ def test_masks_built_on_the_device_equal_the_host_builders(device, dtype):
         assert on_dev.shape == host.shape, (seq, off, w)
         want = fa.Tensor.from_numpy(device, host, dtype).to_numpy()
         assert np.array_equal(on_dev.view(np.uint8), want.view(np.uint8)), (seq, off, w)
+
+
+# ---- head_dim <= 64: the f32 tiled kernel holds both mask forms ---------------------------------------------------
+# Two launches (the scan, the tiled kernel) and no hand-over kernel: the tiled kernel reads what the scan found and
+# masks by interval (bit for bit the analytic call) or adds the mask values, also in its key-split forms.
+
+def _qk_call(device, dtype, q, k, v, mask, **kw):
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    return tq, tk, tv, tq.flash_attention(tk, tv, q.shape[-1] ** -0.5, (tm, fa.MaskKind.QKMask), **kw).to_numpy()
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 64), (fa.F32, 32), (fa.F32, 48), (fa.F16, 40), (fa.BF16, 16)])
+@pytest.mark.parametrize("seq,offset,window", [(512, 0, None), (40, 0, None), (200, 312, None), (96, 160, 64), (304, 0, 7),
+                                               (64, 960, None), (33, 95, None)])
+def test_mask_tensors_made_of_intervals_on_the_two_form_kernel(device, dtype, D, seq, offset, window):
+    mask = oracle.get_mask(seq, offset, window)
+    Skv = mask.shape[1]
+    q, k, v = _normal_qkv(61, 2, 4, 2, seq, Skv, D)
+    tq, tk, tv, out = _qk_call(device, dtype, q, k, v, mask)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "qk")
+    assert_parity(out, ref, _tol(dtype), f"get_mask({seq},{offset},{window}) D{D}")
+    out_a = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, Skv - seq, window or 0)).to_numpy()
+    assert np.array_equal(out.view(np.uint8), out_a.view(np.uint8)), "the interval form was not taken"
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 64), (fa.F32, 32), (fa.F16, 40)])
+@pytest.mark.parametrize("kind", ["bias", "two_runs", "bias_in_some_blocks", "empty_rows", "plus_inf", "block_diagonal"])
+def test_masks_that_are_not_intervals_on_the_two_form_kernel(device, dtype, D, kind):
+    B, H, Hkv, Sq, Skv = 2, 4, 2, 200, 328
+    rng = np.random.default_rng(9)
+    q, k, v = _normal_qkv(62, B, H, Hkv, Sq, Skv, D)
+    mask = oracle.get_mask(Sq, Skv - Sq, None).copy()
+    if kind == "bias":
+        mask = np.where(np.isneginf(mask), mask, rng.normal(0, 1, mask.shape)).astype(np.float32)
+    elif kind == "two_runs":
+        mask[:, 40:50] = NEG_INF      # a hole in every row that reaches it
+    elif kind == "bias_in_some_blocks":
+        mask[70:75, 3] = -2.5         # a few finite entries: the whole call adds values
+        mask[199, 0] = 0.75
+    elif kind == "empty_rows":
+        mask[5, :] = NEG_INF          # rows without a visible key: NaN on both sides
+        mask[130, :] = NEG_INF
+    elif kind == "plus_inf":
+        mask[9, 2] = np.inf
+    elif kind == "block_diagonal":
+        mask[:] = NEG_INF
+        for lo, hi in ((0, 60), (60, 61), (61, 200)):
+            mask[lo:hi, lo:hi + 100] = 0
+    tq, tk, tv, out = _qk_call(device, dtype, q, k, v, mask)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, rounded(mask, dtype), "qk")
+    dead = np.isnan(ref).any(-1)
+    assert np.array_equal(np.isnan(out).any(-1), dead), "rows without a usable value differ"
+    if (~dead).any():
+        assert_parity(out[~dead], ref[~dead], _tol(dtype), kind)
+
+
+@pytest.mark.parametrize("fill", [NEG_INF, -10000.0])
+def test_padding_masks_on_the_two_form_kernel(device, fill):
+    """A BatchKeyMask row per batch: -inf padding is an interval, rbert's -10000.0 is added as it is."""
+    B, H, Hkv, Sq, Skv, D = 3, 4, 4, 150, 256, 64
+    q, k, v = _normal_qkv(63, B, H, Hkv, Sq, Skv, D)
+    mask = np.zeros((B, Skv), np.float32)
+    mask[0, 200:] = fill
+    mask[1, :31] = fill
+    tq, tk, tv, tm = _tensors(device, fa.F32, q, k, v, mask)
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.BatchKeyMask)).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "batch_key")
+    assert_parity(out, ref, TOL_F32, f"padding with {fill}")
+
+
+def test_strided_mask_views_on_the_two_form_kernel(device):
+    """Mask rows that are not contiguous or not 16-byte aligned."""
+    B, H, Hkv, Sq, Skv, D = 1, 4, 2, 100, 200, 64
+    q, k, v = _normal_qkv(64, B, H, Hkv, Sq, Skv, D)
+    mask = oracle.get_mask(Sq, Skv - Sq, None)
+    wide = np.zeros((Sq, Skv + 3), np.float32)
+    wide[:, 1:Skv + 1] = mask
+    tq, tk, tv = _tensors(device, fa.F32, q, k, v)
+    tm = fa.Tensor.from_numpy(device, wide, fa.F32).narrow(1, 1, Skv)       # rows start 4 bytes off a 16-byte boundary
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tm, fa.MaskKind.QKMask)).to_numpy()
+    ref = oracle.flash_attention(q, k, v, D ** -0.5, mask, "qk")
+    assert_parity(out, ref, TOL_F32, "misaligned rows")
+    tmt = fa.Tensor.from_numpy(device, np.ascontiguousarray(mask.T), fa.F32).transpose(0, 1)  # column-major mask
+    out = tq.flash_attention(tk, tv, D ** -0.5, (tmt, fa.MaskKind.QKMask)).to_numpy()
+    assert_parity(out, ref, TOL_F32, "transposed mask")
