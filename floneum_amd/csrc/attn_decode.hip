@@ -50,8 +50,11 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
     *waves = DEC_WAVES;
-    if (decode_use_mfma(D, f32) && !f32 && units >= compute_units && Skv > 2048) {
-        // the 8-wavefront form of the 16-bit matrix-core variant: whole units for every CU, chunks of 2048 keys
+    // the 8-wavefront form of the 16-bit matrix-core variant, chunks of 2048 keys: when every CU gets a whole unit, or,
+    // with more than 8 columns per unit (a multi-token step: twice the matrix and softmax work per key), a chunk
+    const long chunks2048 = (Skv + 2047) / 2048;
+    if (decode_use_mfma(D, f32) && !f32 && Skv > 2048 &&
+        (units >= compute_units || (G > 8 && units * chunks2048 >= compute_units))) {
         *waves = 8;
         *chunk = 2048;
         *nsplit = (Skv + 2047) / 2048;

@@ -76,13 +76,15 @@ def test_decode_step_replayed_with_growing_key_counts(device, dtype):
             assert_parity(replayed[b:b + 1], ref, tol, f"replay {it} sequence {b}")
 
 
-def test_masked_prefill_replayed(device):
-    """A prefill call with a mask tensor is three launches (interval scan, tiled kernel, the kernel for masks that are
-    not intervals), plus, under capture, a kernel that clears the word the scan marks: all of it is recorded, and the
-    mask content may change between replays, from the interval form to a bias and back.  A replay whose mask is made
-    of intervals again must run on the interval form again (a mark left behind by the bias replay would send every
-    later replay to the mask-adding kernel): its result equals the eager call's bit for bit, and the analytic call's."""
-    B, H, Hkv, S, D = 1, 4, 2, 200, 64
+@pytest.mark.parametrize("D", [64, 128])
+def test_masked_prefill_replayed(device, D):
+    """A prefill call with a mask tensor is several launches: the interval scan and the tiled kernel (which at
+    head_dim 64 holds both mask forms), at head_dim 128 also the kernel for masks that are not intervals, plus, under
+    capture, a kernel that clears the word the scan marks.  All of it is recorded, and the mask content may change
+    between replays, from the interval form to a bias and back.  A replay whose mask is made of intervals again must
+    run on the interval form again (a mark left behind by the bias replay would send every later replay to the
+    mask-adding form): its result equals the eager call's bit for bit, and the analytic call's."""
+    B, H, Hkv, S = 1, 4, 2, 200
     q, k, v = _normal_qkv(52, B, H, Hkv, S, S, D)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
     tm = fa.Tensor.empty(device, (S, S), fa.F32)

@@ -80,6 +80,26 @@ def test_multi_token_step(device, dtype, G, D, Sq, Skv, case):
     assert_parity(out, ref, _tol(dtype), f"{case} G{G} D{D} Sq{Sq} Skv{Skv}")
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("case", ["causal", "window", "full"])
+def test_multi_token_step_of_a_batch_that_fills_the_chip(device, dtype, case):
+    """More than 8 columns per KV head and enough (batch, KV head, 2048-key chunk) units for every compute unit: the step
+    runs on the 8-wavefront form of the 16-bit kernel; the last chunk holds 4 keys."""
+    B, Hkv, G, D, Sq, Skv = 11, 8, 4, 128, 3, 4100
+    q, k, v = _normal_qkv(47, B, Hkv * G, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    off = Skv - Sq
+    analytic, mask = {"causal": ((True, off, 0), _analytic_mask(Sq, Skv, True, off, 0)),
+                      "window": ((True, off, 2500), _analytic_mask(Sq, Skv, True, off, 2500)),
+                      "full": (None, None)}[case]
+    kw = {"analytic": analytic} if analytic else {}
+    assert tq.selected_kernel(tk, tv, 0.1, **kw) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, **kw).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                 None if mask is None else "qk")
+    assert_parity(out, ref, _tol(dtype), f"{case}")
+
+
 @pytest.mark.parametrize("dtype", [fa.F16, fa.F32])
 def test_multi_token_step_ragged_batch_and_padding_mask(device, dtype):
     """Per-sequence key counts and a BatchKeyMask on a multi-token step; the output written as [B, Sq, H, D]."""
