@@ -93,8 +93,9 @@ def configs():
         # a formula (interval scan + tiled kernel + the kernel for masks that are not intervals, which exits at once)
         "C1M": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True,
                     mask_tensor=True),
-        # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the vector variant of
-        # the decode kernel; and a 16-bit cache with Gemma-3's key length 256, which the vector variant serves too
+        # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the f32 matrix-core
+        # variant of the decode kernel; and a 16-bit cache with Gemma-3's key length 256 (the 16-bit matrix-core variant
+        # with one workgroup per CU)
         "F2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
         "W2": dict(kind="decode", B=16, H=16, Hkv=4, Sq=1, Skv=4096, D=256, dtype="f16", std=0.5, causal=False),
         # a multi-token decode step: C2's batch with four new rows per sequence at the end of the cache, causal among

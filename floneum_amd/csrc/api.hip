@@ -201,7 +201,7 @@ static bool decode_eligible(const fhip_attn_args *a) {
     if (rows > DECODE_MAX_ROWS) {
         // more rows (a longer draft) still ride along while rows x group fit the 16 columns of one matrix-core block
         const uint32_t Hkv = a->k.shape[1], G = Hkv ? a->q.shape[1] / Hkv : 0;
-        const bool matrix_variant = D == 32 || D == 64 || D == 96 || D == 128;
+        const bool matrix_variant = D % 32 == 0 && D >= 32 && D <= (a->dtype == FHIP_F32 ? 192u : 256u);
         if (!matrix_variant || G == 0 || rows * G > 16) return false;
     }
     if (D % 8 != 0 || D < 8 || D > 256) return false;

@@ -31,11 +31,11 @@ constexpr int DEC_WAVES = 4;
 constexpr int DEC_UNROLL = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 
-// the matrix-core variants: 16-bit tensors on the 16-bit instruction, f32 tensors on the f32 one; other head dims
-// run on the vector variant
+// the matrix-core variants: 16-bit tensors on the 16-bit instruction at every multiple of 32 up to 256, f32 tensors on
+// the f32 one up to 192 (at 256 the vector variant measured 3 % ahead).  Above 128 one workgroup per CU, whose four
+// wavefronts then have the registers and LDS of eight.  Other head dims run on the vector variant.
 static bool decode_use_mfma(int D, bool f32) {
-    (void)f32;
-    return D == 32 || D == 64 || D == 96 || D == 128;
+    return D % 32 == 0 && D >= 32 && D <= (f32 ? 192 : 256);
 }
 
 // query heads handled by one workgroup
@@ -53,17 +53,17 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // the 8-wavefront form of the 16-bit matrix-core variant, chunks of 2048 keys: when every CU gets a whole unit, or,
     // with more than 8 columns per unit (a multi-token step: twice the matrix and softmax work per key), a chunk
     const long chunks2048 = (Skv + 2047) / 2048;
-    if (decode_use_mfma(D, f32) && !f32 && Skv > 2048 &&
+    if (decode_use_mfma(D, f32) && !f32 && D <= 128 && Skv > 2048 &&
         (units >= compute_units || (G > 8 && units * chunks2048 >= compute_units))) {
         *waves = 8;
         *chunk = 2048;
         *nsplit = (Skv + 2047) / 2048;
         return;
     }
-    // the MFMA variant holds two workgroups per CU (LDS), the vector variant four or more; f32 rows carry
+    // the MFMA variant holds two workgroups per CU (LDS; one above head_dim 128), the vector variant four or more; f32 rows carry
     // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at
     // batch 1 with 32768 keys)
-    const int wgs_per_cu = (decode_use_mfma(D, f32) || f32) ? 2 : 4;
+    const int wgs_per_cu = (decode_use_mfma(D, f32) && D > 128) ? 1 : (decode_use_mfma(D, f32) || f32) ? 2 : 4;
     const long target = (long)compute_units * wgs_per_cu;
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
@@ -452,7 +452,7 @@ constexpr int DM_HEADS = 16; // query heads per workgroup (MFMA N dimension)
 // memory system is loaded, so with work enough to keep every CU busy anyway, fewer and longer workgroups stream
 // better (32 ragged sequences of up to 32768 keys: 6.45 -> 6.83 TB/s).
 template <typename T, int D, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void decode_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mfma_kernel(AttnParams p) {
     typedef typename DecMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;          // K tile row pitch (bytes): rows 4 banks apart
     constexpr int VP = D * 2 + 32;          // V tile row pitch (bytes): rows 8 banks apart
@@ -721,7 +721,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void decode_mfma_kernel(Attn
 constexpr int DF_KEYS = 16;  // keys per wavefront step
 
 template <int D>
-__global__ __launch_bounds__(64 * DEC_WAVES, 2) void decode_mfma_f32_kernel(AttnParams p) {
+__global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f32_kernel(AttnParams p) {
     constexpr int KP = D * 4 + 16;             // tile row pitch (bytes): rows 4 banks apart
     constexpr int K_BYTES = DF_KEYS * KP;
     constexpr int WAVE_BYTES = 2 * K_BYTES;    // K tile, V tile
@@ -1127,7 +1127,9 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
                 case 32: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<32>), grid, block, stream, p, p); break;
                 case 64: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<64>), grid, block, stream, p, p); break;
                 case 96: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<96>), grid, block, stream, p, p); break;
-                default: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128>), grid, block, stream, p, p); break;
+                case 128: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128>), grid, block, stream, p, p); break;
+                case 160: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<160>), grid, block, stream, p, p); break;
+                default: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<192>), grid, block, stream, p, p); break;
             }
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);
@@ -1153,7 +1155,11 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
                     case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, DEC_WAVES>), grid, block, stream, p, p); break;
                     case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, DEC_WAVES>), grid, block, stream, p, p); break;
                     case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, DEC_WAVES>), grid, block, stream, p, p); break;
-                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 128: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 160: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 160, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 192: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 192, DEC_WAVES>), grid, block, stream, p, p); break;
+                    case 224: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 224, DEC_WAVES>), grid, block, stream, p, p); break;
+                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 256, DEC_WAVES>), grid, block, stream, p, p); break;
                 }
             }
             FHIP_HIP_CHECK(hipGetLastError());

@@ -142,10 +142,10 @@ typedef enum {
                                     (widened on load) the kernel above does not take; head_dim multiple of
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */
     FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence (up to 16 while rows x GQA group <= 16 at
-                                      head_dim 32/64/96/128), head_dim multiple of 8 up to 256: split-KV
-                                      streaming + LSE combine (matrix cores at head_dim 32/64/96/128, on the
-                                      16-bit or the f32 instruction by the tensors' type; vector units
-                                      otherwise)                                                       */
+                                      the matrix-core head dims), head_dim multiple of 8 up to 256: split-KV
+                                      streaming + LSE combine (matrix cores at every multiple of 32: up to 256
+                                      on the 16-bit instruction, up to 192 on the f32 one, by the tensors'
+                                      type; vector units otherwise)                                     */
 } fhip_kernel_id;
 
 

@@ -361,7 +361,7 @@ def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
 @pytest.mark.parametrize("G,D,Skv", [(4, 128, 1000), (1, 96, 777), (8, 64, 513), (2, 128, 64), (3, 128, 300),
                                      (4, 32, 5000), (1, 128, 1), (16, 128, 260), (20, 64, 700), (4, 72, 900),
                                      (2, 40, 333), (8, 8, 100), (2, 256, 1500), (4, 192, 700), (1, 160, 300),
-                                     (8, 256, 260)])
+                                     (8, 256, 260), (4, 224, 2100), (16, 256, 130)])
 def test_decode_splitkv(device, dtype, G, D, Skv):
     B, Hkv = 3, 2
     q, k, v = _normal_qkv(12, B, Hkv * G, Hkv, 1, Skv, D, 0.5)
@@ -402,7 +402,9 @@ def test_decode_f32_with_the_masks_the_reference_passes(device):
 
 
 @pytest.mark.parametrize("dtype,B,H,Hkv,D,Skv", [(fa.F16, 1, 8, 2, 128, 6000), (fa.F32, 1, 4, 2, 256, 5200),
-                                                  (fa.F32, 2, 6, 3, 64, 9000), (fa.BF16, 3, 4, 1, 96, 7000)])
+                                                  (fa.F32, 2, 6, 3, 64, 9000), (fa.BF16, 3, 4, 1, 96, 7000),
+                                                  (fa.F16, 1, 8, 4, 256, 9000), (fa.BF16, 2, 4, 2, 160, 6000),
+                                                  (fa.F32, 1, 8, 4, 192, 5000)])
 def test_decode_with_many_splits_and_few_rows(device, dtype, B, H, Hkv, D, Skv):
     """One chat stream on a long cache: tens of splits per (batch, head) row and only a few rows, which the combine
     pass handles with four wavefronts per row (two rounds of 128 dims at head_dim 256); ragged lengths on top."""
@@ -420,6 +422,38 @@ def test_decode_with_many_splits_and_few_rows(device, dtype, B, H, Hkv, D, Skv):
         ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
                                      rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
         assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
+@pytest.mark.parametrize("case", ["window", "window_as_tensor", "padding_mask", "full"])
+def test_decode_at_head_dim_256_with_a_sliding_window(device, dtype, case):
+    """Gemma-3's attention shape (key length 256, 8 query heads on 4 KV heads, sliding layers with a window of 1024):
+    a decode step on a long cache, the window as the analytic descriptor and as the [1, Skv] tensor
+    MaskCache::get_mask builds; a left- and right-padded batch as a BatchKeyMask.  16-bit tensors run on the
+    matrix-core variant (one workgroup per CU at this head_dim), f32 tensors on the vector variant."""
+    B, H, Hkv, D, Skv, W = 5, 8, 4, 256, 3100, 1024
+    q, k, v = _normal_qkv(71, B, H, Hkv, 1, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16)
+    mask = kind = None
+    kw = {}
+    m = None
+    if case in ("window", "window_as_tensor"):
+        mask, kind = _analytic_mask(1, Skv, True, Skv - 1, W), "qk"
+        if case == "window":
+            kw["analytic"] = (True, Skv - 1, W)
+        else:
+            m = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "padding_mask":
+        mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+        mask[0, 3000:] = NEG_INF
+        mask[1, :700] = NEG_INF
+        mask[3, 1:] = NEG_INF
+        m = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.BatchKeyMask)
+    assert tq.selected_kernel(tk, tv, 0.1, m, **kw) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, m, **kw).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, kind)
+    assert_parity(out, ref, tol, case)
 
 
 def test_decode_ragged_kv_lens(device):
