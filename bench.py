@@ -101,6 +101,8 @@ def configs():
         # a multi-token decode step: C2's batch with four new rows per sequence at the end of the cache, causal among
         # themselves (a draft being verified); the rows ride beside the heads of a GQA group, the cache is read once
         "M1": dict(kind="decode", B=16, H=32, Hkv=8, Sq=4, Skv=4096, D=128, dtype="f16", std=0.5, causal=True),
+        # eight new rows per sequence: 32 columns per KV head, two column blocks per workgroup of the decode kernel
+        "M2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=8, Skv=4096, D=128, dtype="f16", std=0.5, causal=True),
     }
 
 

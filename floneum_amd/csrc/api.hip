@@ -199,10 +199,13 @@ static bool decode_eligible(const fhip_attn_args *a) {
     const uint32_t D = a->q.shape[3], rows = a->q.shape[2];
     if (rows < 1) return false;
     if (rows > DECODE_MAX_ROWS) {
-        // more rows (a longer draft) still ride along while rows x group fit the 16 columns of one matrix-core block
+        // more rows (a longer draft, a short piece of a prompt) still ride along while rows x group fit the columns one
+        // workgroup of a matrix-core variant takes: two blocks of 16 up to head_dim 128, one above
         const uint32_t Hkv = a->k.shape[1], G = Hkv ? a->q.shape[1] / Hkv : 0;
         const bool matrix_variant = D % 32 == 0 && D >= 32 && D <= (a->dtype == FHIP_F32 ? 192u : 256u);
-        if (!matrix_variant || G == 0 || rows * G > 16) return false;
+        uint32_t max_cols = D <= 128 ? 32u : 16u;
+        if (a->dtype == FHIP_F32) max_cols *= 2;  // two workgroups per KV head (each streams the cache) still beat the f32 prefill kernel
+        if (!matrix_variant || G == 0 || rows * G > max_cols) return false;
     }
     if (D % 8 != 0 || D < 8 || D > 256) return false;
     const int eb = a->dtype == FHIP_F32 ? 4 : 2;

@@ -38,9 +38,10 @@ static bool decode_use_mfma(int D, bool f32) {
     return D % 32 == 0 && D >= 32 && D <= (f32 ? 192 : 256);
 }
 
-// query heads handled by one workgroup
+// columns ((query head, query row) pairs of a KV head) handled by one workgroup: the matrix-core variants take one
+// block of 16, or two up to head_dim 128 when there are more than 16 columns
 static int decode_gt(int G, int D, bool f32) {
-    if (decode_use_mfma(D, f32)) return 16;
+    if (decode_use_mfma(D, f32)) return (G > 16 && D <= 128) ? 32 : 16;
     return G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
 }
 
@@ -451,7 +452,10 @@ constexpr int DM_HEADS = 16; // query heads per workgroup (MFMA N dimension)
 // least one (batch, kv head) unit per CU: a workgroup's first tile takes several microseconds to arrive while the
 // memory system is loaded, so with work enough to keep every CU busy anyway, fewer and longer workgroups stream
 // better (32 ragged sequences of up to 32768 keys: 6.45 -> 6.83 TB/s).
-template <typename T, int D, int WAVES>
+// CB: 16-column blocks per workgroup.  With two, the K and V tiles a wavefront has parked in LDS serve 32 columns (a
+// multi-token step with up to 32 (query head, query row) pairs per KV head): every LDS operand read feeds a matrix step
+// for each block, and each block keeps its own softmax state.
+template <typename T, int D, int WAVES, int CB>
 __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mfma_kernel(AttnParams p) {
     typedef typename DecMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;          // K tile row pitch (bytes): rows 4 banks apart
@@ -463,13 +467,14 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     constexpr int NLD = DM_KEYS * CPR / 64; // 16-byte loads per lane per tile
     constexpr int KB = D / 32;              // contraction blocks of QK^T
     constexpr int NB = D / 16;              // 16-dim blocks of the output
-    constexpr int MERGE_BYTES = WAVES * DM_HEADS * (D + 2) * 4;
+    constexpr int COLS = DM_HEADS * CB;     // columns per workgroup
+    constexpr int MERGE_BYTES = WAVES * COLS * (D + 2) * 4;
     constexpr int LDS_BYTES = WAVES * WAVE_BYTES > MERGE_BYTES ? WAVES * WAVE_BYTES : MERGE_BYTES;
     __shared__ __attribute__((aligned(16))) char smem[LDS_BYTES];
 
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int j = lane & 15;  // head column of this lane
+    const int j = lane & 15;  // column of this lane inside each block
     const int q4 = lane >> 4; // key group
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
@@ -478,15 +483,19 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     // row c % rows of the group (one row per head in a plain decode step, a few in a multi-token step).
     const int rows = p.Sq;
     const int NC = p.G * rows;
-    const int HB = (NC + DM_HEADS - 1) / DM_HEADS;
+    const int HB = (NC + COLS - 1) / COLS;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
-    const int c0 = hb * DM_HEADS;
-    const int nh = min(DM_HEADS, NC - c0);  // columns in use
-    const int cj = c0 + min(j, nh - 1);     // this lane's column
-    const int hj = g * p.G + cj / rows, rj = cj % rows;
+    const int c0 = hb * COLS;
+    const int nh = min(COLS, NC - c0);  // columns in use
+    int hj[CB], rj[CB];                 // head and row of this lane's column in block cb
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const int cj = c0 + min(j + DM_HEADS * cb, nh - 1);
+        hj[cb] = g * p.G + cj / rows, rj[cb] = cj % rows;
+    }
 
     int kv_hi = p.Skv;
     if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
@@ -494,29 +503,38 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     // [lo, hi): the keys some row of the workgroup sees; [lo_j, hi_j): the keys this lane's row sees
     int lo = split * p.chunk;
     int hi = min(lo + p.chunk, kv_hi);
-    int lo_j = lo, hi_j = hi;
+    int lo_j[CB], hi_j[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        lo_j[cb] = lo, hi_j[cb] = hi;
+        if (p.analytic && p.causal) hi_j[cb] = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj[cb]);
+        if (p.analytic && p.window > 0) lo_j[cb] = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj[cb]);
+    }
     if (p.analytic) {
-        if (p.causal) {
-            hi_j = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj);
-            hi = (int)min((int64_t)hi, p.q_pos_offset + rows);  // the last row sees furthest
-        }
-        if (p.window > 0) {
-            lo_j = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj);
-            lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);  // the first row sees the earliest key
-        }
+        if (p.causal) hi = (int)min((int64_t)hi, p.q_pos_offset + rows);                // the last row sees furthest
+        if (p.window > 0) lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);    // the first row sees the earliest key
     }
 
     const uint16_t *kbase = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
     const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
-    const T *mrow = nullptr;
-    if (p.mask_kind == FHIP_MASK_QK) mrow = (const T *)p.mask + rj * p.ms0;
-    if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const T *)p.mask + b * p.ms0;
+    const T *mrow[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        mrow[cb] = nullptr;
+        if (p.mask_kind == FHIP_MASK_QK) mrow[cb] = (const T *)p.mask + rj[cb] * p.ms0;
+        if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow[cb] = (const T *)p.mask + b * p.ms0;
+    }
+    const bool has_mask = p.mask_kind != FHIP_MASK_NONE;
     const float scale2 = p.scale * LOG2E;
 
-    float4_t o[NB];
+    float4_t o[CB][NB];
+    float m[CB], l[CB];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) o[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.0f;
+    for (int cb = 0; cb < CB; cb++) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) o[cb][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+        m[cb] = -INFINITY, l[cb] = 0.0f;
+    }
 
     // one wavefront step = 32 consecutive keys; the four wavefronts interleave their steps
     const int lo_al = lo - (lo % DM_KEYS);
@@ -558,14 +576,15 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     }
 
     // Q^T operand: column j, dims 32 kb + 8 q4 .. +8 (zero for the padding columns)
-    vec8 qreg[KB];
-    {
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + (int64_t)hj * p.qs[1] + (int64_t)rj * p.qs[2];
+    vec8 qreg[CB][KB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + (int64_t)hj[cb] * p.qs[1] + (int64_t)rj[cb] * p.qs[2];
         const bool qvec = p.qs[3] == 1 && (((uintptr_t)qp) & 15) == 0;
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
             uint4_t raw = {0, 0, 0, 0};
-            if (j < nh) {
+            if (j + DM_HEADS * cb < nh) {
                 if (qvec) {
                     raw = *(const uint4_t *)(qp + 32 * kb + 8 * q4);
                 } else {
@@ -578,7 +597,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
                     raw = uint4_t{w[0], w[1], w[2], w[3]};
                 }
             }
-            qreg[kb] = __builtin_bit_cast(vec8, raw);
+            qreg[cb][kb] = __builtin_bit_cast(vec8, raw);
         }
     }
 
@@ -589,54 +608,61 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
         wave_lds_sync();
         load_tile(base + DEPTH * step, set);  // in flight during the math below (beyond the end: a row read again)
 
-        // ---- S^T[key][head] = K . Q^T : two 16-key tiles --------------------------------------------
-        float4_t s[2];
+        // ---- S^T[key][col] = K . Q^T : two 16-key tiles, every K operand read serves all column blocks -------
+        float4_t s[CB][2];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) s[cb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb = 0; kb < KB; kb++) {
                 const uint4_t raw = *DLDS_PTR(uint4_t, (16 * t + j) * KP + (32 * kb + 8 * q4) * 2);
-                s[t] = DecMma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], s[t]);
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++)
+                    s[cb][t] = DecMma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[cb][kb], s[cb][t]);
             }
         }
-        // element (t, r) is key base + 16 t + 4 q4 + r for column j
-        float sv[8];
+        vec8 pop[CB];
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+        for (int cb = 0; cb < CB; cb++) {
+            // element (t, r) is key base + 16 t + 4 q4 + r for column j of block cb
+            float sv[8];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int key = base + 16 * t + 4 * q4 + r;
-                const bool visible = key >= lo_j && key < hi_j;
-                float x = s[t][r] * scale2;
-                if (mrow && visible) x += to_float(mrow[(int64_t)key * p.ms1]) * LOG2E;
-                sv[4 * t + r] = visible ? x : -INFINITY;
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int key = base + 16 * t + 4 * q4 + r;
+                    const bool visible = key >= lo_j[cb] && key < hi_j[cb];
+                    float x = s[cb][t][r] * scale2;
+                    if (has_mask && visible) x += to_float(mrow[cb][(int64_t)key * p.ms1]) * LOG2E;
+                    sv[4 * t + r] = visible ? x : -INFINITY;
+                }
+            float mx = sv[0];
+#pragma unroll
+            for (int e = 1; e < 8; e++) mx = fmaxf(mx, sv[e]);
+            mx = quad_rows_max(mx);
+            const float m_new = fmaxf(m[cb], mx);
+            const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(m[cb] - m_safe);
+            m[cb] = m_new;
+            float pe[8], psum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                pe[e] = __builtin_amdgcn_exp2f(sv[e] - m_safe);
+                psum += pe[e];
             }
-        float mx = sv[0];
+            l[cb] = l[cb] * corr + psum;
 #pragma unroll
-        for (int e = 1; e < 8; e++) mx = fmaxf(mx, sv[e]);
-        mx = quad_rows_max(mx);
-        const float m_new = fmaxf(m, mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
-        m = m_new;
-        float pe[8], psum = 0.0f;
+            for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            pe[e] = __builtin_amdgcn_exp2f(sv[e] - m_safe);
-            psum += pe[e];
+                for (int r = 0; r < 4; r++) o[cb][nb][r] *= corr;
+            // P^T operand: contraction slot (q4, e) is key 4 q4 + e (e < 4) or 16 + 4 q4 + e - 4
+            const uint4_t praw = {DecMma<T>::pack2(pe[0], pe[1]), DecMma<T>::pack2(pe[2], pe[3]),
+                                  DecMma<T>::pack2(pe[4], pe[5]), DecMma<T>::pack2(pe[6], pe[7])};
+            pop[cb] = __builtin_bit_cast(vec8, praw);
         }
-        l = l * corr + psum;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) o[nb][r] *= corr;
-        // P^T operand: contraction slot (q4, e) is key 4 q4 + e (e < 4) or 16 + 4 q4 + e - 4
-        const uint4_t praw = {DecMma<T>::pack2(pe[0], pe[1]), DecMma<T>::pack2(pe[2], pe[3]),
-                              DecMma<T>::pack2(pe[4], pe[5]), DecMma<T>::pack2(pe[6], pe[7])};
-        const vec8 pop = __builtin_bit_cast(vec8, praw);
 
-        // ---- O^T[dim][head] += V^T . P^T ----------------------------------------------------------------
+        // ---- O^T[dim][col] += V^T . P^T -----------------------------------------------------------------
         // the transposing load hands lane i of a 16-lane block V[row0 + 0..3][dim0 + i]; the lane
         // supplies the address of row0 + i / 4, dims dim0 + 4 (i % 4)
         const int trow = 4 * q4 + (j >> 2);
@@ -649,7 +675,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
                 DLDS_PTR(short4_t, K_BYTES + (16 + trow) * VP + nb * 32 + tcol));
             const uint2v_t u0 = __builtin_bit_cast(uint2v_t, a0), u1 = __builtin_bit_cast(uint2v_t, a1);
             const uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
-            o[nb] = DecMma<T>::mfma(__builtin_bit_cast(vec8, araw), pop, o[nb]);
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+                o[cb][nb] = DecMma<T>::mfma(__builtin_bit_cast(vec8, araw), pop[cb], o[cb][nb]);
         }
     };
     for (; base < hi; base += DEPTH * step) {
@@ -659,18 +687,21 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     }
 
     // ---- merge: key groups -> wavefront -> workgroup ------------------------------------------------
-    l = quad_rows_sum(l);
     __syncthreads();  // every wavefront is done with its K/V tile; the LDS is reused for the merge
-    float *macc = (float *)smem;  // [wave][head][D + 2]
-    if (j < nh) {
-        float *dst = macc + ((wave * DM_HEADS + j) * (D + 2));
+    float *macc = (float *)smem;  // [wave][column][D + 2]
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
+    for (int cb = 0; cb < CB; cb++) {
+        const float l_col = quad_rows_sum(l[cb]);
+        if (j + DM_HEADS * cb < nh) {
+            float *dst = macc + ((wave * COLS + j + DM_HEADS * cb) * (D + 2));
 #pragma unroll
-            for (int r = 0; r < 4; r++) dst[16 * nb + 4 * q4 + r] = o[nb][r];
-        if (q4 == 0) {
-            dst[D] = m;
-            dst[D + 1] = l;
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) dst[16 * nb + 4 * q4 + r] = o[cb][nb][r];
+            if (q4 == 0) {
+                dst[D] = m[cb];
+                dst[D + 1] = l_col;
+            }
         }
     }
     __syncthreads();
@@ -678,12 +709,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
         const int hh = idx / D, d = idx % D;
         float M = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
+        for (int w = 0; w < WAVES; w++) M = fmaxf(M, macc[(w * COLS + hh) * (D + 2) + D]);
         const float Ms = (M == -INFINITY) ? 0.0f : M;
         float L = 0.0f, A = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) {
-            const float *src = macc + (w * DM_HEADS + hh) * (D + 2);
+            const float *src = macc + (w * COLS + hh) * (D + 2);
             const float wgt = __builtin_amdgcn_exp2f(src[D] - Ms);
             L += wgt * src[D + 1];
             A += wgt * src[d];
@@ -720,7 +751,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
 // the softmax of a column is computed once, by the four lanes that hold its 16 scores.
 constexpr int DF_KEYS = 16;  // keys per wavefront step
 
-template <int D>
+template <int D, int CB>  // CB: 16-column blocks per workgroup, see decode_mfma_kernel
 __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f32_kernel(AttnParams p) {
     constexpr int KP = D * 4 + 16;             // tile row pitch (bytes): rows 4 banks apart
     constexpr int K_BYTES = DF_KEYS * KP;
@@ -731,59 +762,73 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
     constexpr int KC = D / 16;                 // 16-dim chunks of the contraction of K . Q^T
     constexpr int VW = (D % 64 == 0) ? 4 : 2;  // dims per V read
     constexpr int NBLK = D / (16 * VW);        // output blocks of 16 VW dims
-    constexpr int MERGE_BYTES = DEC_WAVES * DM_HEADS * (D + 2) * 4;
+    constexpr int COLS = DM_HEADS * CB;        // columns per workgroup
+    constexpr int MERGE_BYTES = DEC_WAVES * COLS * (D + 2) * 4;
     constexpr int LDS_BYTES = DEC_WAVES * WAVE_BYTES > MERGE_BYTES ? DEC_WAVES * WAVE_BYTES : MERGE_BYTES;
     __shared__ __attribute__((aligned(16))) char smem[LDS_BYTES];
 
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
-    const int j = lane & 15;  // column of this lane
+    const int j = lane & 15;  // column of this lane inside each block
     const int q4 = lane >> 4; // key group
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
     const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
     const int rows = p.Sq;  // columns are (query head, query row) pairs, see decode_mfma_kernel
     const int NC = p.G * rows;
-    const int HB = (NC + DM_HEADS - 1) / DM_HEADS;
+    const int HB = (NC + COLS - 1) / COLS;
     const int hb = blockIdx.y % HB;
     const int bg = blockIdx.y / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
-    const int c0 = hb * DM_HEADS;
-    const int nh = min(DM_HEADS, NC - c0);
-    const int cj = c0 + min(j, nh - 1);
-    const int hj = g * p.G + cj / rows, rj = cj % rows;
+    const int c0 = hb * COLS;
+    const int nh = min(COLS, NC - c0);
+    int hj[CB], rj[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const int cj = c0 + min(j + DM_HEADS * cb, nh - 1);
+        hj[cb] = g * p.G + cj / rows, rj[cb] = cj % rows;
+    }
 
     int kv_hi = p.Skv;
     if (p.kv_lens) kv_hi = min(kv_hi, max(p.kv_lens[b], 0));
     if (p.kv_lens && split * p.chunk >= kv_hi && split > 0) return;  // the combine pass skips it too
     int lo = split * p.chunk;
     int hi = min(lo + p.chunk, kv_hi);
-    int lo_j = lo, hi_j = hi;
+    int lo_j[CB], hi_j[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        lo_j[cb] = lo, hi_j[cb] = hi;
+        if (p.analytic && p.causal) hi_j[cb] = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj[cb]);
+        if (p.analytic && p.window > 0) lo_j[cb] = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj[cb]);
+    }
     if (p.analytic) {
-        if (p.causal) {
-            hi_j = (int)min((int64_t)hi, p.q_pos_offset + 1 + rj);
-            hi = (int)min((int64_t)hi, p.q_pos_offset + rows);
-        }
-        if (p.window > 0) {
-            lo_j = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1 + rj);
-            lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
-        }
+        if (p.causal) hi = (int)min((int64_t)hi, p.q_pos_offset + rows);
+        if (p.window > 0) lo = (int)max((int64_t)lo, p.q_pos_offset - p.window + 1);
     }
 
     const float *kbase = (const float *)p.k + b * p.ks[0] + g * p.ks[1];
     const float *vbase = (const float *)p.v + b * p.vs[0] + g * p.vs[1];
-    const float *mrow = nullptr;
-    if (p.mask_kind == FHIP_MASK_QK) mrow = (const float *)p.mask + rj * p.ms0;
-    if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow = (const float *)p.mask + b * p.ms0;
+    const float *mrow[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        mrow[cb] = nullptr;
+        if (p.mask_kind == FHIP_MASK_QK) mrow[cb] = (const float *)p.mask + rj[cb] * p.ms0;
+        if (p.mask_kind == FHIP_MASK_BATCH_KEY) mrow[cb] = (const float *)p.mask + b * p.ms0;
+    }
+    const bool has_mask = p.mask_kind != FHIP_MASK_NONE;
     const float scale2 = p.scale * LOG2E;
 
-    float4_t o[NBLK][VW];
+    float4_t o[CB][NBLK][VW];
+    float m[CB], l[CB];
 #pragma unroll
-    for (int nb = 0; nb < NBLK; nb++)
+    for (int cb = 0; cb < CB; cb++) {
 #pragma unroll
-        for (int e = 0; e < VW; e++) o[nb][e] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.0f;
+        for (int nb = 0; nb < NBLK; nb++)
+#pragma unroll
+            for (int e = 0; e < VW; e++) o[cb][nb][e] = float4_t{0.f, 0.f, 0.f, 0.f};
+        m[cb] = -INFINITY, l[cb] = 0.0f;
+    }
 
     // one wavefront step = 16 consecutive keys; the four wavefronts interleave their steps.  Every lane always loads
     // (rows outside [lo, hi) are replaced by the nearest one inside; their scores are masked below).
@@ -814,14 +859,15 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
     if (base < hi) load_tile(base);  // issued first so the Q fetch below overlaps it
 
     // Q^T operand: column j, dims 16 c + 4 q4 .. +4 (zero for the padding columns)
-    float4_t qreg[KC];
-    {
-        const float *qp = (const float *)p.q + b * p.qs[0] + (int64_t)hj * p.qs[1] + (int64_t)rj * p.qs[2];
+    float4_t qreg[CB][KC];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const float *qp = (const float *)p.q + b * p.qs[0] + (int64_t)hj[cb] * p.qs[1] + (int64_t)rj[cb] * p.qs[2];
         const bool qvec = p.qs[3] == 1 && (((uintptr_t)qp) & 15) == 0;
 #pragma unroll
         for (int c = 0; c < KC; c++) {
             float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (j < nh) {
+            if (j + DM_HEADS * cb < nh) {
                 if (qvec) {
                     v = *(const float4_t *)(qp + 16 * c + 4 * q4);
                 } else {
@@ -829,7 +875,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
                     for (int e = 0; e < 4; e++) v[e] = qp[(int64_t)(16 * c + 4 * q4 + e) * p.qs[3]];
                 }
             }
-            qreg[c] = v;
+            qreg[cb][c] = v;
         }
     }
 
@@ -839,43 +885,51 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
         wave_lds_sync();
         load_tile(base + step);  // in flight during the math below (beyond the end: a row read again)
 
-        // ---- S^T[key][col] = K . Q^T ---------------------------------------------------------------------
-        float4_t s = {0.f, 0.f, 0.f, 0.f};
+        // ---- S^T[key][col] = K . Q^T : every K operand read serves all column blocks ----------------------
+        float4_t s[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) s[cb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
             const float4_t a = *DLDS_PTR(float4_t, j * KP + (16 * c + 4 * q4) * 4);
 #pragma unroll
-            for (int i = 0; i < 4; i++) s = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], qreg[c][i], s, 0, 0, 0);
+            for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) s[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], qreg[cb][c][i], s[cb], 0, 0, 0);
         }
-        // element r is key base + 4 q4 + r for column j
-        float sv[4];
+        float pe[CB][4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int key = base + 4 * q4 + r;
-            const bool visible = key >= lo_j && key < hi_j;
-            float x = s[r] * scale2;
-            if (mrow && visible) x += mrow[(int64_t)key * p.ms1] * LOG2E;
-            sv[r] = visible ? x : -INFINITY;
+        for (int cb = 0; cb < CB; cb++) {
+            // element r is key base + 4 q4 + r for column j of block cb
+            float sv[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int key = base + 4 * q4 + r;
+                const bool visible = key >= lo_j[cb] && key < hi_j[cb];
+                float x = s[cb][r] * scale2;
+                if (has_mask && visible) x += mrow[cb][(int64_t)key * p.ms1] * LOG2E;
+                sv[r] = visible ? x : -INFINITY;
+            }
+            float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+            mx = quad_rows_max(mx);
+            const float m_new = fmaxf(m[cb], mx);
+            const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(m[cb] - m_safe);
+            m[cb] = m_new;
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                pe[cb][r] = __builtin_amdgcn_exp2f(sv[r] - m_safe);
+                psum += pe[cb][r];
+            }
+            l[cb] = l[cb] * corr + psum;
+#pragma unroll
+            for (int nb = 0; nb < NBLK; nb++)
+#pragma unroll
+                for (int e = 0; e < VW; e++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) o[cb][nb][e][r] *= corr;
         }
-        float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-        mx = quad_rows_max(mx);
-        const float m_new = fmaxf(m, mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - m_safe);
-        m = m_new;
-        float pe[4], psum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            pe[r] = __builtin_amdgcn_exp2f(sv[r] - m_safe);
-            psum += pe[r];
-        }
-        l = l * corr + psum;
-#pragma unroll
-        for (int nb = 0; nb < NBLK; nb++)
-#pragma unroll
-            for (int e = 0; e < VW; e++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) o[nb][e][r] *= corr;
 
         // ---- O^T[dim][col] += V^T . P^T : step ks contracts the keys 4 q4 + ks ----------------------------
 #pragma unroll
@@ -886,33 +940,42 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
                 if constexpr (VW == 4) {
                     const float4_t a = *DLDS_PTR(float4_t, voff);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[ks], o[nb][e], 0, 0, 0);
+                    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            o[cb][nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[cb][ks], o[cb][nb][e], 0, 0, 0);
                 } else {
                     typedef float float2v_t __attribute__((ext_vector_type(2)));
                     const float2v_t a = *DLDS_PTR(float2v_t, voff);
 #pragma unroll
-                    for (int e = 0; e < 2; e++) o[nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[ks], o[nb][e], 0, 0, 0);
+                    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+                        for (int e = 0; e < 2; e++)
+                            o[cb][nb][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], pe[cb][ks], o[cb][nb][e], 0, 0, 0);
                 }
             }
         }
     }
 
     // ---- merge: key groups -> wavefront -> workgroup ------------------------------------------------
-    l = quad_rows_sum(l);
     __syncthreads();  // every wavefront is done with its K/V tile; the LDS is reused for the merge
     float *macc = (float *)smem;  // [wave][column][D + 2]
-    if (j < nh) {
-        float *dst = macc + ((wave * DM_HEADS + j) * (D + 2));
-        // element (nb, e, r) of this lane is dim 16 VW nb + VW (4 q4 + r) + e
 #pragma unroll
-        for (int nb = 0; nb < NBLK; nb++)
+    for (int cb = 0; cb < CB; cb++) {
+        const float l_col = quad_rows_sum(l[cb]);
+        if (j + DM_HEADS * cb < nh) {
+            float *dst = macc + ((wave * COLS + j + DM_HEADS * cb) * (D + 2));
+            // element (nb, e, r) of this lane is dim 16 VW nb + VW (4 q4 + r) + e
 #pragma unroll
-            for (int e = 0; e < VW; e++)
+            for (int nb = 0; nb < NBLK; nb++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) dst[16 * VW * nb + VW * (4 * q4 + r) + e] = o[nb][e][r];
-        if (q4 == 0) {
-            dst[D] = m;
-            dst[D + 1] = l;
+                for (int e = 0; e < VW; e++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) dst[16 * VW * nb + VW * (4 * q4 + r) + e] = o[cb][nb][e][r];
+            if (q4 == 0) {
+                dst[D] = m[cb];
+                dst[D + 1] = l_col;
+            }
         }
     }
     __syncthreads();
@@ -920,12 +983,12 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
         const int hh = idx / D, d = idx % D;
         float M = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, macc[(w * DM_HEADS + hh) * (D + 2) + D]);
+        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, macc[(w * COLS + hh) * (D + 2) + D]);
         const float Ms = (M == -INFINITY) ? 0.0f : M;
         float L = 0.0f, A = 0.0f;
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; w++) {
-            const float *src = macc + (w * DM_HEADS + hh) * (D + 2);
+            const float *src = macc + (w * COLS + hh) * (D + 2);
             const float wgt = __builtin_amdgcn_exp2f(src[D] - Ms);
             L += wgt * src[D + 1];
             A += wgt * src[d];
@@ -1110,6 +1173,42 @@ static void launch_vec(const AttnParams &p, dim3 grid, hipStream_t stream, int g
     }
 }
 
+// the matrix-core variants by head_dim; above 128 only the form with four wavefronts and one column block exists
+template <typename T, int WAVES, int CB>
+static void launch_mfma_16(const AttnParams &p, dim3 grid, hipStream_t stream) {
+    const dim3 block(64 * WAVES);
+    switch (p.D) {
+        case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, WAVES, CB>), grid, block, stream, p, p); return;
+        case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, WAVES, CB>), grid, block, stream, p, p); return;
+        case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, WAVES, CB>), grid, block, stream, p, p); return;
+        case 128: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, WAVES, CB>), grid, block, stream, p, p); return;
+        default: break;
+    }
+    if constexpr (WAVES == DEC_WAVES && CB == 1) {
+        switch (p.D) {
+            case 160: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 160, WAVES, 1>), grid, block, stream, p, p); return;
+            case 192: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 192, WAVES, 1>), grid, block, stream, p, p); return;
+            case 224: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 224, WAVES, 1>), grid, block, stream, p, p); return;
+            default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 256, WAVES, 1>), grid, block, stream, p, p); return;
+        }
+    }
+}
+template <int CB>
+static void launch_mfma_f32(const AttnParams &p, dim3 grid, hipStream_t stream) {
+    const dim3 block(64 * DEC_WAVES);
+    switch (p.D) {
+        case 32: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<32, CB>), grid, block, stream, p, p); return;
+        case 64: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<64, CB>), grid, block, stream, p, p); return;
+        case 96: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<96, CB>), grid, block, stream, p, p); return;
+        case 128: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128, CB>), grid, block, stream, p, p); return;
+        default: break;
+    }
+    if constexpr (CB == 1) {
+        if (p.D == 160) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<160, 1>), grid, block, stream, p, p);
+        else FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<192, 1>), grid, block, stream, p, p);
+    }
+}
+
 template <typename T>
 static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     constexpr bool F32 = sizeof(T) == 4;
@@ -1123,14 +1222,8 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     dim3 grid((unsigned)p.nsplit, (unsigned)gy), block(64 * DEC_WAVES);
     if constexpr (F32) {
         if (decode_use_mfma(p.D, true)) {
-            switch (p.D) {
-                case 32: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<32>), grid, block, stream, p, p); break;
-                case 64: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<64>), grid, block, stream, p, p); break;
-                case 96: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<96>), grid, block, stream, p, p); break;
-                case 128: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128>), grid, block, stream, p, p); break;
-                case 160: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<160>), grid, block, stream, p, p); break;
-                default: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<192>), grid, block, stream, p, p); break;
-            }
+            if (gt == 32) launch_mfma_f32<2>(p, grid, stream);
+            else launch_mfma_f32<1>(p, grid, stream);
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);
             if (p.nsplit > 1) {
@@ -1143,24 +1236,11 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     if constexpr (!F32) {
         if (decode_use_mfma(p.D, false)) {
             if (p.dec_waves == 8) {
-                const dim3 block8(64 * 8);
-                switch (p.D) {
-                    case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, 8>), grid, block8, stream, p, p); break;
-                    case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, 8>), grid, block8, stream, p, p); break;
-                    case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, 8>), grid, block8, stream, p, p); break;
-                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, 8>), grid, block8, stream, p, p); break;
-                }
+                if (gt == 32) launch_mfma_16<T, 8, 2>(p, grid, stream);
+                else launch_mfma_16<T, 8, 1>(p, grid, stream);
             } else {
-                switch (p.D) {
-                    case 32: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 32, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 64: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 64, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 96: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 96, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 128: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 128, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 160: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 160, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 192: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 192, DEC_WAVES>), grid, block, stream, p, p); break;
-                    case 224: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 224, DEC_WAVES>), grid, block, stream, p, p); break;
-                    default: FHIP_LAUNCH_MAIN((decode_mfma_kernel<T, 256, DEC_WAVES>), grid, block, stream, p, p); break;
-                }
+                if (gt == 32) launch_mfma_16<T, DEC_WAVES, 2>(p, grid, stream);
+                else launch_mfma_16<T, DEC_WAVES, 1>(p, grid, stream);
             }
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);

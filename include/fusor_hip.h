@@ -141,11 +141,12 @@ typedef enum {
     FHIP_KERNEL_PREFILL_F32 = 3, /* f32 arithmetic on the f32 MFMA, LDS-tiled: f32 tensors, and 16-bit tensors
                                     (widened on load) the kernel above does not take; head_dim multiple of
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */
-    FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence (up to 16 while rows x GQA group <= 16 at
-                                      the matrix-core head dims), head_dim multiple of 8 up to 256: split-KV
-                                      streaming + LSE combine (matrix cores at every multiple of 32: up to 256
-                                      on the 16-bit instruction, up to 192 on the f32 one, by the tensors'
-                                      type; vector units otherwise)                                     */
+    FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence, head_dim multiple of 8 up to 256: split-KV
+                                      streaming + LSE combine.  Matrix cores at every head_dim that is a multiple
+                                      of 32 (up to 256 on the 16-bit instruction, up to 192 on the f32 one, by
+                                      the tensors' type), vector units otherwise.  At the matrix-core head dims
+                                      more rows ride along while rows x GQA group <= 32 (16 above head_dim 128;
+                                      twice that for f32 tensors): an 8-token draft on a 4-way GQA model       */
 } fhip_kernel_id;
 
 

@@ -3,7 +3,7 @@
 The reference fuzzes its fused kernel against its unfused path over random shapes
 (fusor-ml/core/src/composite/flash_attention.rs:559-1060); this does the same through the C ABI with everything the
 boundary accepts mixed freely: the three element types, head dims on and off the tile widths (8 ... 256, odd ones for
-the general kernel), GQA group sizes, batch, decode / multi-token decode / square / chunk-on-cache / tiny / long-cache shapes, and every way
+the general kernel), GQA group sizes, batch, decode / multi-token decode / longer drafts / square / chunk-on-cache / tiny / long-cache shapes, and every way
 of masking (none, the analytic descriptor, MaskCache tensors, finite biases, padding masks with -inf or -10000.0, key
 counts).  Rows without a visible key must be NaN on both sides.
 """
@@ -34,11 +34,14 @@ def _case(rng, device):
     Hkv = int(rng.integers(1, 4))
     H = Hkv * int(rng.choice([1, 2, 4, 8]))
     B = int(rng.integers(1, 4))
-    mode = rng.choice(["decode", "multi", "square", "chunk", "tiny", "long"])
+    mode = rng.choice(["decode", "multi", "draft", "square", "chunk", "tiny", "long"])
     if mode == "decode":
         Sq, Skv = 1, int(rng.integers(1, 3000))
     elif mode == "multi":  # a multi-token decode step: a few new rows at the end of a cache
         Sq = int(rng.integers(2, 5))
+        Skv = Sq + int(rng.integers(0, 3000))
+    elif mode == "draft":  # more rows than 4: on the decode kernels while rows x GQA group fit a workgroup's columns
+        Sq = int(rng.integers(5, 17))
         Skv = Sq + int(rng.integers(0, 3000))
     elif mode == "square":
         Sq = Skv = int(rng.integers(1, 400))

@@ -1,4 +1,4 @@
-"""Multi-token decode steps (2..4 new query rows on a cache) on the split-KV decode kernels.
+"""Multi-token decode steps (a few new query rows on a cache) on the split-KV decode kernels.
 
 The reference fuzzes exactly this shape (fusor-ml/core/src/composite/flash_attention.rs:807-921: q_seq_len 1..4,
 kv_seq_len = q_seq_len + 0..31, a [q_seq_len, kv_seq_len] mask tensor); kalosm-llama reaches it when a turn feeds a
@@ -138,10 +138,16 @@ def test_rows_fully_masked_by_their_own_limits_are_nan(device):
     assert_parity(out[:, :, [0, 2]], ref[:, :, [0, 2]], TOL_F32, "visible rows")
 
 
-@pytest.mark.parametrize("dtype,G,Sq,D", [(fa.F16, 1, 16, 128), (fa.F32, 2, 8, 64), (fa.BF16, 1, 9, 96), (fa.F16, 4, 4, 128)])
-def test_longer_drafts_while_rows_times_group_fit_one_block(device, dtype, G, Sq, D):
-    """Up to 16 rows when rows x GQA group fit the 16 columns of one matrix-core block (a 16-token draft on an MHA model);
-    one row more, or a head_dim the matrix-core variants do not take, and the call is a prefill call again."""
+@pytest.mark.parametrize("dtype,G,Sq,D", [(fa.F16, 1, 16, 128), (fa.F32, 2, 8, 64), (fa.BF16, 1, 9, 96), (fa.F16, 4, 4, 128),
+                                          (fa.F16, 4, 8, 128), (fa.F32, 4, 7, 128), (fa.BF16, 2, 16, 64), (fa.F16, 1, 32, 96),
+                                          (fa.F32, 4, 8, 128), (fa.BF16, 4, 5, 128), (fa.F16, 8, 3, 32), (fa.F16, 1, 16, 256),
+                                          (fa.F32, 2, 8, 192), (fa.F32, 1, 32, 32), (fa.F32, 4, 16, 128), (fa.F32, 1, 32, 192),
+                                          (fa.F32, 4, 11, 64)])
+def test_longer_drafts_while_rows_times_group_fit_one_workgroup(device, dtype, G, Sq, D):
+    """More than 4 rows while rows x GQA group fit the columns one workgroup of a matrix-core variant takes: two blocks
+    of 16 up to head_dim 128 (an 8-token draft on a 4-way GQA model, 32 tokens on an MHA model), one block above; f32
+    tensors twice that, on two workgroups per KV head.  One row more, or a head_dim the matrix-core variants do not
+    take, and the call is a prefill call again."""
     B, Hkv, Skv = 2, 2, 2100
     q, k, v = _normal_qkv(45, B, Hkv * G, Hkv, Sq, Skv, D, 0.5)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
@@ -151,7 +157,17 @@ def test_longer_drafts_while_rows_times_group_fit_one_block(device, dtype, G, Sq
     ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
                                  _analytic_mask(Sq, Skv, True, Skv - Sq, 0), "qk")
     assert_parity(out, ref, _tol(dtype), f"G{G} Sq{Sq} D{D}")
-    if Sq * G == 16:
+    # the same rows through a sliding window and as a mask tensor (one mask row per query row)
+    w = 700
+    mask = _analytic_mask(Sq, Skv, True, Skv - Sq, w)
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "qk")
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, Skv - Sq, w)).to_numpy()
+    assert_parity(out, ref, _tol(dtype), f"window, G{G} Sq{Sq} D{D}")
+    tm = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    assert tq.selected_kernel(tk, tv, 0.1, tm) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, tm).to_numpy()
+    assert_parity(out, ref, _tol(dtype), f"window as a tensor, G{G} Sq{Sq} D{D}")
+    if Sq * G == (32 if D <= 128 else 16) * (2 if dtype == fa.F32 else 1):
         q2 = np.concatenate([q, q[:, :, :1]], 2)
         t2 = fa.Tensor.from_numpy(device, q2, dtype)
         assert t2.selected_kernel(tk, tv, 0.1, analytic=(True, Skv - Sq - 1, 0)) != fa.KERNEL_DECODE_SPLITKV
