@@ -4,9 +4,10 @@
 // Keys/values are walked in tiles of 64 rows that go from global memory straight into a three-stage
 // LDS ring (direct-to-LDS buffer loads, no staging registers).  Per tile and wavefront:
 //   S^T (64 keys x 32 queries)  = K_tile . Q^T      v_mfma_f32_32x32x16  (A = K from LDS, B = Q in registers)
-//   Q is multiplied by scale * log2(e) once, and the first MFMA of a tile takes -m (the running row
-//   maximum) as its C operand, so the accumulators come out as base-2 exponents relative to the
-//   maximum and go straight into exp2: no multiply or subtract per score
+//   Q is multiplied by scale * log2(e) once (f16; for bf16 only by its power-of-two part, the rest multiplies
+//   the scores in f32), and the first MFMA of a tile takes -m (the running row maximum) as its C operand, so
+//   the accumulators come out as base-2 exponents relative to the maximum and go straight into exp2: no
+//   multiply or subtract per score in f16
 //   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of
 //   it per 32-key block, so the row max / row sum are in-lane folds plus one exchange with the
 //   lane 32 away (v_permlane32_swap); the running maximum is only moved (and O rescaled) when a
@@ -180,6 +181,15 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // base-2 exponents and the softmax needs no multiply per score
     // (the loads are issued here, the scaling waits until the first K/V tiles are on their way too)
     const float scale2 = p.scale * PF_LOG2E;
+    // f16: Q takes the whole factor scale2 (one rounding to 11 bits per element of Q: a score is off by about
+    // 2^-11.5 of the root sum of squares of its terms, 5e-4 of an exponent for unit-variance inputs; it grows in
+    // proportion to the scores).  bf16 would keep 8 bits only, so there scale2 = pw * rr with pw a power of two and rr
+    // in [1, 2): Q takes pw, which is exact, and rr multiplies every score in f32 right before exp2 (one more vector
+    // instruction per score, 4 % of an 8192 x 8192 call); the S^T accumulators, m and negm are then in units of 1 / rr.
+    constexpr bool EXACT_SCALE = std::is_same<T, bf16_t>::value;
+    const float pw = EXACT_SCALE ? __uint_as_float(__float_as_uint(scale2) & 0x7F800000u) : scale2;
+    const float rr = EXACT_SCALE ? scale2 / pw : 1.0f;
+    const float slack_u = PF_RESCALE_SLACK / rr;
     vec8 qreg[D / 16];
     {
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
@@ -436,10 +446,10 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
         mx = half_swap_max(mx);
         const bool first = (m == -INFINITY);  // no visible key so far (negm is 0 then)
-        const bool grow = first ? (mx > -INFINITY) : (mx > PF_RESCALE_SLACK);
+        const bool grow = first ? (mx > -INFINITY) : (mx > slack_u);
         if (__builtin_amdgcn_ballot_w64(grow) != 0) {
             const float delta = grow ? mx : 0.0f;
-            const float corr = first ? 0.0f : __builtin_amdgcn_exp2f(-delta);
+            const float corr = first ? 0.0f : __builtin_amdgcn_exp2f(-delta * rr);
             m = grow ? (first ? mx : m + mx) : m;
             l *= corr;
 #pragma unroll
@@ -458,11 +468,11 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[t][r]);
+                const float p0 = __builtin_amdgcn_exp2f(EXACT_SCALE ? s[t][r] * rr : s[t][r]);
 #ifdef FHIP_EXP_HALF_EXP
                 const float p1 = p0;
 #else
-                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
+                const float p1 = __builtin_amdgcn_exp2f(EXACT_SCALE ? s[t][r + 1] * rr : s[t][r + 1]);
 #endif
                 pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
                 l += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
@@ -560,7 +570,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             issue_tile(0);
         }
 #pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) qreg[kb] = Mma<T>::scaled(qreg[kb], scale2);
+        for (int kb = 0; kb < D / 16; kb++) qreg[kb] = Mma<T>::scaled(qreg[kb], pw);
         wait_tiles(integral_constant<int, 0>{});
         lds_barrier();
         if (group == 0) {
@@ -612,8 +622,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         if (group == 1) return;
         const float m1 = park[(D / 2) * 256], l1 = park[(D / 2 + 1) * 256];
         const float mn = fmaxf(m, m1);
-        const float c0 = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m - mn);
-        const float c1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m1 - mn);
+        const float c0 = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m - mn) * rr);
+        const float c1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - mn) * rr);
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
@@ -635,7 +645,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     char *const og = parked ? (char *)(p.partials + (int64_t)ksplit * p.pf_pitch) : (char *)p.out;
     if (parked && query < p.Sq && h2 == 0) {
         float *ws = (float *)og + b * os0 + h * os1 + (int64_t)query * os2;
-        ws[D] = m;
+        ws[D] = m * rr;  // base-2 exponent units
         ws[D + 1] = l_tot;
     }
     if (out_vec || parked) {

@@ -13,7 +13,7 @@ import pytest
 import floneum_amd as fa
 import oracle
 from floneum_amd import synth
-from conftest import TOL_16, TOL_F32, assert_parity
+from conftest import TOL_16, TOL_F32, assert_parity, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -689,3 +689,28 @@ def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype,
             ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
                                          rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
             assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
+
+
+@pytest.mark.parametrize("dtype,std,tol", [(fa.BF16, 8.0, dict(max_abs=None, rel_l2=8e-3)), (fa.BF16, 30.0, dict(max_abs=None, rel_l2=8e-3)),
+                                           (fa.F16, 3.0, dict(max_abs=None, rel_l2=1e-3)), (fa.F16, 8.0, dict(max_abs=None, rel_l2=3e-3))])
+@pytest.mark.parametrize("D,Sq,Skv", [(128, 300, 300), (64, 200, 1500), (96, 260, 260)])
+def test_tiled_16bit_prefill_at_large_score_magnitudes(device, dtype, std, tol, D, Sq, Skv):
+    """Inputs far wider than the unit-variance benchmark tensors: scaled scores of standard deviation std^2 (9 ... 900),
+    softmax rows close to one-hot.  bf16: the kernel multiplies the scores by the non-power-of-two part of
+    scale * log2(e) in f32 (Q takes only the power of two), so the error does not grow with the scores.  f16: Q takes
+    the whole factor, rounded to 11 bits; the error grows in proportion to the scores and stays inside the gate for
+    scores of standard deviation 9, about three times the gate at 64."""
+    B, H, Hkv = 1, 4, 2
+    rng = np.random.default_rng(77)
+    q = rng.normal(0, std, (B, H, Sq, D)).astype(np.float32)
+    k = rng.normal(0, std, (B, Hkv, Skv, D)).astype(np.float32)
+    v = rng.normal(0, std, (B, Hkv, Skv, D)).astype(np.float32)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    analytic = (True, Skv - Sq, 0)
+    assert tq.selected_kernel(tk, tv, D ** -0.5, analytic=analytic) == fa.KERNEL_PREFILL_MFMA
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out_dtype=fa.F32).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 _analytic_mask(Sq, Skv, True, Skv - Sq, 0), "qk")
+    assert np.isfinite(out).all()
+    rl = rel_l2(out, ref)
+    assert rl <= tol["rel_l2"], f"rel-L2 {rl:.2e} at std {std}, D{D}"
