@@ -1219,7 +1219,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         set_error("decode: batch * kv_heads * head_blocks = %ld exceeds the grid limit 65535", gy);
         return FHIP_ERR_UNSUPPORTED;
     }
-    dim3 grid((unsigned)p.nsplit, (unsigned)gy), block(64 * DEC_WAVES);
+    dim3 grid((unsigned)p.nsplit, (unsigned)gy);
     if constexpr (F32) {
         if (decode_use_mfma(p.D, true)) {
             if (gt == 32) launch_mfma_f32<2>(p, grid, stream);

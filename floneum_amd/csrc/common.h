@@ -153,6 +153,7 @@ struct RopeRows {
     const void *norm_w, *norm_b;  // [D] weight (nullptr: no norm) and optional bias, of norm_dtype
     int32_t norm_dtype;
     float eps;
+    int32_t vec;  // rows and pointers allow the 16-byte forms (set by fill_row_job)
 };
 struct RowJobs {
     RopeRows job[3];

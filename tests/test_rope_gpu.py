@@ -131,6 +131,27 @@ def test_norm_rope_bit_exact(device, dtype, interleaved, bias, D, start):
     assert np.array_equal(alone.view(np.uint8), ref_n.view(np.uint8))
 
 
+@pytest.mark.parametrize("in_dtype,out_dtype", [(fa.F32, fa.F32), (fa.F32, fa.F16), (fa.F16, fa.F16), (fa.BF16, fa.F32)])
+@pytest.mark.parametrize("D,interleaved", [(128, False), (256, False), (64, True), (128, True)])
+def test_prompt_sized_rope_and_norm_rope_bit_exact(device, in_dtype, out_dtype, D, interleaved):
+    """The rows of a prompt (thousands, in row blocks of the wide forms, the last block partial; the sum of squares of
+    head_dim 128 and 256 rows whose order matters) with the conversion to the cache's type on the way out."""
+    B, H, S, start = 1, 6, 333, 19
+    rc = fa.RopeCache(D, 512, 500000.0, device)
+    rng = np.random.default_rng(D + S)
+    x = (_x(5, (B, H, S, D)) * rng.choice([1.0, 30.0, 1e-3], (B, H, S, 1))).astype(np.float32)
+    w = rng.normal(1, 0.3, D).astype(np.float32)
+    t = fa.Tensor.from_numpy(device, x, in_dtype)
+    out = rc.apply(t, start, interleaved, out_dtype=out_dtype).to_numpy()
+    fn = oracle.rope_interleaved if interleaved else oracle.rope
+    ref = _cast_out(fn(rounded(x, in_dtype), rc.cos_host, rc.sin_host, start), out_dtype)
+    assert np.array_equal(out.view(np.uint8), ref.view(np.uint8)), "rope"
+    norm = fa.RmsNorm(w, None, 1e-6, in_dtype, device)
+    out = rc.apply(t, start, interleaved, out_dtype=out_dtype, norm=norm).to_numpy()
+    ref = _norm_then_rope(x, in_dtype, w, None, 1e-6, rc, start, interleaved, out_dtype)
+    assert np.array_equal(out.view(np.uint8), ref.view(np.uint8)), "norm + rope"
+
+
 def test_norm_sum_order_and_reference_test_rows(device):
     """The device sum is the reference's left-to-right fold (a row where any other order differs), and the
     rows of the reference's own tests (rms_norm.rs:163-186) come out as expected."""
