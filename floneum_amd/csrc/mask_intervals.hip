@@ -138,18 +138,54 @@ __global__ __launch_bounds__(256) void mask_build_kernel(W *out, uint32_t rows, 
     }
 }
 
+// the same, 16 bytes per lane and step (V = 4 f32 or 8 16-bit elements of one row; cols % V == 0, out 16-byte aligned)
+template <typename W, int V>
+__global__ __launch_bounds__(256) void mask_build_wide_kernel(W *out, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
+                                                              uint64_t window, W ninf) {
+    const uint64_t per_row = cols / V, total = (uint64_t)rows * per_row;
+    for (uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256) {
+        const uint64_t i = idx / per_row, c0 = (idx % per_row) * V;
+        W vals[V];
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+            const uint64_t c = c0 + e;
+            bool masked = false;
+            if (c >= off) {
+                const uint64_t j = c - off;
+                masked = has_window ? (i < j || j + window <= i) : (j > i);
+            }
+            vals[e] = masked ? ninf : (W)0;
+        }
+        uint4_t raw;
+        __builtin_memcpy(&raw, vals, 16);
+        *(uint4_t *)(out + i * cols + c0) = raw;
+    }
+}
+
 int launch_mask_build(void *out, fhip_dtype dtype, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
                       uint64_t window, hipStream_t stream) {
     const uint64_t total = (uint64_t)rows * cols;
     if (total == 0) return FHIP_OK;
-    const uint64_t blocks = (total + 255) / 256;
+    const int V = dtype == FHIP_F32 ? 4 : 8;
+    const bool wide = cols % V == 0 && ((uintptr_t)out % 16) == 0;
+    const uint64_t blocks = ((wide ? total / V : total) + 255) / 256;
     const dim3 grid((unsigned)(blocks < 65536 * 4 ? blocks : 65536 * 4)), block(256);
-    if (dtype == FHIP_F32)
-        hipLaunchKernelGGL(mask_build_kernel<uint32_t>, grid, block, 0, stream, (uint32_t *)out, rows, cols, off, has_window,
-                           window, 0xFF800000u);
-    else
-        hipLaunchKernelGGL(mask_build_kernel<uint16_t>, grid, block, 0, stream, (uint16_t *)out, rows, cols, off, has_window,
-                           window, (uint16_t)(dtype == FHIP_F16 ? 0xFC00u : 0xFF80u));
+    if (dtype == FHIP_F32) {
+        if (wide)
+            hipLaunchKernelGGL((mask_build_wide_kernel<uint32_t, 4>), grid, block, 0, stream, (uint32_t *)out, rows, cols, off,
+                               has_window, window, 0xFF800000u);
+        else
+            hipLaunchKernelGGL(mask_build_kernel<uint32_t>, grid, block, 0, stream, (uint32_t *)out, rows, cols, off, has_window,
+                               window, 0xFF800000u);
+    } else {
+        const uint16_t ninf = (uint16_t)(dtype == FHIP_F16 ? 0xFC00u : 0xFF80u);
+        if (wide)
+            hipLaunchKernelGGL((mask_build_wide_kernel<uint16_t, 8>), grid, block, 0, stream, (uint16_t *)out, rows, cols, off,
+                               has_window, window, ninf);
+        else
+            hipLaunchKernelGGL(mask_build_kernel<uint16_t>, grid, block, 0, stream, (uint16_t *)out, rows, cols, off, has_window,
+                               window, ninf);
+    }
     FHIP_HIP_CHECK(hipGetLastError());
     return FHIP_OK;
 }
