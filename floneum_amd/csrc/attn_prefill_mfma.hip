@@ -149,21 +149,27 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 
     // workgroup -> (query block, batch, head): long query blocks first, and heads laid out so
     // the workgroups that land on one XCD (id % 8) share a KV head whenever H is a multiple of 8
-    const int bh_count = p.B * p.H;
+    // Packed form (key-split form only, at most 32 query rows, GQA group a multiple of 4): the workgroup's four row
+    // blocks are rows 0..31 of four query heads that share a KV head, so the K and V tiles it moves serve all four
+    // and a few new rows on a long cache read the cache once per KV head, not once per query head.
+    const int pack = KS ? p.pf_pack : 0;
+    const int heads = pack ? p.H / 4 : p.H;  // head units per batch entry
+    const int bh_count = p.B * heads;
     const int nks = max(p.pf_nsplit, 1);
     const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
     const int id = blockIdx.x / nks;
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
-    const int b = rem / p.H;
-    int h = rem % p.H;
-    if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
+    const int b = rem / heads;
+    int h = rem % heads;
+    if (pack) h = 4 * h + (wave & 3);
+    else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
 
-    const int q0 = qb * BM;
-    const int qw0 = q0 + 32 * (KS ? (wave & 3) : wave);  // KS: both groups own the same 128 rows
+    const int q0 = pack ? 0 : qb * BM;
+    const int qw0 = pack ? 0 : q0 + 32 * (KS ? (wave & 3) : wave);  // KS: both groups own the same 128 rows
     const int query = qw0 + ln;
-    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, pack ? 32 : BM, qw0, lane);
     if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -719,11 +725,13 @@ static bool use_key_split_form(const AttnParams &p) {
 }
 
 template <typename T>
-static int launch_t(const AttnParams &p, hipStream_t stream) {
+static int launch_t(const AttnParams &p0, hipStream_t stream) {
+    AttnParams p = p0;
     const bool ks = use_key_split_form(p);
+    p.pf_pack = ks ? prefill_mfma_pack(p.B, p.H, p.G, p.Sq, p.Skv, p.cus > 0 ? p.cus : 256) : 0;
     const int bm = ks ? PF_BM / 2 : PF_BM;
-    const int nqb = (p.Sq + bm - 1) / bm;
-    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
+    const int nqb = p.pf_pack ? 1 : (p.Sq + bm - 1) / bm;
+    const long blocks = (long)nqb * p.B * (p.pf_pack ? p.H / 4 : p.H) * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -751,11 +759,20 @@ static int launch_t(const AttnParams &p, hipStream_t stream) {
 
 // Few query rows on a long cache: 256-row query blocks alone leave most CUs idle, so the keys are split over
 // workgroups too, down to 1024 keys per share, until there are about two workgroups per CU.
-void prefill_mfma_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+// Query heads per workgroup of the packed form (0: not packed).  Packing divides the workgroups by four, and a share of
+// the keys is at least 1024 keys long, so it is taken only when the packed grid can still fill the chip (batch 8 on 8192
+// keys: 98 -> 66..81 us for 12..32 rows; at batch 1 the unpacked grid's 256 workgroups are quicker than 64 packed ones).
+int prefill_mfma_pack(int B, int H, int G, int Sq, int Skv, int compute_units) {
+    if (!(Sq <= 32 && G >= 4 && G % 4 == 0) || Skv <= 2 * PF_BN) return 0;
+    const long shares = Skv / 1024 > 1 ? Skv / 1024 : 1;
+    return (long)B * (H / 4) * shares >= compute_units ? 4 : 0;
+}
+
+void prefill_mfma_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
     *nsplit = 1;
     *chunk = Skv;
     if (causal_square) return;
-    const long wgs = (long)B * H * ((Sq + PF_BM - 1) / PF_BM);
+    const long wgs = (long)B * (prefill_mfma_pack(B, H, G, Sq, Skv, compute_units) ? H / 4 : H) * ((Sq + PF_BM - 1) / PF_BM);
     if (2 * wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy: parking and
                                           // merging partial results would cost more than it gains (measured)
     const long want = (2L * compute_units + wgs - 1) / wgs;

@@ -173,6 +173,48 @@ def test_longer_drafts_while_rows_times_group_fit_one_workgroup(device, dtype, G
         assert t2.selected_kernel(tk, tv, 0.1, analytic=(True, Skv - Sq - 1, 0)) != fa.KERNEL_DECODE_SPLITKV
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("G,Sq,D,case", [(4, 12, 128, "causal"), (4, 32, 128, "window"), (8, 17, 64, "mask_tensor"),
+                                         (4, 9, 96, "ragged"), (4, 24, 128, "full")])
+def test_rows_beyond_the_decode_kernel_share_the_kv_tiles_of_a_gqa_group(device, dtype, G, Sq, D, case):
+    """9..32 new rows on a long cache in 16-bit: the tiled prefill kernel in its packed form, where a workgroup's four
+    32-row blocks are four query heads of one KV head (the cache is read once per KV head); taken when the packed
+    grid still fills the chip, which this batch does."""
+    B, Hkv, Skv = 16, 4, 4100
+    H = Hkv * G
+    assert B * (H // 4) * (Skv // 1024) >= device.compute_units, "the packed form would not be chosen"
+    q, k, v = _normal_qkv(48, B, H, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    off = Skv - Sq
+    kw, m, mask, kind = {}, None, None, None
+    if case in ("causal", "window", "mask_tensor"):
+        w = 0 if case == "causal" else 1500
+        mask, kind = _analytic_mask(Sq, Skv, True, off, w), "qk"
+        if case == "mask_tensor":
+            m = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+        else:
+            kw["analytic"] = (True, off, w)
+    out_buf = fa.Tensor.empty(device, (B, Sq, H, D), dtype)      # written as [B, Sq, H, D]
+    lens = None
+    if case == "ragged":
+        lens = np.array([Skv - 3 * i * 67 for i in range(B)], np.int32)
+        lens[3] = 40
+        kw["kv_lens"] = fa.IntTensor(device, lens)
+    if m is None:  # (the selection of a call with a mask tensor depends on the workspace the call brings)
+        assert tq.selected_kernel(tk, tv, 0.1, **kw) == fa.KERNEL_PREFILL_MFMA
+    tq.flash_attention(tk, tv, D ** -0.5, m, out=out_buf.transpose(1, 2), **kw)
+    got = out_buf.to_numpy().transpose(0, 2, 1, 3)
+    if lens is None:
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, kind)
+        assert_parity(got, ref, _tol(dtype), f"{case} G{G} Sq{Sq} D{D}")
+    else:
+        for b in range(B):
+            n = int(lens[b])
+            ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                         rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+            assert_parity(got[b:b + 1], ref, _tol(dtype), f"ragged b{b} len{n}")
+
+
 def test_five_rows_at_a_head_dim_of_the_vector_variant_is_a_prefill_call(device):
     q, k, v = _normal_qkv(46, 1, 2, 2, 5, 300, 80)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F32) for a in (q, k, v))
