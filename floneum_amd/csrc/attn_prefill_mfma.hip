@@ -760,12 +760,13 @@ static int launch_t(const AttnParams &p0, hipStream_t stream) {
 // Few query rows on a long cache: 256-row query blocks alone leave most CUs idle, so the keys are split over
 // workgroups too, down to 1024 keys per share, until there are about two workgroups per CU.
 // Query heads per workgroup of the packed form (0: not packed).  Packing divides the workgroups by four, and a share of
-// the keys is at least 1024 keys long, so it is taken only when the packed grid can still fill the chip (batch 8 on 8192
-// keys: 98 -> 66..81 us for 12..32 rows; at batch 1 the unpacked grid's 256 workgroups are quicker than 64 packed ones).
+// the keys is at least 1024 keys long, so it is taken when the packed grid still reaches half the CUs (12..32 rows:
+// batch 8 on 8192 keys 98 -> 66..81 us, batch 4 on 4096 keys 45 -> 28 us, batch 1 on 32768 keys 68 -> 40 us; with a
+// quarter of the CUs, batch 1 on 8192 keys, the unpacked grid is as quick: 25.7 against 26.5 us).
 int prefill_mfma_pack(int B, int H, int G, int Sq, int Skv, int compute_units) {
     if (!(Sq <= 32 && G >= 4 && G % 4 == 0) || Skv <= 2 * PF_BN) return 0;
     const long shares = Skv / 1024 > 1 ? Skv / 1024 : 1;
-    return (long)B * (H / 4) * shares >= compute_units ? 4 : 0;
+    return 2 * (long)B * (H / 4) * shares >= compute_units ? 4 : 0;
 }
 
 void prefill_mfma_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {

@@ -240,7 +240,7 @@ def test_prefill_key_split_planning_on_256_cus():
 
     assert shares(128, 8192, fa.F32, 130) == 4    # a new chat turn: 4 query blocks x 32 heads x 4 shares of 2048 keys
     assert shares(128, 8192, fa.F16, 132) == 8    # one 128-row block per head x 8 shares of 1024 keys
-    assert shares(32, 32768, fa.F16, 132) == 16
+    assert shares(32, 32768, fa.F16, 132) == 32   # packed: 8 head quads x 32 shares of 1024 keys (unpacked it was 32 heads x 16)
     assert shares(512, 512, fa.F32, 130) == 0     # square causal prompts are left alone
     assert shares(2048, 2048, fa.F16, 132) == 0
 
