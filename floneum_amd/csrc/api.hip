@@ -261,6 +261,22 @@ static bool f32_adds_masks(const fhip_attn_args *a) { return a->q.shape[3] <= 12
 // is queued behind it.
 static bool f32_serves_both_mask_forms(const fhip_attn_args *a) { return a->q.shape[3] <= 64; }
 
+// The keys a decode call can see at all, when the analytic descriptor alone says so (no mask tensor, no per-sequence key
+// counts): [*lo0, *lo0 + *len) with *lo0 a multiple of 128.  The kernels are handed the tensors from key *lo0 on (and the
+// query position moved by as much), so the split-KV plan covers this range only: a window of 4096 keys at the end of a
+// 16384-key cache is spread over as many workgroups as a 4096-key cache would be.
+static void decode_visible_range(const fhip_attn_args *a, int *lo0, int *len) {
+    const int64_t Skv = a->k.shape[2], rows = a->q.shape[2];
+    int64_t lo = 0, hi = Skv;
+    if (a->analytic.enabled && !a->kv_lens && a->mask_kind == FHIP_MASK_NONE) {
+        if (a->analytic.causal) hi = std::min<int64_t>(hi, a->analytic.q_pos_offset + rows);
+        if (a->analytic.window > 0) lo = std::max<int64_t>(0, a->analytic.q_pos_offset - a->analytic.window + 1);
+    }
+    if (hi <= lo) lo = 0, hi = Skv;  // nothing visible: the rows come out NaN however the keys are split
+    *lo0 = (int)(lo / 128 * 128);
+    *len = (int)(hi - *lo0);
+}
+
 // Key split of a call the f32-arithmetic tiled kernel serves (few query rows on a long cache), and where its
 // partial results go in the workspace: behind the mask scratch, 256-byte aligned.
 static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
@@ -707,7 +723,10 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
         int chunk, nsplit, waves;
         const int B = (int)args->q.shape[0], H = (int)args->q.shape[1], D = (int)args->q.shape[3];
         const int Hkv = (int)args->k.shape[1], Skv = (int)args->k.shape[2], rows = (int)args->q.shape[2];
-        decode_plan(B, Hkv, H / Hkv * rows, Skv, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr,
+        int lo0, len;
+        decode_visible_range(args, &lo0, &len);
+        (void)Skv;
+        decode_plan(B, Hkv, H / Hkv * rows, len, D, compute_units > 0 ? compute_units : 256, args->kv_lens != nullptr,
                     args->dtype == FHIP_F32, &chunk, &nsplit, &waves);
         *bytes = decode_workspace_bytes(B, H * rows, Hkv, D, nsplit);
     }
@@ -811,6 +830,15 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
+            int lo0, vis_len;
+            decode_visible_range(args, &lo0, &vis_len);
+            if (lo0 > 0 || vis_len < p.Skv) {  // the kernels see keys lo0 .. lo0 + vis_len as keys 0 .. vis_len
+                const int64_t eb = elem_bytes(args->dtype);
+                p.k = (const char *)p.k + lo0 * p.ks[2] * eb;
+                p.v = (const char *)p.v + lo0 * p.vs[2] * eb;
+                p.Skv = vis_len;
+                p.q_pos_offset -= lo0;
+            }
             decode_plan(p.B, p.Hkv, p.G * p.Sq, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr,
                         args->dtype == FHIP_F32, &p.chunk, &p.nsplit, &p.dec_waves);
             const size_t need = decode_workspace_bytes(p.B, p.H * p.Sq, p.Hkv, p.D, p.nsplit);

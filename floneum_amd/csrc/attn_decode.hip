@@ -51,15 +51,25 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     const int hb = (G + gt - 1) / gt;
     const long units = (long)B * Hkv * hb;
     *waves = DEC_WAVES;
-    // the 8-wavefront form of the 16-bit matrix-core variant, chunks of 2048 keys: when every CU gets a whole unit, or,
-    // with more than 8 columns per unit (a multi-token step: twice the matrix and softmax work per key), a chunk
-    const long chunks2048 = (Skv + 2047) / 2048;
-    if (decode_use_mfma(D, f32) && !f32 && D <= 128 && Skv > 2048 &&
-        (units >= compute_units || (G > 8 && units * chunks2048 >= compute_units))) {
-        *waves = 8;
-        *chunk = 2048;
-        *nsplit = (Skv + 2047) / 2048;
-        return;
+    // The 8-wavefront form of the 16-bit matrix-core variant (one workgroup per CU).  With a whole (batch, KV head) unit
+    // or more per CU: chunks of 2048 keys.  With more than 8 columns per unit (a multi-token step: twice the matrix and
+    // softmax work per key) also below that, when an even share of the keys per CU is at least 2048 keys long: then
+    // every CU gets one workgroup and all are equally long.
+    if (decode_use_mfma(D, f32) && !f32 && D <= 128 && Skv > 2048) {
+        if (units >= compute_units) {
+            *waves = 8;
+            *chunk = 2048;
+            *nsplit = (Skv + 2047) / 2048;
+            return;
+        }
+        const long ns = compute_units / units;  // >= 1
+        const long c = ((Skv + ns - 1) / ns + 127) / 128 * 128;
+        if (G > 8 && c >= 2048) {
+            *waves = 8;
+            *chunk = (int)c;
+            *nsplit = (int)((Skv + c - 1) / c);
+            return;
+        }
     }
     // the MFMA variant holds two workgroups per CU (LDS; one above head_dim 128), the vector variant four or more; f32 rows carry
     // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at

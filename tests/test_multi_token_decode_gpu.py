@@ -122,6 +122,23 @@ def test_multi_token_step_ragged_batch_and_padding_mask(device, dtype):
     del out
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.F32, fa.BF16])
+@pytest.mark.parametrize("Sq,off,window,D", [(1, 1000, 300, 128), (3, 1000, 300, 128), (4, 2995, 0, 64), (2, 140, 0, 128),
+                                             (1, 2999, 129, 96), (8, 1500, 1400, 128), (1, 5, 3, 80)])
+def test_decode_sees_only_a_stretch_of_the_cache(device, dtype, Sq, off, window, D):
+    """The analytic descriptor leaves the start of the cache (a window) and / or its end (query positions in the middle
+    of the cache) out: the split-KV plan and the kernels work on the visible stretch alone."""
+    B, H, Hkv, Skv = 2, 8, 2, 3000
+    q, k, v = _normal_qkv(49, B, H, Hkv, Sq, Skv, D, 0.5)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    analytic = (True, off, window)
+    assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic) == fa.KERNEL_DECODE_SPLITKV
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 _analytic_mask(Sq, Skv, True, off, window), "qk")
+    assert_parity(out, ref, _tol(dtype), f"Sq{Sq} off{off} window{window} D{D}")
+
+
 def test_rows_fully_masked_by_their_own_limits_are_nan(device):
     """A window so short and an offset so placed that some rows see no key: those rows are NaN (0/0) as in the
     reference, the others are right."""
