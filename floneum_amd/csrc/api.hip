@@ -217,11 +217,14 @@ static bool decode_eligible(const fhip_attn_args *a) {
 static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     if (a->dtype == FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
-    if (!(D == 64 || D == 96 || D == 128)) return false;
+    const bool wide = D == 160 || D == 192 || D == 224 || D == 256;  // attn_prefill_mfma_wide.hip
+    if (!(D == 64 || D == 96 || D == 128 || wide)) return false;
+    if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
+    // scales in f32; 64-bit tile addresses, 32-bit byte offsets inside a 32-key tile
+    if (wide) return a->k.stride[2] >= 0 && a->v.stride[2] >= 0 && a->k.stride[2] < (1 << 25) && a->v.stride[2] < (1 << 25);
     // the kernel folds scale * log2(e) into Q (rounded back to the input type): the factor must not
     // be able to push a finite element out of range
     if (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f)) return false;
-    if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
     // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv
     // head) slice must span less than 2 GiB
     const uint64_t Skv = a->k.shape[2];
@@ -288,8 +291,12 @@ static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratc
 static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
     const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
     const int Hkv = (int)a->k.shape[1];
-    prefill_mfma_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
-                      (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
+    if (a->q.shape[3] > 128)  // the wide-head form: 128-row query blocks
+        prefill_mfma_wide_plan((int)a->q.shape[0], (int)a->q.shape[1], (int)a->q.shape[2], (int)a->k.shape[2], causal_square,
+                               cus > 0 ? cus : 256, nsplit, chunk);
+    else
+        prefill_mfma_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
+                          (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
 }
 
 // assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
@@ -733,6 +740,11 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     return FHIP_OK;
 }
 
+// the 16-bit tiled prefill kernels: 64 / 96 / 128, and the wide-head form above
+static int launch_mfma_by_head_dim(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
+    return p.D > 128 ? launch_prefill_mfma_wide(p, dtype, stream) : launch_prefill_mfma(p, dtype, stream);
+}
+
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     if (!s) {
         set_error("stream is NULL");
@@ -814,7 +826,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         pt.iv_bad = bad;
         const bool both_forms = id == FHIP_KERNEL_PREFILL_F32 && f32_serves_both_mask_forms(args);
         pt.iv_either = both_forms ? 1 : 0;
-        rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_prefill_mfma(pt, args->dtype, s->s) : launch_prefill_f32(pt, args->dtype, s->s);
+        rc = id == FHIP_KERNEL_PREFILL_MFMA ? launch_mfma_by_head_dim(pt, args->dtype, s->s) : launch_prefill_f32(pt, args->dtype, s->s);
         if (rc) return rc;
         FHIP_MARK_MAIN_DONE(p, s->s);
         if (both_forms) return FHIP_OK;
@@ -827,7 +839,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     }
     switch (id) {
         case FHIP_KERNEL_GENERIC: rc = launch_generic(p, args->dtype, s->s); break;
-        case FHIP_KERNEL_PREFILL_MFMA: rc = launch_prefill_mfma(p, args->dtype, s->s); break;
+        case FHIP_KERNEL_PREFILL_MFMA: rc = launch_mfma_by_head_dim(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
             int lo0, vis_len;

@@ -1,0 +1,424 @@
+// Prefill attention for f16 / bf16 at head dims 160, 192, 224 and 256 (Gemma-3's key length is 256) on the gfx950
+// matrix cores.
+//
+// The 256-row kernel of attn_prefill_mfma.hip keeps Q and O^T of 32 rows in a wavefront's registers with two wavefronts
+// per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is four wavefronts,
+// one per SIMD with the whole register file, and 128 query rows of one (batch, head); the keys are walked in tiles of 32
+// that all four wavefronts share through a double-buffered LDS tile (global -> registers -> LDS, the next tile's loads
+// in flight during the math).  Per tile and wavefront, on v_mfma_f32_16x16x32 with the 32 query rows as two blocks of
+// 16 columns (the arithmetic of the split-KV decode kernel with two column blocks, attn_decode.hip):
+//   S^T[key][row]  = K . Q^T     A = K from LDS (one 16-byte read feeds both column blocks), B = Q in registers
+//   scores scaled in f32 (scale * log2 e), masked by the row's visible interval, online softmax per column
+//   O^T[dim][row] += V^T . P^T   A = V^T from row-major LDS with ds_read_b64_tr_b16, B = the probabilities
+// Masks: the analytic descriptor, key counts, or the interval form of a mask tensor (attn_bounds.h); a mask tensor that
+// is not made of intervals is served by the kernel queued behind this one, as for the other tiled kernels.
+//
+// Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199 with the f32 accumulation of 16-bit
+// inputs of fusor-ml/core/src/composite/flash_attention.rs:186-203,323-327.
+#include <type_traits>
+
+#include "attn_bounds.h"
+#include "common.h"
+#include "device_utils.h"
+
+namespace fhip {
+
+namespace {
+
+constexpr float PW_LOG2E = 1.4426950408889634f;
+constexpr int PW_WAVES = 4;
+constexpr int PW_BM = 32 * PW_WAVES;  // query rows per workgroup
+constexpr int PW_KEYS = 32;           // keys per tile
+constexpr float PW_RESCALE_SLACK = 8.0f;
+
+#define PWLDS_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
+
+typedef uint32_t uint2w_t __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct WideMma;
+template <>
+struct WideMma<half_t> {
+    typedef half8_t vec8;
+    static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float x, float y) {
+        half2_t h = {(half_t)x, (half_t)y};
+        return __builtin_bit_cast(uint32_t, h);
+    }
+};
+template <>
+struct WideMma<bf16_t> {
+    typedef bf16x8_t vec8;
+    static __device__ __forceinline__ float4_t mfma(vec8 a, vec8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float x, float y) {
+        typedef __bf16 bf16x2w_t __attribute__((ext_vector_type(2)));
+        const bf16x2w_t h = {(__bf16)x, (__bf16)y};  // v_cvt_pk_bf16_f32: round to nearest even
+        return __builtin_bit_cast(uint32_t, h);
+    }
+};
+
+// max / sum over the four lanes l, l^16, l^32, l^48 (same column, the four key groups)
+__device__ __forceinline__ float pw_quad_max(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float pw_quad_sum(float x) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
+    typedef typename WideMma<T>::vec8 vec8;
+    constexpr int KP = D * 2 + 16;           // K tile row pitch (bytes): rows 4 banks apart
+    constexpr int VP = D * 2 + 32;           // V tile row pitch (bytes): rows 8 banks apart
+    constexpr int K_BYTES = PW_KEYS * KP;
+    constexpr int V_BYTES = PW_KEYS * VP;
+    constexpr int STAGE = K_BYTES + V_BYTES;
+    constexpr int CPR = D / 8;               // 16-byte chunks per row
+    constexpr int CHUNKS = PW_KEYS * CPR;    // per tensor and tile
+    constexpr int NLD = 2 * CHUNKS / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
+    constexpr int KB = D / 32;               // contraction blocks of K . Q^T
+    constexpr int NB = D / 16;               // 16-dim blocks of the output
+    constexpr int CB = 2;                    // 16-column blocks: the wavefront's 32 query rows
+    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    auto lds_base = (__attribute__((address_space(3))) char *)smem;
+
+    if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the kernel behind takes the call
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int j = lane & 15;   // column inside a block
+    const int q4 = lane >> 4;  // key group
+
+    // workgroup -> (share of the keys, query block, batch, head): long (late) query blocks first
+    const int bh_count = p.B * p.H;
+    const int nks = max(p.pf_nsplit, 1);
+    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
+    const int id = blockIdx.x / nks;
+    const int qb = nqb - 1 - id / bh_count;
+    const int rem = id % bh_count;
+    const int b = rem / p.H;
+    int h = rem % p.H;
+    // consecutive workgroups land on consecutive XCDs (id % 8), each with an L2 of its own: with H a multiple of 8 the
+    // heads are dealt so that an XCD works on H / 8 neighbouring heads, i.e. on as few KV heads as possible
+    if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
+    const int g = h / p.G;
+    const int q0 = qb * PW_BM, qw0 = q0 + 32 * wave;
+
+    // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this
+    // lane's two rows (element test).  row_bounds gives lane l the interval of row qw0 + l % 32.
+    RowBounds rb = row_bounds(p, b, q0, PW_BM, qw0, lane);
+    if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
+        const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
+        rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
+        rb.lo_w = max(rb.lo_w, c_lo), rb.hi_w = min(rb.hi_w, c_hi);
+        rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
+        rb.klo = max(rb.klo, c_lo), rb.khi = min(rb.khi, c_hi);
+    }
+    int klo[CB], khi[CB], row[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        klo[cb] = __shfl(rb.klo, 16 * cb + j, 64);
+        khi[cb] = __shfl(rb.khi, 16 * cb + j, 64);
+        row[cb] = qw0 + 16 * cb + j;
+    }
+    // the same in every lane: kept in scalar registers, so that the branches on them are plain jumps
+    const int lo_wg = __builtin_amdgcn_readfirstlane(rb.lo_wg), hi_wg = __builtin_amdgcn_readfirstlane(rb.hi_wg);
+    // the keys every row of the wavefront sees
+    const int full_lo_w = __builtin_amdgcn_readfirstlane(rb.full_lo_w), full_hi_w = __builtin_amdgcn_readfirstlane(rb.full_hi_w);
+
+    const uint16_t *kbase = (const uint16_t *)p.k + b * p.ks[0] + g * p.ks[1];
+    const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
+    const float scale2 = p.scale * PW_LOG2E;
+
+    // tile movement: every thread takes NLD 16-byte chunks of K and of V; rows beyond the key axis repeat the last row
+    // (their scores are masked by the rows' intervals, which end at the key count)
+    // The K and the V tile are one list of 2 * CHUNKS 16-byte pieces, dealt to the 256 threads NLD at a time (an exact
+    // division for every head dim served; with 160 and 224 one of a thread's pieces is of K in half the threads and
+    // of V in the others).  A piece sits at a fixed byte offset from its tile's first key (the host admits row strides
+    // below 2^25 elements only, so it fits 32 bits); the tiles' own addresses are the same in every lane.
+    static_assert(NLD * 64 * PW_WAVES == 2 * CHUNKS, "pieces per thread");
+    uint4_t st[NLD];  // the tile in flight from HBM
+    // With 32 pieces per row (head dim 256) a thread's pieces are the same column of every eighth row: two offsets
+    // and constant steps describe them all, which the full register file of this head dim needs.
+    constexpr bool AFFINE = (64 * PW_WAVES) % CPR == 0;
+    constexpr int RSTEP = 64 * PW_WAVES / CPR;  // AFFINE: rows between a thread's consecutive pieces
+    uint32_t goff_[AFFINE ? 2 : NLD], loff_[AFFINE ? 2 : NLD];
+    if constexpr (AFFINE) {
+        const int r = tid / CPR, c = tid % CPR;
+        goff_[0] = (r * (uint32_t)p.ks[2] + c * 8) * 2;
+        goff_[1] = (r * (uint32_t)p.vs[2] + c * 8) * 2;
+        loff_[0] = r * KP + c * 16;
+        loff_[1] = K_BYTES + r * VP + c * 16;
+    } else {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = tid + 64 * PW_WAVES * u;
+            const bool is_v = cid >= CHUNKS;
+            const int r = (is_v ? cid - CHUNKS : cid) / CPR, c = (is_v ? cid - CHUNKS : cid) % CPR;
+            goff_[u] = (r * (uint32_t)(is_v ? p.vs[2] : p.ks[2]) + c * 8) * 2;
+            loff_[u] = is_v ? K_BYTES + r * VP + c * 16 : r * KP + c * 16;
+        }
+    }
+    const uint32_t kstep = RSTEP * (uint32_t)p.ks[2] * 2, vstep = RSTEP * (uint32_t)p.vs[2] * 2;
+    auto goff = [&](int u) __attribute__((always_inline)) -> uint32_t {
+        if constexpr (AFFINE) return u < NLD / 2 ? goff_[0] + u * kstep : goff_[1] + (u - NLD / 2) * vstep;
+        else return goff_[u];
+    };
+    auto loff = [&](int u) __attribute__((always_inline)) -> uint32_t {
+        if constexpr (AFFINE)
+            return u < NLD / 2 ? loff_[0] + u * RSTEP * KP : loff_[1] + (u - NLD / 2) * RSTEP * VP;
+        else return loff_[u];
+    };
+    auto load_tile = [&](int j0) __attribute__((always_inline)) {
+        const char *kt = (const char *)(kbase + (int64_t)j0 * p.ks[2]);
+        const char *vt = (const char *)(vbase + (int64_t)j0 * p.vs[2]);
+        if (j0 + PW_KEYS <= p.Skv) {
+#pragma unroll
+            for (int u = 0; u < NLD; u++) {
+                const bool is_v = tid + 64 * PW_WAVES * u >= CHUNKS;  // known at compile time except for the mixed piece
+                st[u] = *(const uint4_t *)((is_v ? vt : kt) + goff(u));
+            }
+            return;
+        }
+        // the last tile of a cache whose length is no multiple of the tile: rows past the end repeat the last key
+        const int last = p.Skv - 1 - j0;
+#pragma unroll
+        for (int u = 0; u < NLD; u++) {
+            const int cid = tid + 64 * PW_WAVES * u;
+            const bool is_v = cid >= CHUNKS;
+            const int r = (is_v ? cid - CHUNKS : cid) / CPR, c = (is_v ? cid - CHUNKS : cid) % CPR;
+            const int64_t row_stride = is_v ? p.vs[2] : p.ks[2];
+            st[u] = *(const uint4_t *)((is_v ? vt : kt) + (min(r, last) * row_stride + c * 8) * 2);
+        }
+    };
+    auto store_tile = [&](int stage_base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NLD; u++) *PWLDS_PTR(uint4_t, stage_base + loff(u)) = st[u];
+    };
+
+    const int j_begin = (lo_wg / PW_KEYS) * PW_KEYS;
+    const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PW_KEYS - 1) / PW_KEYS : 0;
+    if (ntiles > 0) load_tile(j_begin);  // issued first so the Q fetch below overlaps it
+
+    // Q^T operand: column j of block cb, dims 32 kb + 8 q4 .. +8 (rows beyond Sq repeat the last row; never stored)
+    vec8 qreg[CB][KB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)min(row[cb], p.Sq - 1) * p.qs[2];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+            qreg[cb][kb] = __builtin_bit_cast(vec8, *(const uint4_t *)(qp + 32 * kb + 8 * q4));
+    }
+
+    float4_t o[CB][NB];
+    float m[CB], l[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) o[cb][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+        m[cb] = -INFINITY, l[cb] = 0.0f;
+    }
+
+    // A tile in three parts.  tile_front brings tile t into LDS and computes the wavefront's masked scores (log2 units)
+    // and their per-column maxima; move_reference raises the reference maximum of the columns that need it and
+    // rescales O and l; tile_back turns the scores into probabilities and adds P . V.  The reference maximum of a
+    // column moves only when a tile exceeds it by more than 2^8 (probabilities then reach 2^8 at most, well inside
+    // f16 / bf16 range), which after the first tile almost never happens: the loop below runs front + back and leaves
+    // for move_reference only then, so that in the loop nothing but the matrix instructions touches O.
+    float sv[CB][8], mx[CB];
+    int sbase = 0;
+    // (A tile none of the wavefront's rows sees is not skipped: its scores are -inf, its probabilities 0.  A jump
+    // around the P . V block makes the compiler carry two copies of O and move one into the other on every tile,
+    // which costs more than the few such tiles on the diagonal of a causal mask.)
+    auto tile_front = [&](int t) __attribute__((always_inline)) -> bool {  // true: move the reference first
+        const int j0 = j_begin + t * PW_KEYS;
+        sbase = (t & 1) * STAGE;
+        store_tile(sbase);
+        __syncthreads();  // tile t is in LDS; every wavefront is done with tile t - 1, whose stage the next store takes
+        if (t + 1 < ntiles) load_tile(j0 + PW_KEYS);
+        const bool all_visible = j0 >= full_lo_w && j0 + PW_KEYS <= full_hi_w;  // no element test needed
+
+        // S^T[key][col] = K . Q^T : two 16-key halves, every K operand read serves both column blocks
+        float4_t s[CB][2];
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) s[cb][hf] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) {
+                const uint4_t raw = *PWLDS_PTR(uint4_t, sbase + (16 * hf + j) * KP + (32 * kb + 8 * q4) * 2);
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++)
+                    s[cb][hf] = WideMma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[cb][kb], s[cb][hf]);
+            }
+        }
+        bool grow = false;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            // element (hf, r) is key j0 + 16 hf + 4 q4 + r for column j of block cb
+            if (all_visible) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) sv[cb][e] = s[cb][e >> 2][e & 3] * scale2;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int key = j0 + 16 * (e >> 2) + 4 * q4 + (e & 3);
+                    sv[cb][e] = (key >= klo[cb] && key < khi[cb]) ? s[cb][e >> 2][e & 3] * scale2 : -INFINITY;
+                }
+            }
+            float x = sv[cb][0];
+#pragma unroll
+            for (int e = 1; e < 8; e++) x = fmaxf(x, sv[cb][e]);
+            mx[cb] = pw_quad_max(x);
+            grow |= (m[cb] == -INFINITY) ? (mx[cb] > -INFINITY) : (mx[cb] > m[cb] + PW_RESCALE_SLACK);
+        }
+        return __builtin_amdgcn_ballot_w64(grow) != 0;
+    };
+    auto move_reference = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            const bool first = m[cb] == -INFINITY;
+            const bool grow = first ? (mx[cb] > -INFINITY) : (mx[cb] > m[cb] + PW_RESCALE_SLACK);
+            const float m_new = grow ? mx[cb] : m[cb];
+            const float corr = (grow && !first) ? __builtin_amdgcn_exp2f(m[cb] - m_new) : 1.0f;
+            m[cb] = m_new;
+            l[cb] *= corr;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[cb][nb][r] *= corr;
+        }
+    };
+    auto tile_back = [&]() __attribute__((always_inline)) {
+        vec8 pop[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            const float m_safe = (m[cb] == -INFINITY) ? 0.0f : m[cb];
+            float pe[8], psum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                pe[e] = __builtin_amdgcn_exp2f(sv[cb][e] - m_safe);
+                psum += pe[e];
+            }
+            l[cb] += psum;
+            // P^T operand: contraction slot (q4, e) is key 4 q4 + e (e < 4) or 16 + 4 q4 + e - 4
+            const uint4_t praw = {WideMma<T>::pack2(pe[0], pe[1]), WideMma<T>::pack2(pe[2], pe[3]),
+                                  WideMma<T>::pack2(pe[4], pe[5]), WideMma<T>::pack2(pe[6], pe[7])};
+            pop[cb] = __builtin_bit_cast(vec8, praw);
+        }
+        // O^T[dim][col] += V^T . P^T: the transposing load hands lane i of a 16-lane block V[row0 + 0..3][dim0 + i];
+        // the lane supplies the address of row0 + i / 4, dims dim0 + 4 (i % 4)
+        const int trow = 4 * q4 + (j >> 2);
+        const int tcol = 4 * (j & 3) * 2;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                PWLDS_PTR(short4_t, sbase + K_BYTES + trow * VP + nb * 32 + tcol));
+            const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                PWLDS_PTR(short4_t, sbase + K_BYTES + (16 + trow) * VP + nb * 32 + tcol));
+            const uint2w_t u0 = __builtin_bit_cast(uint2w_t, a0), u1 = __builtin_bit_cast(uint2w_t, a1);
+            const uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+                o[cb][nb] = WideMma<T>::mfma(__builtin_bit_cast(vec8, araw), pop[cb], o[cb][nb]);
+        }
+    };
+    for (int t = 0;;) {
+        for (; t < ntiles; t++) {
+            if (tile_front(t)) break;
+            tile_back();
+        }
+        if (t >= ntiles) break;
+        move_reference();
+        tile_back();
+        t++;
+    }
+
+    // ---- epilogue: out[row][16 nb + 4 q4 + r] = O^T / l (no visible key: 0 / 0 = NaN like the reference) -------
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const float l_col = pw_quad_sum(l[cb]);
+        if (row[cb] >= p.Sq) continue;
+        if (nks > 1) {
+            // this share's state: O unnormalised, then (m, l); the merge kernel normalises
+            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + row[cb]) * nks + ksplit) * p.pf_pitch;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) *(float4_t *)(ws + 16 * nb + 4 * q4) = o[cb][nb];
+            if (q4 == 0) {
+                ws[D] = m[cb];
+                ws[D + 1] = l_col;
+            }
+            continue;
+        }
+        const int64_t ob = b * p.os[0] + h * p.os[1] + (int64_t)row[cb] * p.os[2];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float val = o[cb][nb][r] / l_col;
+                const int64_t oi = ob + (int64_t)(16 * nb + 4 * q4 + r) * p.os[3];
+                if (p.out_f32) ((float *)p.out)[oi] = val;
+                else ((T *)p.out)[oi] = from_float<T>(val);
+            }
+    }
+}
+
+template <typename T>
+int launch_wide_t(const AttnParams &p, hipStream_t stream) {
+    const int nqb = (p.Sq + PW_BM - 1) / PW_BM;
+    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
+    if (blocks > 0x7fffffffL) {
+        set_error("prefill: too many workgroups (%ld)", blocks);
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)blocks), block(64 * PW_WAVES);
+    switch (p.D) {
+        case 160: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 160>), grid, block, stream, p, p, nqb); break;
+        case 192: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 192>), grid, block, stream, p, p, nqb); break;
+        case 224: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 224>), grid, block, stream, p, p, nqb); break;
+        case 256: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 256>), grid, block, stream, p, p, nqb); break;
+        default: set_error("wide prefill MFMA kernel: head_dim %d not in {160, 192, 224, 256}", p.D); return FHIP_ERR_UNSUPPORTED;
+    }
+    FHIP_HIP_CHECK(hipGetLastError());
+    if (p.pf_nsplit > 1) return launch_prefill_merge(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
+    return FHIP_OK;
+}
+
+}  // namespace
+
+// Few query rows on a long cache: 128-row query blocks alone leave most CUs idle, so the keys are split over workgroups
+// too, down to 1024 keys per share, until there are about two workgroups per CU (the rule of the other tiled kernels).
+void prefill_mfma_wide_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+    *nsplit = 1;
+    *chunk = Skv;
+    if (causal_square) return;
+    const long wgs = (long)B * H * ((Sq + PW_BM - 1) / PW_BM);
+    if (2 * wgs > compute_units) return;
+    const long want = (2L * compute_units + wgs - 1) / wgs;
+    const long most = Skv / 1024;
+    const long ns = want < most ? want : most;
+    if (ns < 2) return;
+    long c = (Skv + ns - 1) / ns;
+    c = (c + PW_KEYS - 1) / PW_KEYS * PW_KEYS;
+    *chunk = (int)c;
+    *nsplit = (int)((Skv + c - 1) / c);
+}
+
+int launch_prefill_mfma_wide(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
+    if (dtype == FHIP_F16) return launch_wide_t<half_t>(p, stream);
+    if (dtype == FHIP_BF16) return launch_wide_t<bf16_t>(p, stream);
+    set_error("wide prefill MFMA kernel takes f16/bf16 only");
+    return FHIP_ERR_UNSUPPORTED;
+}
+
+}  // namespace fhip

@@ -167,7 +167,10 @@ def test_kernel_selection():
     assert selected(a)[1] == fa.KERNEL_GENERIC
     # 16-bit head dims their own matrix-core kernel does not take run on the f32-arithmetic kernel
     assert selected(make_args(Sq=64, Skv=64, D=80))[1] == fa.KERNEL_PREFILL_F32
-    assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_F32
+    assert selected(make_args(Sq=64, Skv=64, D=200, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_F32
+    # ... and 160 / 192 / 224 / 256 on the wide-head form of the 16-bit kernel
+    assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_MFMA
+    assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.F32))[1] == fa.KERNEL_PREFILL_F32
     assert selected(make_args(Sq=64, Skv=64, D=264))[1] == fa.KERNEL_GENERIC
     # innermost stride != 1 or a misaligned base pointer -> generic
     a = make_args(Sq=64, Skv=64, D=128)

@@ -317,7 +317,7 @@ def test_prefill_f32_wide_heads(device, D, case):
 
 
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
-@pytest.mark.parametrize("D,case", [(80, "causal"), (256, "causal"), (192, "window_offset"), (32, "full_ragged"), (40, "causal"),
+@pytest.mark.parametrize("D,case", [(80, "causal"), (144, "causal"), (200, "window_offset"), (32, "full_ragged"), (40, "causal"),
                                     (128, "bias"), (64, "bias"), (96, "bias_batch_key")])
 def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
     """Head dims and mask tensors the 16-bit matrix-core kernel does not take run on the tiled kernel that computes
@@ -355,6 +355,65 @@ def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
         out32 = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out_dtype=fa.F32).to_numpy()
         assert out32.dtype == np.float32
         assert_parity(out32, ref, TOL_F32, f"f32 result, D{D} {case}")
+
+
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("D", [160, 192, 224, 256])
+@pytest.mark.parametrize("case", ["causal", "chunk_window", "ragged", "mask_tensor", "bias", "padding_mask", "cache_views", "full"])
+def test_wide_head_dims_on_the_16_bit_matrix_cores(device, dtype, D, case):
+    """Head dims 160 ... 256 (Gemma-3's key length is 256) in 16-bit: the four-wavefront tiled kernel, 128 query rows per
+    workgroup and 32-key tiles; every way of masking, rows and keys that do not fill their last block or tile, K and V
+    as narrowed views of a larger cache allocation, GQA, and the output in f32 as well."""
+    B, H, Hkv = 2, 6, 2
+    Sq, Skv = {"causal": (300, 300), "chunk_window": (130, 1000), "ragged": (70, 777), "mask_tensor": (150, 419),
+               "bias": (90, 200), "padding_mask": (129, 333), "cache_views": (200, 200), "full": (33, 1)}[case]
+    q, k, v = _normal_qkv(16, B, H, Hkv, Sq, Skv, D)
+    tq = fa.Tensor.from_numpy(device, q, dtype)
+    if case == "cache_views":
+        kbuf, vbuf = np.zeros((B, Hkv, 256, D), np.float32), np.zeros((B, Hkv, 256, D), np.float32)
+        kbuf[:, :, :Skv], vbuf[:, :, :Skv] = k, v
+        tk = fa.Tensor.from_numpy(device, kbuf, dtype).narrow(2, 0, Skv)
+        tv = fa.Tensor.from_numpy(device, vbuf, dtype).narrow(2, 0, Skv)
+    else:
+        tk, tv = fa.Tensor.from_numpy(device, k, dtype), fa.Tensor.from_numpy(device, v, dtype)
+    mask, kind, mt, kw = None, None, None, {}
+    lens = None
+    if case in ("causal", "cache_views"):
+        kw["analytic"] = (True, 0, 0)
+        mask, kind = _analytic_mask(Sq, Skv, True, 0, 0), "qk"
+    elif case == "chunk_window":
+        kw["analytic"] = (True, Skv - Sq, 333)
+        mask, kind = _analytic_mask(Sq, Skv, True, Skv - Sq, 333), "qk"
+    elif case == "ragged":
+        lens = np.array([777, 95], np.int32)
+        kw["kv_lens"] = fa.IntTensor(device, lens)
+    elif case == "mask_tensor":
+        mask, kind = oracle.get_mask(Sq, Skv - Sq, None), "qk"
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "bias":  # not made of intervals: the kernel queued behind the tiled one serves the call
+        mask, kind = np.random.default_rng(3).normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
+        mask[:, 100:140] = NEG_INF
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "padding_mask":
+        mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+        mask[0, 300:] = NEG_INF
+        mask[1, :50] = NEG_INF
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.BatchKeyMask)
+    if mt is None:
+        assert tq.selected_kernel(tk, tv, 0.1, **kw) == fa.KERNEL_PREFILL_MFMA
+    tol = dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16
+    for out_dtype in (None, fa.F32):
+        out = tq.flash_attention(tk, tv, D ** -0.5, mt, out_dtype=out_dtype, **kw).to_numpy()
+        if lens is None:
+            ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                         None if mask is None else rounded(mask, dtype), kind)
+            assert_parity(out, ref, tol, f"D{D} {case} out {out_dtype}")
+        else:
+            for b in range(B):
+                n = int(lens[b])
+                ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                             rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+                assert_parity(out[b:b + 1], ref, tol, f"D{D} ragged b{b} out {out_dtype}")
 
 
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
@@ -689,6 +748,35 @@ def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype,
             ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
                                          rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
             assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
+
+
+@pytest.mark.parametrize("dtype,tol", [(fa.F16, 2e-3), (fa.BF16, 8e-3)])
+@pytest.mark.parametrize("D", [160, 256])
+@pytest.mark.parametrize("growth", [0.02, 0.3, 3.0, 40.0])
+def test_wide_head_prefill_when_the_row_maximum_keeps_rising(device, dtype, tol, D, growth):
+    """The wide-head kernel moves a column's reference maximum (and rescales its accumulators) only when a tile
+    exceeds it by more than 2^8.  Scores that climb along the keys by `growth` per 32-key tile on top of unit noise
+    walk through every regime: never again after the first tile, once in many tiles, every tile, and every tile by
+    far more than the slack (softmax rows close to one-hot on the last visible key)."""
+    B, H, Hkv, Sq, Skv = 1, 4, 2, 200, 1100
+    rng = np.random.default_rng(5)
+    q = rng.normal(0, 1, (B, H, Sq, D)).astype(np.float32)
+    k = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    v = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    # dim 0 of every query is sqrt(D), dim 0 of key j is growth * j / 32: the scaled score gains growth per tile
+    q[..., 0] = D ** 0.5
+    k[..., 0] = (growth / 32.0) * np.arange(Skv, dtype=np.float32)[None, None, :]
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    for analytic in ((True, Skv - Sq, 0), (True, Skv - Sq, 300), None):
+        kw = {} if analytic is None else {"analytic": analytic}
+        assert tq.selected_kernel(tk, tv, D ** -0.5, **kw) == fa.KERNEL_PREFILL_MFMA
+        out = tq.flash_attention(tk, tv, D ** -0.5, out_dtype=fa.F32, **kw).to_numpy()
+        mask = None if analytic is None else _analytic_mask(Sq, Skv, *analytic)
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                     None if mask is None else "qk")
+        assert np.isfinite(out).all()
+        rl = rel_l2(out, ref)
+        assert rl <= tol, f"rel-L2 {rl:.2e} at growth {growth}, D{D}, mask {analytic}"
 
 
 @pytest.mark.parametrize("dtype,std,tol", [(fa.BF16, 8.0, dict(max_abs=None, rel_l2=8e-3)), (fa.BF16, 30.0, dict(max_abs=None, rel_l2=8e-3)),
