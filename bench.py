@@ -98,6 +98,8 @@ def configs():
         # with one workgroup per CU)
         "F2": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f32", std=0.5, causal=False),
         "W2": dict(kind="decode", B=16, H=16, Hkv=4, Sq=1, Skv=4096, D=256, dtype="f16", std=0.5, causal=False),
+        # a 4096-token prompt at that key length in 16-bit (the four-wavefront tiled kernel for head dims 160 ... 256)
+        "W3": dict(kind="prefill", B=1, H=16, Hkv=4, Sq=4096, Skv=4096, D=256, dtype="f16", std=1.0, causal=True),
         # a multi-token decode step: C2's batch with four new rows per sequence at the end of the cache, causal among
         # themselves (a draft being verified); the rows ride beside the heads of a GQA group, the cache is read once
         "M1": dict(kind="decode", B=16, H=32, Hkv=8, Sq=4, Skv=4096, D=128, dtype="f16", std=0.5, causal=True),
