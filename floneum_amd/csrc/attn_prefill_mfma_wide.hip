@@ -5,8 +5,9 @@
 // per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is four wavefronts,
 // one per SIMD with the whole register file, and 128 query rows of one (batch, head); the keys are walked in tiles of 32
 // that all four wavefronts share through a double-buffered LDS tile (global -> registers -> LDS, the next tile's loads
-// in flight during the math).  Per tile and wavefront, on v_mfma_f32_16x16x32 with the 32 query rows as two blocks of
-// 16 columns (the arithmetic of the split-KV decode kernel with two column blocks, attn_decode.hip):
+// in flight during the math).  (Head dim 192 runs as eight wavefronts of 16 rows instead, see wide_waves.)  Per tile and
+// wavefront, on v_mfma_f32_16x16x32 with the 32 query rows as two blocks of 16 columns (the arithmetic of the split-KV
+// decode kernel with two column blocks, attn_decode.hip):
 //   S^T[key][row]  = K . Q^T     A = K from LDS (one 16-byte read feeds both column blocks), B = Q in registers
 //   scores scaled in f32 (scale * log2 e), masked by the row's visible interval, online softmax per column
 //   O^T[dim][row] += V^T . P^T   A = V^T from row-major LDS with ds_read_b64_tr_b16, B = the probabilities
@@ -26,8 +27,7 @@ namespace fhip {
 namespace {
 
 constexpr float PW_LOG2E = 1.4426950408889634f;
-constexpr int PW_WAVES = 4;
-constexpr int PW_BM = 32 * PW_WAVES;  // query rows per workgroup
+constexpr int PW_BM = 128;  // query rows per workgroup: four wavefronts of 32 rows or eight of 16
 constexpr int PW_KEYS = 32;           // keys per tile
 constexpr float PW_RESCALE_SLACK = 8.0f;
 
@@ -75,7 +75,7 @@ __device__ __forceinline__ float pw_quad_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <typename T, int D>
+template <typename T, int D, int PW_WAVES>
 __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
     typedef typename WideMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;           // K tile row pitch (bytes): rows 4 banks apart
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
     constexpr int NLD = 2 * CHUNKS / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
     constexpr int KB = D / 32;               // contraction blocks of K . Q^T
     constexpr int NB = D / 16;               // 16-dim blocks of the output
-    constexpr int CB = 2;                    // 16-column blocks: the wavefront's 32 query rows
+    constexpr int CB = 8 / PW_WAVES;         // 16-column blocks: the wavefront's 32 or 16 query rows
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
     // heads are dealt so that an XCD works on H / 8 neighbouring heads, i.e. on as few KV heads as possible
     if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
-    const int q0 = qb * PW_BM, qw0 = q0 + 32 * wave;
+    const int q0 = qb * PW_BM, qw0 = q0 + 16 * CB * wave;
 
     // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this
     // lane's two rows (element test).  row_bounds gives lane l the interval of row qw0 + l % 32.
@@ -249,13 +249,17 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
         const bool all_visible = j0 >= full_lo_w && j0 + PW_KEYS <= full_hi_w;  // no element test needed
 
         // S^T[key][col] = K . Q^T : two 16-key halves, every K operand read serves both column blocks
+        // (contraction blocks outermost: four accumulators take turns, so that a matrix instruction never waits for
+        // the result of the one just issued)
         float4_t s[CB][2];
 #pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
+        for (int hf = 0; hf < 2; hf++)
 #pragma unroll
             for (int cb = 0; cb < CB; cb++) s[cb][hf] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kb = 0; kb < KB; kb++) {
+        for (int kb = 0; kb < KB; kb++) {
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
                 const uint4_t raw = *PWLDS_PTR(uint4_t, sbase + (16 * hf + j) * KP + (32 * kb + 8 * q4) * 2);
 #pragma unroll
                 for (int cb = 0; cb < CB; cb++)
@@ -373,6 +377,12 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
     }
 }
 
+// Wavefronts per workgroup.  Eight wavefronts of 16 rows (two per SIMD, half the register file each) hide each other's
+// dependent phases but read every K and V operand from LDS for half as many matrix instructions: measured +16 % at
+// head_dim 192 and -5 % at 256 (f16, 4096 x 4096 causal).  160 and 224 do not deal their tile pieces evenly to 512
+// threads.
+constexpr int wide_waves(int d) { return d == 192 ? 8 : 4; }
+
 template <typename T>
 int launch_wide_t(const AttnParams &p, hipStream_t stream) {
     const int nqb = (p.Sq + PW_BM - 1) / PW_BM;
@@ -381,12 +391,12 @@ int launch_wide_t(const AttnParams &p, hipStream_t stream) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
     }
-    const dim3 grid((unsigned)blocks), block(64 * PW_WAVES);
+    const dim3 grid((unsigned)blocks), block(64 * wide_waves(p.D));
     switch (p.D) {
-        case 160: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 160>), grid, block, stream, p, p, nqb); break;
-        case 192: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 192>), grid, block, stream, p, p, nqb); break;
-        case 224: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 224>), grid, block, stream, p, p, nqb); break;
-        case 256: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 256>), grid, block, stream, p, p, nqb); break;
+        case 160: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 160, wide_waves(160)>), grid, block, stream, p, p, nqb); break;
+        case 192: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 192, wide_waves(192)>), grid, block, stream, p, p, nqb); break;
+        case 224: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 224, wide_waves(224)>), grid, block, stream, p, p, nqb); break;
+        case 256: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 256, wide_waves(256)>), grid, block, stream, p, p, nqb); break;
         default: set_error("wide prefill MFMA kernel: head_dim %d not in {160, 192, 224, 256}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());
