@@ -30,7 +30,7 @@ NATIVE = {fa.F16: (1e-2, 2e-3), fa.BF16: (1e-1, 2e-2)}
 
 def _case(rng, device):
     dtype = [fa.F32, fa.F16, fa.BF16][rng.integers(3)]
-    D = int(rng.choice([8, 16, 32, 40, 64, 80, 96, 128, 160, 192, 256, 12, 36, 100, 33]))
+    D = int(rng.choice([8, 16, 32, 40, 64, 80, 96, 128, 160, 192, 224, 256, 12, 36, 100, 33]))
     Hkv = int(rng.integers(1, 4))
     H = Hkv * int(rng.choice([1, 2, 4, 8]))
     B = int(rng.integers(1, 4))
