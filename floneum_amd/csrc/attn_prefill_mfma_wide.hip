@@ -27,7 +27,7 @@ namespace fhip {
 namespace {
 
 constexpr float PW_LOG2E = 1.4426950408889634f;
-constexpr int PW_BM = 128;  // query rows per workgroup: four wavefronts of 32 rows or eight of 16
+constexpr int PW_BM = 128;  // query rows per workgroup: four wavefronts of 32 rows or eight of 16 (64 on small grids)
 constexpr int PW_KEYS = 32;           // keys per tile
 constexpr float PW_RESCALE_SLACK = 8.0f;
 
@@ -75,8 +75,10 @@ __device__ __forceinline__ float pw_quad_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <typename T, int D, int PW_WAVES>
-__global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
+// PW_WAVES wavefronts of 16 * CB query rows: <4, 2> and <8, 1> are one workgroup per CU, <4, 1> (64-row workgroups
+// for grids that would leave CUs idle) two.
+template <typename T, int D, int PW_WAVES, int CB>
+__global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
     typedef typename WideMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;           // K tile row pitch (bytes): rows 4 banks apart
     constexpr int VP = D * 2 + 32;           // V tile row pitch (bytes): rows 8 banks apart
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
     constexpr int NLD = 2 * CHUNKS / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
     constexpr int KB = D / 32;               // contraction blocks of K . Q^T
     constexpr int NB = D / 16;               // 16-dim blocks of the output
-    constexpr int CB = 8 / PW_WAVES;         // 16-column blocks: the wavefront's 32 or 16 query rows
+    constexpr int BM = 16 * CB * PW_WAVES;   // query rows per workgroup (CB 16-column blocks per wavefront)
     __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
@@ -112,11 +114,11 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
     // heads are dealt so that an XCD works on H / 8 neighbouring heads, i.e. on as few KV heads as possible
     if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
-    const int q0 = qb * PW_BM, qw0 = q0 + 16 * CB * wave;
+    const int q0 = qb * BM, qw0 = q0 + 16 * CB * wave;
 
     // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this
     // lane's two rows (element test).  row_bounds gives lane l the interval of row qw0 + l % 32.
-    RowBounds rb = row_bounds(p, b, q0, PW_BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
     if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -383,20 +385,37 @@ __global__ __launch_bounds__(64 * PW_WAVES, 1) void prefill_mfma_wide_kernel(Att
 // threads.
 constexpr int wide_waves(int d) { return d == 192 ? 8 : 4; }
 
+template <typename T, int D>
+void launch_wide_d(const AttnParams &p, int bm, const dim3 &grid, int nqb, hipStream_t stream) {
+    if (bm == 64) {
+        FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, D, 4, 1>), grid, dim3(256), stream, p, p, nqb);
+    } else {
+        constexpr int W = wide_waves(D);
+        FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, D, W, 8 / W>), grid, dim3(64 * W), stream, p, p, nqb);
+    }
+}
+
 template <typename T>
 int launch_wide_t(const AttnParams &p, hipStream_t stream) {
-    const int nqb = (p.Sq + PW_BM - 1) / PW_BM;
+    // A grid of fewer than two 128-row workgroups per CU that cannot split the keys (a causal prompt of up to a few
+    // thousand tokens) runs as 64-row workgroups, two per CU: twice the workgroups of half the length, which fill idle
+    // CUs and even out the long and short row blocks of a causal mask, each reading K and V from LDS for half as
+    // many matrix instructions (f16, head_dim 256, 16 heads: 512 tokens 48 -> 33 us, 1024: 72 -> 52, 2048: 125 -> 108,
+    // 3072: 179 -> 170).
+    const long wgs128 = (long)p.B * p.H * ((p.Sq + PW_BM - 1) / PW_BM);
+    const int bm = (p.pf_nsplit <= 1 && wgs128 < 2 * p.cus) ? 64 : PW_BM;
+    const int nqb = (p.Sq + bm - 1) / bm;
     const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
     }
-    const dim3 grid((unsigned)blocks), block(64 * wide_waves(p.D));
+    const dim3 grid((unsigned)blocks);
     switch (p.D) {
-        case 160: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 160, wide_waves(160)>), grid, block, stream, p, p, nqb); break;
-        case 192: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 192, wide_waves(192)>), grid, block, stream, p, p, nqb); break;
-        case 224: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 224, wide_waves(224)>), grid, block, stream, p, p, nqb); break;
-        case 256: FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, 256, wide_waves(256)>), grid, block, stream, p, p, nqb); break;
+        case 160: launch_wide_d<T, 160>(p, bm, grid, nqb, stream); break;
+        case 192: launch_wide_d<T, 192>(p, bm, grid, nqb, stream); break;
+        case 224: launch_wide_d<T, 224>(p, bm, grid, nqb, stream); break;
+        case 256: launch_wide_d<T, 256>(p, bm, grid, nqb, stream); break;
         default: set_error("wide prefill MFMA kernel: head_dim %d not in {160, 192, 224, 256}", p.D); return FHIP_ERR_UNSUPPORTED;
     }
     FHIP_HIP_CHECK(hipGetLastError());

@@ -750,6 +750,39 @@ def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype,
             assert_parity(out[b:b + 1], ref, tol, f"sequence {b} of length {n}")
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
+@pytest.mark.parametrize("D", [160, 192, 224, 256])
+@pytest.mark.parametrize("case", ["causal", "chunk_window", "ragged"])
+def test_wide_head_dims_on_a_grid_that_fills_the_chip(device, dtype, D, case):
+    """The wide-head kernel has two workgroup shapes: 128 query rows (one workgroup per CU) when those fill the chip
+    twice over or the keys are split, 64 rows (two per CU) otherwise.  The other tests of these head dims are small
+    grids; here 4 x 64 heads x 2 row blocks reach twice the CU count, so the 128-row form runs (its second row block
+    holds two rows)."""
+    B, H, Hkv, Sq = 4, 64, 16, 130
+    assert B * H * ((Sq + 127) // 128) >= 2 * device.compute_units
+    Skv = {"causal": 130, "chunk_window": 400, "ragged": 333}[case]
+    q, k, v = _normal_qkv(23, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    kw, mask, lens = {}, None, None
+    if case == "causal":
+        kw["analytic"] = (True, 0, 0)
+        mask = _analytic_mask(Sq, Skv, True, 0, 0)
+    elif case == "chunk_window":
+        kw["analytic"] = (True, Skv - Sq, 200)
+        mask = _analytic_mask(Sq, Skv, True, Skv - Sq, 200)
+    else:
+        lens = np.array([333, 41, 1, 200], np.int32)
+        kw["kv_lens"] = fa.IntTensor(device, lens)
+    assert tq.selected_kernel(tk, tv, 0.1, **kw) == fa.KERNEL_PREFILL_MFMA
+    out = tq.flash_attention(tk, tv, D ** -0.5, **kw).to_numpy()
+    tol = dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16
+    for b in range(B):
+        n = Skv if lens is None else int(lens[b])
+        ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                     rounded(v[b:b + 1, :, :n], dtype), D ** -0.5, mask, None if mask is None else "qk")
+        assert_parity(out[b:b + 1], ref, tol, f"D{D} {case}, sequence {b}")
+
+
 @pytest.mark.parametrize("dtype,tol", [(fa.F16, 2e-3), (fa.BF16, 8e-3)])
 @pytest.mark.parametrize("D", [160, 256])
 @pytest.mark.parametrize("growth", [0.02, 0.3, 3.0, 40.0])
