@@ -5,7 +5,7 @@
 // per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is four wavefronts,
 // one per SIMD with the whole register file, and 128 query rows of one (batch, head); the keys are walked in tiles of 32
 // that all four wavefronts share through a double-buffered LDS tile (global -> registers -> LDS, the next tile's loads
-// in flight during the math).  (Head dim 192 runs as eight wavefronts of 16 rows instead, see wide_waves.)  Per tile and
+// in flight during the math).  (Head dims below 256 run as eight wavefronts of 16 rows instead, see wide_waves.)  Per tile and
 // wavefront, on v_mfma_f32_16x16x32 with the 32 query rows as two blocks of 16 columns (the arithmetic of the split-KV
 // decode kernel with two column blocks, attn_decode.hip):
 //   S^T[key][row]  = K . Q^T     A = K from LDS (one 16-byte read feeds both column blocks), B = Q in registers
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     constexpr int STAGE = K_BYTES + V_BYTES;
     constexpr int CPR = D / 8;               // 16-byte chunks per row
     constexpr int CHUNKS = PW_KEYS * CPR;    // per tensor and tile
-    constexpr int NLD = 2 * CHUNKS / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
+    constexpr int NLD = (2 * CHUNKS + 64 * PW_WAVES - 1) / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
     constexpr int KB = D / 32;               // contraction blocks of K . Q^T
     constexpr int NB = D / 16;               // 16-dim blocks of the output
     constexpr int BM = 16 * CB * PW_WAVES;   // query rows per workgroup (CB 16-column blocks per wavefront)
@@ -144,11 +144,16 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
 
     // tile movement: every thread takes NLD 16-byte chunks of K and of V; rows beyond the key axis repeat the last row
     // (their scores are masked by the rows' intervals, which end at the key count)
-    // The K and the V tile are one list of 2 * CHUNKS 16-byte pieces, dealt to the 256 threads NLD at a time (an exact
-    // division for every head dim served; with 160 and 224 one of a thread's pieces is of K in half the threads and
-    // of V in the others).  A piece sits at a fixed byte offset from its tile's first key (the host admits row strides
-    // below 2^25 elements only, so it fits 32 bits); the tiles' own addresses are the same in every lane.
-    static_assert(NLD * 64 * PW_WAVES == 2 * CHUNKS, "pieces per thread");
+    // The K and the V tile are one list of 2 * CHUNKS 16-byte pieces, dealt to the threads NLD at a time (with 160 and
+    // 224 one of a thread's pieces is of K in half the threads and of V in the others; with eight wavefronts at those
+    // head dims the last round of pieces goes to the first four wavefronts only, a whole-wavefront condition).  A piece
+    // sits at a fixed byte offset from its tile's first key (the host admits row strides below 2^25 elements only, so
+    // it fits 32 bits); the tiles' own addresses are the same in every lane.
+    constexpr int LAST_ROUND = 2 * CHUNKS - 64 * PW_WAVES * (NLD - 1);  // pieces of the last round
+    static_assert(LAST_ROUND % 64 == 0 && LAST_ROUND > 0, "whole wavefronts in the last round");
+    auto has_piece = [&](int u) __attribute__((always_inline)) -> bool {
+        return LAST_ROUND == 64 * PW_WAVES || u < NLD - 1 || wave < LAST_ROUND / 64;
+    };
     uint4_t st[NLD];  // the tile in flight from HBM
     // With 32 pieces per row (head dim 256) a thread's pieces are the same column of every eighth row: two offsets
     // and constant steps describe them all, which the full register file of this head dim needs.
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
 #pragma unroll
             for (int u = 0; u < NLD; u++) {
                 const bool is_v = tid + 64 * PW_WAVES * u >= CHUNKS;  // known at compile time except for the mixed piece
-                st[u] = *(const uint4_t *)((is_v ? vt : kt) + goff(u));
+                if (has_piece(u)) st[u] = *(const uint4_t *)((is_v ? vt : kt) + goff(u));
             }
             return;
         }
@@ -200,12 +205,13 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
             const bool is_v = cid >= CHUNKS;
             const int r = (is_v ? cid - CHUNKS : cid) / CPR, c = (is_v ? cid - CHUNKS : cid) % CPR;
             const int64_t row_stride = is_v ? p.vs[2] : p.ks[2];
-            st[u] = *(const uint4_t *)((is_v ? vt : kt) + (min(r, last) * row_stride + c * 8) * 2);
+            if (has_piece(u)) st[u] = *(const uint4_t *)((is_v ? vt : kt) + (min(r, last) * row_stride + c * 8) * 2);
         }
     };
     auto store_tile = [&](int stage_base) __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < NLD; u++) *PWLDS_PTR(uint4_t, stage_base + loff(u)) = st[u];
+        for (int u = 0; u < NLD; u++)
+            if (has_piece(u)) *PWLDS_PTR(uint4_t, stage_base + loff(u)) = st[u];
     };
 
     const int j_begin = (lo_wg / PW_KEYS) * PW_KEYS;
@@ -380,10 +386,10 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
 }
 
 // Wavefronts per workgroup.  Eight wavefronts of 16 rows (two per SIMD, half the register file each) hide each other's
-// dependent phases but read every K and V operand from LDS for half as many matrix instructions: measured +16 % at
-// head_dim 192 and -5 % at 256 (f16, 4096 x 4096 causal).  160 and 224 do not deal their tile pieces evenly to 512
-// threads.
-constexpr int wide_waves(int d) { return d == 192 ? 8 : 4; }
+// dependent phases but read every K and V operand from LDS for half as many matrix instructions: measured (f16,
+// 4096 x 4096 causal) +15 % at head_dim 160, +16 % at 192, +6 % at 224 and -5 % at 256, where the eight-wavefront form
+// leaves 7 of its 256 registers free.
+constexpr int wide_waves(int d) { return d == 256 ? 4 : 8; }
 
 template <typename T, int D>
 void launch_wide_d(const AttnParams &p, int bm, const dim3 &grid, int nqb, hipStream_t stream) {
