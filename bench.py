@@ -606,6 +606,11 @@ def main():
             r = run_config(name, steps, warmup, with_cpu=not a.no_cpu)
             r["steps"], r["warmup"] = steps, warmup
             line["configs"][name] = r
+        # (W2 / W3: a decode step and a 4096-token prompt at Gemma-3's key length 256 in f16; no CPU leg)
+        for name, (steps, warmup) in (("W2", (100, 10)), ("W3", (50, 100))):
+            r = run_config(name, steps, warmup, with_cpu=False)
+            r["steps"], r["warmup"] = steps, warmup
+            line["configs"][name] = r
     print(json.dumps(line))
 
 
