@@ -292,8 +292,8 @@ static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *
     const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
     const int Hkv = (int)a->k.shape[1];
     if (a->q.shape[3] > 128)  // the wide-head form: 128-row query blocks
-        prefill_mfma_wide_plan((int)a->q.shape[0], (int)a->q.shape[1], (int)a->q.shape[2], (int)a->k.shape[2], causal_square,
-                               cus > 0 ? cus : 256, nsplit, chunk);
+        prefill_mfma_wide_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
+                               (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
     else
         prefill_mfma_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
                           (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);

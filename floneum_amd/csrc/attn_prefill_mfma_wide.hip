@@ -102,23 +102,30 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     const int q4 = lane >> 4;  // key group
 
     // workgroup -> (share of the keys, query block, batch, head): long (late) query blocks first
-    const int bh_count = p.B * p.H;
+    // Packed form (at most 32 query rows, GQA group a multiple of 4; not for the 64-row workgroups): the workgroup's
+    // wavefronts hold rows 0..31 of four query heads that share a KV head (wavefront w: head w % 4, and with eight
+    // wavefronts rows 16 (w / 4) ...), so the K and V tiles it moves serve all four and a few new rows on a long cache
+    // read the cache once per KV head, not once per query head.
+    const int pack = (PW_WAVES * CB == 8) ? p.pf_pack : 0;
+    const int heads = pack ? p.H / 4 : p.H;  // head units per batch entry
+    const int bh_count = p.B * heads;
     const int nks = max(p.pf_nsplit, 1);
     const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
     const int id = blockIdx.x / nks;
     const int qb = nqb - 1 - id / bh_count;
     const int rem = id % bh_count;
-    const int b = rem / p.H;
-    int h = rem % p.H;
+    const int b = rem / heads;
+    int h = rem % heads;
     // consecutive workgroups land on consecutive XCDs (id % 8), each with an L2 of its own: with H a multiple of 8 the
     // heads are dealt so that an XCD works on H / 8 neighbouring heads, i.e. on as few KV heads as possible
-    if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
+    if (pack) h = 4 * h + (wave & 3);
+    else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
-    const int q0 = qb * BM, qw0 = q0 + 16 * CB * wave;
+    const int q0 = pack ? 0 : qb * BM, qw0 = pack ? 16 * CB * (wave >> 2) : q0 + 16 * CB * wave;
 
     // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this
     // lane's two rows (element test).  row_bounds gives lane l the interval of row qw0 + l % 32.
-    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, pack ? 32 : BM, qw0, lane);
     if (nks > 1) {  // few query rows on a long cache: this workgroup takes one share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -402,16 +409,21 @@ void launch_wide_d(const AttnParams &p, int bm, const dim3 &grid, int nqb, hipSt
 }
 
 template <typename T>
-int launch_wide_t(const AttnParams &p, hipStream_t stream) {
+int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
+    AttnParams p = p_in;
+    p.pf_pack = prefill_mfma_pack(p.B, p.H, p.G, p.Sq, p.Skv, p.cus > 0 ? p.cus : 256);
     // A grid of fewer than two 128-row workgroups per CU that cannot split the keys (a causal prompt of up to a few
     // thousand tokens) runs as 64-row workgroups, two per CU: twice the workgroups of half the length, which fill idle
     // CUs and even out the long and short row blocks of a causal mask, each reading K and V from LDS for half as
     // many matrix instructions (f16, head_dim 256, 16 heads: 512 tokens 48 -> 33 us, 1024: 72 -> 52, 2048: 125 -> 108,
     // 3072: 179 -> 170).
     const long wgs128 = (long)p.B * p.H * ((p.Sq + PW_BM - 1) / PW_BM);
-    const int bm = (p.pf_nsplit <= 1 && wgs128 < 2 * p.cus) ? 64 : PW_BM;
-    const int nqb = (p.Sq + bm - 1) / bm;
-    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
+    // (With the keys split, up to 64 rows are one row block either way: the 64-row form computes half as much per tile
+    // and runs two workgroups per CU: f16, head_dim 256, B8 x 16 heads, 64 rows on 8192 keys 271 -> 181 us.)
+    const bool small = p.pf_nsplit <= 1 ? wgs128 < 2 * p.cus : p.Sq <= 64;
+    const int bm = (!p.pf_pack && small) ? 64 : PW_BM;
+    const int nqb = p.pf_pack ? 1 : (p.Sq + bm - 1) / bm;
+    const long blocks = (long)nqb * p.B * (p.pf_pack ? p.H / 4 : p.H) * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -433,17 +445,28 @@ int launch_wide_t(const AttnParams &p, hipStream_t stream) {
 
 // Few query rows on a long cache: 128-row query blocks alone leave most CUs idle, so the keys are split over workgroups
 // too, down to 1024 keys per share, until there are about two workgroups per CU (the rule of the other tiled kernels).
-void prefill_mfma_wide_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+void prefill_mfma_wide_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk) {
     *nsplit = 1;
     *chunk = Skv;
     if (causal_square) return;
-    const long wgs = (long)B * H * ((Sq + PW_BM - 1) / PW_BM);
-    if (2 * wgs > compute_units) return;
-    const long want = (2L * compute_units + wgs - 1) / wgs;
-    const long most = Skv / 1024;
-    const long ns = want < most ? want : most;
-    if (ns < 2) return;
-    long c = (Skv + ns - 1) / ns;
+    const int pack = prefill_mfma_pack(B, H, G, Sq, Skv, compute_units);
+    const long wgs = (long)B * (pack ? H / 4 : H) * ((Sq + PW_BM - 1) / PW_BM);
+    // places for workgroups: one per CU, two for the 64-row form that serves up to 64 rows.  A tile takes this kernel
+    // microseconds whatever part of the row block is real, so a grid that leaves places empty splits its keys.
+    const long places = (!pack && Sq <= 64 ? 2L : 1L) * compute_units;
+    if (wgs >= places) return;
+    // The share count that needs the fewest tile steps: rounds of `places` workgroups, each walking its share of the
+    // keys tile by tile, plus a few steps for parking and merging the partial results of a split.
+    const long most = Skv / 1024 < 64 ? Skv / 1024 : 64;
+    long best_ns = 1, best_cost = (Skv + PW_KEYS - 1) / PW_KEYS;
+    for (long ns = 2; ns <= most; ns++) {
+        const long rounds = (wgs * ns + places - 1) / places;
+        const long tiles = ((Skv + ns - 1) / ns + PW_KEYS - 1) / PW_KEYS;
+        const long cost = rounds * tiles + 4;
+        if (cost < best_cost) best_cost = cost, best_ns = ns;
+    }
+    if (best_ns < 2) return;
+    long c = (Skv + best_ns - 1) / best_ns;
     c = (c + PW_KEYS - 1) / PW_KEYS * PW_KEYS;
     *chunk = (int)c;
     *nsplit = (int)((Skv + c - 1) / c);

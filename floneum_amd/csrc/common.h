@@ -111,7 +111,7 @@ int launch_decode(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 // the same for head dims 160 / 192 / 224 / 256 (four wavefronts per workgroup, 128 query rows, 32-key tiles)
 int launch_prefill_mfma_wide(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
-void prefill_mfma_wide_plan(int B, int H, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk);
+void prefill_mfma_wide_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk);
 // f32 arithmetic on the f32 matrix cores; `dtype` is the tensors' storage type (16-bit rows are widened on load)
 int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 

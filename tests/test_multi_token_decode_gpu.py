@@ -192,7 +192,10 @@ def test_longer_drafts_while_rows_times_group_fit_one_workgroup(device, dtype, G
 
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
 @pytest.mark.parametrize("G,Sq,D,case", [(4, 12, 128, "causal"), (4, 32, 128, "window"), (8, 17, 64, "mask_tensor"),
-                                         (4, 9, 96, "ragged"), (4, 24, 128, "full")])
+                                         (4, 9, 96, "ragged"), (4, 24, 128, "full"),
+                                         # the wide-head kernel's packed form (four wavefronts of 32 rows at 256, eight of 16 below)
+                                         (4, 5, 256, "causal"), (4, 32, 256, "window"), (8, 17, 256, "mask_tensor"),
+                                         (4, 9, 160, "ragged"), (4, 24, 192, "full"), (4, 31, 224, "causal")])
 def test_rows_beyond_the_decode_kernel_share_the_kv_tiles_of_a_gqa_group(device, dtype, G, Sq, D, case):
     """9..32 new rows on a long cache in 16-bit: the tiled prefill kernel in its packed form, where a workgroup's four
     32-row blocks are four query heads of one KV head (the cache is read once per KV head); taken when the packed
