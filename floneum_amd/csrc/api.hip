@@ -202,9 +202,10 @@ static bool decode_eligible(const fhip_attn_args *a) {
         // more rows (a longer draft, a short piece of a prompt) still ride along while rows x group fit the columns one
         // workgroup of a matrix-core variant takes: two blocks of 16 up to head_dim 128, one above
         const uint32_t Hkv = a->k.shape[1], G = Hkv ? a->q.shape[1] / Hkv : 0;
-        const bool matrix_variant = D % 32 == 0 && D >= 32 && D <= (a->dtype == FHIP_F32 ? 192u : 256u);
-        uint32_t max_cols = D <= 128 ? 32u : 16u;
-        if (a->dtype == FHIP_F32) max_cols *= 2;  // two workgroups per KV head (each streams the cache) still beat the f32 prefill kernel
+        const bool matrix_variant = D % 32 == 0 && D >= 32 && D <= 256u;
+        // f32: two column blocks per workgroup up to head_dim 192, and two workgroups per KV head (each streams the
+        // cache) still beat the f32 prefill kernel
+        const uint32_t max_cols = a->dtype == FHIP_F32 ? (D <= 192 ? 64u : 32u) : (D <= 128 ? 32u : 16u);
         if (!matrix_variant || G == 0 || rows * G > max_cols) return false;
     }
     if (D % 8 != 0 || D < 8 || D > 256) return false;

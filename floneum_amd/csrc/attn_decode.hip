@@ -32,16 +32,21 @@ constexpr int DEC_UNROLL = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 
 // the matrix-core variants: 16-bit tensors on the 16-bit instruction at every multiple of 32 up to 256, f32 tensors on
-// the f32 one up to 192 (at 256 the vector variant measured 3 % ahead).  Above 128 one workgroup per CU, whose four
-// wavefronts then have the registers and LDS of eight.  Other head dims run on the vector variant.
-static bool decode_use_mfma(int D, bool f32) {
-    return D % 32 == 0 && D >= 32 && D <= (f32 ? 192 : 256);
+// the f32 one likewise, except that at 224 and 256 a step of up to four columns per KV head (a plain decode step of a
+// 4-way group) stays on the vector variant: the two are within 10 % of each other there, either way by shape, while
+// with more columns the vector variant streams the cache once per query row (4 rows, B8 x 8192 keys, head_dim 256:
+// 396 us against 110).  Above 128 one workgroup per CU, whose four wavefronts then have the registers and LDS of
+// eight.  Other head dims run on the vector variant.  cols: (query head, query row) pairs of a KV head.
+static bool decode_use_mfma(int D, bool f32, int cols) {
+    if (!(D % 32 == 0 && D >= 32 && D <= 256)) return false;
+    return !(f32 && D > 192 && cols <= 4);
 }
 
 // columns ((query head, query row) pairs of a KV head) handled by one workgroup: the matrix-core variants take one
-// block of 16, or two up to head_dim 128 when there are more than 16 columns
+// block of 16, or two when there are more than 16 columns: up to head_dim 128, and up to 192 for f32 tensors (f32, B8 x
+// 8192 keys, 8 rows of a 4-way group at 192: 156 -> 115 us; at 256 the two blocks spill registers: 203 -> 291 us)
 static int decode_gt(int G, int D, bool f32) {
-    if (decode_use_mfma(D, f32)) return (G > 16 && D <= 128) ? 32 : 16;
+    if (decode_use_mfma(D, f32, G)) return (G > 16 && D <= (f32 ? 192 : 128)) ? 32 : 16;
     return G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
 }
 
@@ -55,7 +60,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // or more per CU: chunks of 2048 keys.  With more than 8 columns per unit (a multi-token step: twice the matrix and
     // softmax work per key) also below that, when an even share of the keys per CU is at least 2048 keys long: then
     // every CU gets one workgroup and all are equally long.
-    if (decode_use_mfma(D, f32) && !f32 && D <= 128 && Skv > 2048) {
+    if (decode_use_mfma(D, f32, G) && !f32 && D <= 128 && Skv > 2048) {
         if (units >= compute_units) {
             *waves = 8;
             *chunk = 2048;
@@ -74,7 +79,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // the MFMA variant holds two workgroups per CU (LDS; one above head_dim 128), the vector variant four or more; f32 rows carry
     // twice the bytes per workgroup step and do best with two as well (measured: +3 % at batch 16, +16 % at
     // batch 1 with 32768 keys)
-    const int wgs_per_cu = (decode_use_mfma(D, f32) && D > 128) ? 1 : (decode_use_mfma(D, f32) || f32) ? 2 : 4;
+    const int wgs_per_cu = (decode_use_mfma(D, f32, G) && D > 128) ? 1 : (decode_use_mfma(D, f32, G) || f32) ? 2 : 4;
     const long target = (long)compute_units * wgs_per_cu;
     // short chunks even out a ragged batch (measured: 512 beats 1024 by 12 % on a 128..32768-token
     // batch); with equal lengths the longer chunk is 2-3 % ahead
@@ -85,7 +90,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     // (the vector variant's step is 16 rows of 64 / LPK keys: 64 keys at head_dim 128 in f32, where one step
     // per workgroup is one memory round trip less than two)
     int step_keys = f32 ? 64 : 128;  // matrix-core variants: four wavefronts of 16 (f32) or 32 keys
-    if (!decode_use_mfma(D, f32)) {
+    if (!decode_use_mfma(D, f32, G)) {
         const int lpk = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
         step_keys = 16 * (64 / lpk);
         if (step_keys > 128) step_keys = 128;
@@ -96,7 +101,7 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     const long ns_min = (Skv + max_chunk - 1) / max_chunk;
     if (ns > ns_max) ns = ns_max;
     if (ns < ns_min) ns = ns_min;
-    if (ns < 1 || (Skv <= 256 && decode_use_mfma(D, f32))) ns = 1;
+    if (ns < 1 || (Skv <= 256 && decode_use_mfma(D, f32, G))) ns = 1;
     long c = (Skv + ns - 1) / ns;
     c = (c + step_keys - 1) / step_keys * step_keys;  // whole workgroup steps
     *chunk = (int)c;
@@ -1213,9 +1218,11 @@ static void launch_mfma_f32(const AttnParams &p, dim3 grid, hipStream_t stream) 
         case 128: FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<128, CB>), grid, block, stream, p, p); return;
         default: break;
     }
+    if (p.D == 160) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<160, CB>), grid, block, stream, p, p);
+    else if (p.D == 192) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<192, CB>), grid, block, stream, p, p);
     if constexpr (CB == 1) {
-        if (p.D == 160) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<160, 1>), grid, block, stream, p, p);
-        else FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<192, 1>), grid, block, stream, p, p);
+        if (p.D == 224) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<224, 1>), grid, block, stream, p, p);
+        else if (p.D == 256) FHIP_LAUNCH_MAIN((decode_mfma_f32_kernel<256, 1>), grid, block, stream, p, p);
     }
 }
 
@@ -1231,7 +1238,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
     }
     dim3 grid((unsigned)p.nsplit, (unsigned)gy);
     if constexpr (F32) {
-        if (decode_use_mfma(p.D, true)) {
+        if (decode_use_mfma(p.D, true, p.G * p.Sq)) {
             if (gt == 32) launch_mfma_f32<2>(p, grid, stream);
             else launch_mfma_f32<1>(p, grid, stream);
             FHIP_HIP_CHECK(hipGetLastError());
@@ -1244,7 +1251,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         }
     }
     if constexpr (!F32) {
-        if (decode_use_mfma(p.D, false)) {
+        if (decode_use_mfma(p.D, false, p.G * p.Sq)) {
             if (p.dec_waves == 8) {
                 if (gt == 32) launch_mfma_16<T, 8, 2>(p, grid, stream);
                 else launch_mfma_16<T, 8, 1>(p, grid, stream);

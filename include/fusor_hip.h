@@ -143,10 +143,11 @@ typedef enum {
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */
     FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence, head_dim multiple of 8 up to 256: split-KV
                                       streaming + LSE combine.  Matrix cores at every head_dim that is a multiple
-                                      of 32 (up to 256 on the 16-bit instruction, up to 192 on the f32 one, by
-                                      the tensors' type), vector units otherwise.  At the matrix-core head dims
+                                      of 32 up to 256 (the 16-bit or the f32 instruction, by the tensors' type;
+                                      f32 at 224 / 256 from five columns per KV head on), vector units otherwise.  At the matrix-core head dims
                                       more rows ride along while rows x GQA group <= 32 (16 above head_dim 128;
-                                      twice that for f32 tensors): an 8-token draft on a 4-way GQA model       */
+                                      f32 tensors: 64 up to head_dim 192, 32 above): an 8-token draft on a 4-way
+                                      GQA model                                                               */
 } fhip_kernel_id;
 
 

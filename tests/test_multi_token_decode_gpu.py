@@ -159,11 +159,13 @@ def test_rows_fully_masked_by_their_own_limits_are_nan(device):
                                           (fa.F16, 4, 8, 128), (fa.F32, 4, 7, 128), (fa.BF16, 2, 16, 64), (fa.F16, 1, 32, 96),
                                           (fa.F32, 4, 8, 128), (fa.BF16, 4, 5, 128), (fa.F16, 8, 3, 32), (fa.F16, 1, 16, 256),
                                           (fa.F32, 2, 8, 192), (fa.F32, 1, 32, 32), (fa.F32, 4, 16, 128), (fa.F32, 1, 32, 192),
-                                          (fa.F32, 4, 11, 64)])
+                                          (fa.F32, 4, 11, 64), (fa.F32, 4, 8, 256), (fa.F32, 4, 2, 256), (fa.F32, 1, 5, 224),
+                                          (fa.F32, 8, 4, 256), (fa.F32, 1, 4, 256), (fa.F32, 2, 3, 224), (fa.F32, 4, 16, 192),
+                                          (fa.F32, 4, 8, 160), (fa.F32, 2, 32, 192), (fa.F32, 4, 5, 192)])
 def test_longer_drafts_while_rows_times_group_fit_one_workgroup(device, dtype, G, Sq, D):
     """More than 4 rows while rows x GQA group fit the columns one workgroup of a matrix-core variant takes: two blocks
     of 16 up to head_dim 128 (an 8-token draft on a 4-way GQA model, 32 tokens on an MHA model), one block above; f32
-    tensors twice that, on two workgroups per KV head.  One row more, or a head_dim the matrix-core variants do not
+    tensors two blocks up to head_dim 192 and twice the columns, on two workgroups per KV head.  One row more, or a head_dim the matrix-core variants do not
     take, and the call is a prefill call again."""
     B, Hkv, Skv = 2, 2, 2100
     q, k, v = _normal_qkv(45, B, Hkv * G, Hkv, Sq, Skv, D, 0.5)
@@ -184,7 +186,7 @@ def test_longer_drafts_while_rows_times_group_fit_one_workgroup(device, dtype, G
     assert tq.selected_kernel(tk, tv, 0.1, tm) == fa.KERNEL_DECODE_SPLITKV
     out = tq.flash_attention(tk, tv, D ** -0.5, tm).to_numpy()
     assert_parity(out, ref, _tol(dtype), f"window as a tensor, G{G} Sq{Sq} D{D}")
-    if Sq * G == (32 if D <= 128 else 16) * (2 if dtype == fa.F32 else 1):
+    if Sq * G == ((64 if D <= 192 else 32) if dtype == fa.F32 else (32 if D <= 128 else 16)):
         q2 = np.concatenate([q, q[:, :, :1]], 2)
         t2 = fa.Tensor.from_numpy(device, q2, dtype)
         assert t2.selected_kernel(tk, tv, 0.1, analytic=(True, Skv - Sq - 1, 0)) != fa.KERNEL_DECODE_SPLITKV
