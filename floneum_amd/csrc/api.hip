@@ -285,8 +285,9 @@ static void decode_visible_range(const fhip_attn_args *a, int *lo0, int *len) {
 // partial results go in the workspace: behind the mask scratch, 256-byte aligned.
 static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
     const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
-    prefill_f32_plan((int)a->q.shape[0], (int)a->q.shape[1], (int)a->q.shape[2], (int)a->k.shape[2], (int)a->q.shape[3],
-                     causal_square, cus > 0 ? cus : 256, nsplit, chunk);
+    const int Hkv = (int)a->k.shape[1];
+    prefill_f32_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
+                     (int)a->k.shape[2], (int)a->q.shape[3], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
 }
 static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratch_bytes(a) + 255) & ~(size_t)255; }
 static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {

@@ -517,21 +517,27 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     const int hf = wave & 1;   // which half of the dims
     const int d0 = PFW_DH * hf;
 
-    const int bh_count = p.B * p.H;
+    // Packed form (at most 32 query rows, an even GQA group): the two pairs hold rows 0..31 of two query heads that share
+    // a KV head, so both work on every tile the workgroup moves (with one head per workgroup the second pair has no
+    // rows) and a few new rows on a long cache need half the workgroups.
+    const int pack = p.pf_pack;
+    const int heads = pack ? p.H / 2 : p.H;  // head units per batch entry
+    const int bh_count = p.B * heads;
     const int nks = max(p.pf_nsplit, 1);
     const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
     const int id = snake_order(blockIdx.x / nks, gridDim.x / nks, p.snake_cus);
     const int qb = nqb - 1 - id / bh_count;
     int rem = id % bh_count;
-    const int b = rem / p.H;
-    int h = rem % p.H;
-    if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
+    const int b = rem / heads;
+    int h = rem % heads;
+    if (pack) h = 2 * h + pr;
+    else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
 
-    const int q0 = qb * BM;
-    const int qw0 = q0 + 32 * pr;
+    const int q0 = pack ? 0 : qb * BM;
+    const int qw0 = pack ? 0 : q0 + 32 * pr;
     const int query = qw0 + ln;
-    RowBounds rb = row_bounds(p, b, q0, BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, pack ? 32 : BM, qw0, lane);
     if (nks > 1) {  // this workgroup's share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
@@ -699,14 +705,19 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
 template <typename T>
 static int launch_merge_t(const AttnParams &p, hipStream_t stream);
 
+// query heads that share one workgroup of the wide-head kernel (0: one head, up to 64 rows)
+static int prefill_f32_wide_pack(int G, int Sq, int D) { return (D > 128 && Sq <= 32 && G >= 2 && G % 2 == 0) ? 2 : 0; }
+
 template <typename T>
-static int launch_wide(const AttnParams &p, hipStream_t stream) {
-    if (p.mask && !p.iv) {
+static int launch_wide(const AttnParams &p_in, hipStream_t stream) {
+    if (p_in.mask && !p_in.iv) {
         set_error("prefill f32: a mask tensor without its interval form is not supported above head_dim 128");
         return FHIP_ERR_UNSUPPORTED;
     }
-    const int nqb = (p.Sq + 63) / 64;
-    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
+    AttnParams p = p_in;
+    p.pf_pack = prefill_f32_wide_pack(p.G, p.Sq, p.D);
+    const int nqb = p.pf_pack ? 1 : (p.Sq + 63) / 64;
+    const long blocks = (long)nqb * p.B * (p.pf_pack ? p.H / 2 : p.H) * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill f32: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -764,15 +775,21 @@ static int launch_split(const AttnParams &p, hipStream_t stream) {
 // most CUs idle, so the keys are split over workgroups as well, down to 512 keys per share, until there are about
 // two workgroups per CU.  Square causal calls are left alone (their shares would be uneven, and they fill the
 // chip from 1024 rows on).
-void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk) {
+void prefill_f32_plan(int B, int H, int G, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk) {
     *nsplit = 1;
     *chunk = Skv;
     if (causal_square) return;
     const int bm = D > 128 ? 64 : 32;  // the finest query blocking the kernel has
-    const long wgs = (long)B * H * ((Sq + bm - 1) / bm);
+    const int pack = prefill_f32_wide_pack(G, Sq, D);
+    const long wgs = pack ? (long)B * (H / 2) : (long)B * H * ((Sq + bm - 1) / bm);
     if (wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy (two workgroups per CU)
     const long want = (2L * compute_units + wgs - 1) / wgs;
-    const long most = Skv / 512;
+    // Shares of at least 512 keys (256 in the packed form, which has half the workgroups).  The wide-head kernel takes
+    // ~7 us per 32-key tile when a workgroup is alone on its CU, most of it waiting for the tile's rows: it goes down to
+    // 128 keys while longer shares leave CUs without a workgroup (B1 x 2048 keys, 9 rows: 55 -> 36 us; shorter shares
+    // than needed merge too often: B1 x 8192 keys, 32 rows: 84 us with 256 shares of 8 tiles, 101 us with 512 of 4)
+    long most = Skv / (pack ? 256 : 512);
+    if (D > 128 && (want < most ? want : most) * wgs < compute_units) most = Skv / 128;
     long ns = want < most ? want : most;
     if (ns < 2) return;
     long c = (Skv + ns - 1) / ns;

@@ -56,11 +56,11 @@ struct AttnParams {
     // and parks (O unnormalised, m, l) per row in `partials` [B, H, Sq, pf_nsplit, pf_pitch]; a merge kernel follows.
     int32_t pf_nsplit, pf_chunk;
     int32_t pf_pitch;  // floats per (row, share) in `partials`: D + 2, or D + 4 where rows are written in 16-byte pieces
-    int32_t pf_pack;   // 16-bit tiled kernel, set by its launcher: query heads per workgroup of the packed form, or 0
+    int32_t pf_pack;   // tiled kernels, set by their launchers: query heads per workgroup of the packed form, or 0
 };
 
 // the key split of a tiled f32 prefill call (1 = none) and the scratch it needs
-void prefill_f32_plan(int B, int H, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk);
+void prefill_f32_plan(int B, int H, int G, int Sq, int Skv, int D, bool causal_square, int compute_units, int *nsplit, int *chunk);
 size_t prefill_f32_workspace_bytes(int B, int H, int Sq, int D, int nsplit);
 // the same for the 16-bit matrix-core prefill kernel (256-row query blocks, one workgroup per CU)
 void prefill_mfma_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk);

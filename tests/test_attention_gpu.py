@@ -719,6 +719,47 @@ def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
     assert_parity(out_t.to_numpy(), ref, tol, f"unsplit, {case} D{D}")
 
 
+@pytest.mark.parametrize("dtype,D,G,Sq", [(fa.F32, 256, 4, 20), (fa.F32, 256, 2, 32), (fa.F32, 160, 4, 17), (fa.F32, 200, 6, 17),
+                                          (fa.F16, 144, 2, 30), (fa.F32, 256, 3, 20)])
+@pytest.mark.parametrize("case", ["causal_offset", "window", "mask_tensor", "kv_lens", "full"])
+def test_few_rows_above_head_dim_128_in_f32_arithmetic_pair_two_heads(device, dtype, D, G, Sq, case):
+    """Up to 32 new rows on a long cache above head_dim 128 on the f32-arithmetic kernel (Gemma-3's key length in the
+    type kalosm-llama calls with): with an even GQA group the workgroup's two wavefront pairs hold the rows of two query
+    heads of one KV head and share its K/V tiles; with an odd group (the last case) one head per workgroup as before.
+    With the workspace the library asks for (keys split over workgroups) and without any."""
+    B, Hkv, Skv = 2, 2, 3000
+    H = Hkv * G
+    q, k, v = _normal_qkv(19, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    mask, kind, analytic, mt, lens_t = None, None, None, None, None
+    if case == "causal_offset":
+        analytic = (True, Skv - Sq, 0)
+    elif case == "window":
+        analytic = (True, Skv - Sq, 1000)
+    elif case == "mask_tensor":
+        mask, kind = oracle.get_mask(Sq, Skv - Sq), "qk"
+        mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+    elif case == "kv_lens":
+        lens = np.array([2222, 77], np.int32)
+        lens_t = fa.IntTensor(device, lens)
+        mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+        mask[0, 2222:] = NEG_INF
+        mask[1, 77:] = NEG_INF
+    if analytic is not None:
+        mask, kind = _analytic_mask(Sq, Skv, *analytic), "qk"
+    if mt is None:
+        assert tq.selected_kernel(tk, tv, 0.1, analytic=analytic, kv_lens=lens_t) == fa.KERNEL_PREFILL_F32
+    out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic, kv_lens=lens_t).to_numpy()
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                 None if mask is None else rounded(mask, dtype), kind)
+    tol = TOL_F32 if dtype == fa.F32 else TOL_16
+    assert_parity(out, ref, tol, f"split keys, {case} D{D} G{G} Sq{Sq}")
+    out_t = fa.Tensor.empty(device, (B, Sq, H, D), dtype)  # written as [B, Sq, H, D], no workspace
+    args = tq._attn_args(tk, tv, D ** -0.5, mt, analytic, lens_t, None, fa.KERNEL_AUTO, out_t.transpose(1, 2))
+    fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+    assert_parity(out_t.to_numpy().transpose(0, 2, 1, 3), ref, tol, f"unsplit, {case} D{D} G{G} Sq{Sq}")
+
+
 @pytest.mark.parametrize("dtype,D,Sq", [(fa.F16, 96, 1), (fa.BF16, 128, 1), (fa.F16, 64, 2), (fa.F16, 32, 1)])
 def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype, D, Sq):
     """At least one (batch, kv head) unit per CU and more than 2048 keys: the 16-bit matrix-core variant runs with eight
