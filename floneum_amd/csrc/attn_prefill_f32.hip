@@ -784,12 +784,18 @@ void prefill_f32_plan(int B, int H, int G, int Sq, int Skv, int D, bool causal_s
     const long wgs = pack ? (long)B * (H / 2) : (long)B * H * ((Sq + bm - 1) / bm);
     if (wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy (two workgroups per CU)
     const long want = (2L * compute_units + wgs - 1) / wgs;
-    // Shares of at least 512 keys (256 in the packed form, which has half the workgroups).  The wide-head kernel takes
-    // ~7 us per 32-key tile when a workgroup is alone on its CU, most of it waiting for the tile's rows: it goes down to
-    // 128 keys while longer shares leave CUs without a workgroup (B1 x 2048 keys, 9 rows: 55 -> 36 us; shorter shares
-    // than needed merge too often: B1 x 8192 keys, 32 rows: 84 us with 256 shares of 8 tiles, 101 us with 512 of 4)
+    // Shares of at least 512 keys (256 in the packed form, which has half the workgroups); while that leaves CUs without
+    // a workgroup, down to 256 and then 128 keys: a workgroup alone on its CU spends most of a tile waiting for the
+    // tile's rows (~7 us per 32-key tile in the wide-head kernel, ~2 us below), so more, shorter workgroups win until
+    // the chip is full (f32, B1: head_dim 256, 2048 keys, 9 rows 55 -> 36 us; head_dim 128, 2048 keys, 20 rows 34 -> 26,
+    // 1024 keys 33 -> 21).  Shorter shares than needed merge too often (head_dim 256, B1 x 8192 keys, 32 rows: 84 us with
+    // 256 shares of 8 tiles, 101 us with 512 of 4).
     long most = Skv / (pack ? 256 : 512);
-    if (D > 128 && (want < most ? want : most) * wgs < compute_units) most = Skv / 128;
+    // (only for calls that are clearly a few rows on a longer cache: a square prompt masked by a tensor keeps the plan
+    // of its analytic twin, and with it the same bits)
+    const bool few_rows = 2L * Sq <= Skv;
+    if (few_rows && (want < most ? want : most) * wgs < compute_units) most = Skv / 256;
+    if (few_rows && (want < most ? want : most) * wgs < compute_units) most = Skv / 128;
     long ns = want < most ? want : most;
     if (ns < 2) return;
     long c = (Skv + ns - 1) / ns;
