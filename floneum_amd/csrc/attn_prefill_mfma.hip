@@ -777,7 +777,13 @@ void prefill_mfma_plan(int B, int H, int G, int Sq, int Skv, bool causal_square,
     if (2 * wgs > compute_units) return;  // the query blocks alone keep at least half the chip busy: parking and
                                           // merging partial results would cost more than it gains (measured)
     const long want = (2L * compute_units + wgs - 1) / wgs;
-    const long most = Skv / 1024;
+    long most = Skv / 1024;
+    // A few rows on a short cache: shares down to 512 keys, and for up to 64 rows to 256, while CUs would stay without a
+    // workgroup (f16, 32/8 heads, head_dim 128, B1: 12...32 rows on 2048 keys 24.6 -> 17.8 us, on 4096 keys 24.7 -> 20.7;
+    // 128 rows on 2048 keys 28.8 -> 25.7).  On 1024 keys two shares of 512 lose with more than 64 rows (21.2 -> 23.4 us).
+    const bool few_rows = 2L * Sq <= Skv && (Sq <= 64 || Skv >= 2048);
+    if (few_rows && (want < most ? want : most) * wgs < compute_units) most = Skv / 512;
+    if (few_rows && Sq <= 64 && (want < most ? want : most) * wgs < compute_units) most = Skv / 256;
     long ns = want < most ? want : most;
     if (ns < 2) return;
     long c = (Skv + ns - 1) / ns;
