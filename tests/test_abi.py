@@ -232,12 +232,12 @@ def test_prefill_key_split_planning_on_256_cus():
     need = ctypes.c_size_t()
     L = fa.lib()
 
-    def shares(Sq, Skv, dtype, pitch, analytic=True):
-        a = make_args(B=1, H=32, Hkv=8, Sq=Sq, Skv=Skv, D=128, dtype=dtype)
+    def shares(Sq, Skv, dtype, pitch, analytic=True, D=128, H=32, Hkv=8):
+        a = make_args(B=1, H=H, Hkv=Hkv, Sq=Sq, Skv=Skv, D=D, dtype=dtype)
         if analytic:
             a.analytic.enabled, a.analytic.causal, a.analytic.q_pos_offset = 1, 1, Skv - Sq
         assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
-        per = 32 * Sq * pitch * 4
+        per = H * Sq * pitch * 4
         assert need.value % per == 0
         return need.value // per
 
@@ -246,6 +246,17 @@ def test_prefill_key_split_planning_on_256_cus():
     assert shares(32, 32768, fa.F16, 132) == 32   # packed: 8 head quads x 32 shares of 1024 keys (unpacked it was 32 heads x 16)
     assert shares(512, 512, fa.F32, 130) == 0     # square causal prompts are left alone
     assert shares(2048, 2048, fa.F16, 132) == 0
+    # a few rows on a short cache: shorter shares while CUs would stay without a workgroup
+    assert shares(20, 2048, fa.F16, 132) == 8     # 256 keys (up to 64 rows)
+    assert shares(128, 2048, fa.F16, 132) == 4    # 512 keys
+    assert shares(128, 1024, fa.F16, 132) == 0    # two shares of 512 keys lose there
+    assert shares(20, 2048, fa.F32, 130) == 8     # 256 keys fill the chip (64 thirty-two-row workgroups x 8)
+    assert shares(20, 1024, fa.F32, 130) == 8     # 128 keys
+    # head_dim 256: two query heads per workgroup in f32 arithmetic (8 workgroups before the split)
+    assert shares(20, 2048, fa.F32, 258, D=256, H=16, Hkv=4) == 16   # 128 keys
+    assert shares(48, 8192, fa.F32, 258, D=256, H=16, Hkv=4) == 16   # unpacked above 32 rows: 512 keys
+    assert shares(20, 8192, fa.F16, 260, D=256, H=16, Hkv=4) == 8    # the wide-head 16-bit kernel, four heads per workgroup
+    assert shares(64, 8192, fa.F16, 260, D=256, H=16, Hkv=4) == 8    # 64-row workgroups, two per CU
 
 
 # ---- masks: bit-exact against the checker and the reference's vectors -----------------------------------
