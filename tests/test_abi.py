@@ -250,7 +250,7 @@ def test_prefill_key_split_planning_on_256_cus():
     assert shares(20, 2048, fa.F16, 132) == 8     # 256 keys (up to 64 rows)
     assert shares(128, 2048, fa.F16, 132) == 4    # 512 keys
     assert shares(128, 1024, fa.F16, 132) == 0    # two shares of 512 keys lose there
-    assert shares(20, 2048, fa.F32, 130) == 8     # 256 keys fill the chip (64 thirty-two-row workgroups x 8)
+    assert shares(20, 2048, fa.F32, 130) == 8     # 256 keys fill the chip (32 thirty-two-row workgroups x 8)
     assert shares(20, 1024, fa.F32, 130) == 8     # 128 keys
     # head_dim 256: two query heads per workgroup in f32 arithmetic (8 workgroups before the split)
     assert shares(20, 2048, fa.F32, 258, D=256, H=16, Hkv=4) == 16   # 128 keys
