@@ -221,11 +221,9 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     const bool wide = D == 160 || D == 192 || D == 224 || D == 256;  // attn_prefill_mfma_wide.hip
     if (!(D == 64 || D == 96 || D == 128 || wide)) return false;
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
-    // scales in f32; 64-bit tile addresses, 32-bit byte offsets inside a 32-key tile
-    if (wide) return a->k.stride[2] >= 0 && a->v.stride[2] >= 0 && a->k.stride[2] < (1 << 25) && a->v.stride[2] < (1 << 25);
-    // the kernel folds scale * log2(e) into Q (rounded back to the input type): the factor must not
-    // be able to push a finite element out of range
-    if (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f)) return false;
+    // the kernel for 64 / 96 / 128 folds scale * log2(e) into Q (rounded back to the input type): the factor must not
+    // be able to push a finite element out of range (the wide-head kernel scales the scores in f32)
+    if (!wide && (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f))) return false;
     // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv
     // head) slice must span less than 2 GiB
     const uint64_t Skv = a->k.shape[2];

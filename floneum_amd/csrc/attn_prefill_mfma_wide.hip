@@ -2,13 +2,13 @@
 // matrix cores.
 //
 // The 256-row kernel of attn_prefill_mfma.hip keeps Q and O^T of 32 rows in a wavefront's registers with two wavefronts
-// per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is four wavefronts,
-// one per SIMD with the whole register file, and 128 query rows of one (batch, head); the keys are walked in tiles of 32
-// that all four wavefronts share through a double-buffered LDS tile (global -> registers -> LDS, the next tile's loads
-// in flight during the math).  (Head dims below 256 run as eight wavefronts of 16 rows instead, see wide_waves.)  Per tile and
-// wavefront, on v_mfma_f32_16x16x32 with the 32 query rows as two blocks of 16 columns (the arithmetic of the split-KV
-// decode kernel with two column blocks, attn_decode.hip):
-//   S^T[key][row]  = K . Q^T     A = K from LDS (one 16-byte read feeds both column blocks), B = Q in registers
+// per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is eight wavefronts
+// of 16 query rows, two per SIMD, and 128 query rows of one (batch, head) (four wavefronts of 16 rows and 64 query rows,
+// two workgroups per CU, on small grids); the keys are walked in tiles of 32 that all wavefronts share through LDS,
+// loaded straight into it (no staging registers) with the next two tiles on their way during the math.  Per tile and
+// wavefront, on v_mfma_f32_16x16x32 with the query rows as blocks of 16 columns (the arithmetic of the split-KV decode
+// kernel, attn_decode.hip; the template also holds a form with two column blocks per wavefront):
+//   S^T[key][row]  = K . Q^T     A = K from LDS (one 16-byte read feeds every column block), B = Q in registers
 //   scores scaled in f32 (scale * log2 e), masked by the row's visible interval, online softmax per column
 //   O^T[dim][row] += V^T . P^T   A = V^T from row-major LDS with ds_read_b64_tr_b16, B = the probabilities
 // Masks: the analytic descriptor, key counts, or the interval form of a mask tensor (attn_bounds.h); a mask tensor that
@@ -84,14 +84,16 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     constexpr int VP = D * 2 + 32;           // V tile row pitch (bytes): rows 8 banks apart
     constexpr int K_BYTES = PW_KEYS * KP;
     constexpr int V_BYTES = PW_KEYS * VP;
-    constexpr int STAGE = K_BYTES + V_BYTES;
-    constexpr int CPR = D / 8;               // 16-byte chunks per row
-    constexpr int CHUNKS = PW_KEYS * CPR;    // per tensor and tile
-    constexpr int NLD = (2 * CHUNKS + 64 * PW_WAVES - 1) / (64 * PW_WAVES);  // 16-byte pieces per thread and tile (K and V together)
+    // a tile is filled 1 KB at a time (see the tile movement below): each tensor's region is whole pieces
+    constexpr int NIK = (K_BYTES + 1023) / 1024, NIV = (V_BYTES + 1023) / 1024;
+    constexpr int V_AT = NIK * 1024;                  // where the V tile starts in a stage
+    constexpr int STAGE = (NIK + NIV) * 1024;
     constexpr int KB = D / 32;               // contraction blocks of K . Q^T
     constexpr int NB = D / 16;               // 16-dim blocks of the output
     constexpr int BM = 16 * CB * PW_WAVES;   // query rows per workgroup (CB 16-column blocks per wavefront)
-    __shared__ __attribute__((aligned(16))) char smem[2 * STAGE];
+    // tiles in LDS: the one in use and the next two on their way; the two-per-CU form has room for one on its way only
+    constexpr int NSTAGE = PW_WAVES * CB == 8 ? 3 : 2;
+    __shared__ __attribute__((aligned(16))) char smem[NSTAGE * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
     if (p.iv_bad && *p.iv_bad == p.bad_tag) return;  // the mask is not made of intervals: the kernel behind takes the call
@@ -149,81 +151,72 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     const uint16_t *vbase = (const uint16_t *)p.v + b * p.vs[0] + g * p.vs[1];
     const float scale2 = p.scale * PW_LOG2E;
 
-    // tile movement: every thread takes NLD 16-byte chunks of K and of V; rows beyond the key axis repeat the last row
-    // (their scores are masked by the rows' intervals, which end at the key count)
-    // The K and the V tile are one list of 2 * CHUNKS 16-byte pieces, dealt to the threads NLD at a time (with 160 and
-    // 224 one of a thread's pieces is of K in half the threads and of V in the others; with eight wavefronts at those
-    // head dims the last round of pieces goes to the first four wavefronts only, a whole-wavefront condition).  A piece
-    // sits at a fixed byte offset from its tile's first key (the host admits row strides below 2^25 elements only, so
-    // it fits 32 bits); the tiles' own addresses are the same in every lane.
-    constexpr int LAST_ROUND = 2 * CHUNKS - 64 * PW_WAVES * (NLD - 1);  // pieces of the last round
-    static_assert(LAST_ROUND % 64 == 0 && LAST_ROUND > 0, "whole wavefronts in the last round");
-    auto has_piece = [&](int u) __attribute__((always_inline)) -> bool {
-        return LAST_ROUND == 64 * PW_WAVES || u < NLD - 1 || wave < LAST_ROUND / 64;
+    // ---- tile movement: global -> LDS directly, no staging registers ---------------------------------------------------
+    // A direct load writes the 64 lanes' 16 bytes to 1 KB of consecutive LDS, wherever each lane reads from.  The K tile
+    // (rows of 2 D bytes at pitch KP) and the V tile (pitch VP) are therefore filled 1 KB at a time: piece i of a tile
+    // covers its bytes [1024 i, 1024 i + 1024), lane l of it the 16 bytes at 1024 i + 16 l, which belong to row
+    // pos / pitch, byte pos % pitch of the row; lanes that fall into the padding between rows or behind the last row
+    // (each tensor's region is a whole number of pieces) fetch from beyond the buffer, i.e. zeros.  The NIK + NIV pieces of a tile pair are dealt round robin to the wavefronts.  K and V are raw buffers of
+    // (Skv - 1) rows + 2 D bytes: a row beyond the key axis reads as zero (its scores are masked by the rows' intervals,
+    // which end at the key count), so no clamps and no 64-bit address arithmetic in the loop.
+    constexpr int NJ = (NIK + NIV + PW_WAVES - 1) / PW_WAVES;  // pieces per wavefront and tile pair
+    const int krow_bytes = (int)p.ks[2] * 2, vrow_bytes = (int)p.vs[2] * 2;
+    auto descriptor = [&](const uint16_t *base, int row_bytes) __attribute__((always_inline)) {
+        const uint64_t ptr = (uint64_t)base;
+        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((p.Skv - 1) * row_bytes + D * 2),
+                       0x00020000u};
     };
-    uint4_t st[NLD];  // the tile in flight from HBM
-    // With 32 pieces per row (head dim 256) a thread's pieces are the same column of every eighth row: two offsets
-    // and constant steps describe them all, which the full register file of this head dim needs.
-    constexpr bool AFFINE = (64 * PW_WAVES) % CPR == 0;
-    constexpr int RSTEP = 64 * PW_WAVES / CPR;  // AFFINE: rows between a thread's consecutive pieces
-    uint32_t goff_[AFFINE ? 2 : NLD], loff_[AFFINE ? 2 : NLD];
-    if constexpr (AFFINE) {
-        const int r = tid / CPR, c = tid % CPR;
-        goff_[0] = (r * (uint32_t)p.ks[2] + c * 8) * 2;
-        goff_[1] = (r * (uint32_t)p.vs[2] + c * 8) * 2;
-        loff_[0] = r * KP + c * 16;
-        loff_[1] = K_BYTES + r * VP + c * 16;
-    } else {
+    const uint4_t krs = descriptor(kbase, krow_bytes), vrs = descriptor(vbase, vrow_bytes);
+    int piece_voff[NJ];   // this lane's byte offset from the tile's first key (beyond the buffer for a lane without data)
+    int piece_lds[NJ];    // where the piece starts in a stage (the same in every lane)
 #pragma unroll
-        for (int u = 0; u < NLD; u++) {
-            const int cid = tid + 64 * PW_WAVES * u;
-            const bool is_v = cid >= CHUNKS;
-            const int r = (is_v ? cid - CHUNKS : cid) / CPR, c = (is_v ? cid - CHUNKS : cid) % CPR;
-            goff_[u] = (r * (uint32_t)(is_v ? p.vs[2] : p.ks[2]) + c * 8) * 2;
-            loff_[u] = is_v ? K_BYTES + r * VP + c * 16 : r * KP + c * 16;
-        }
+    for (int jj = 0; jj < NJ; jj++) {
+        // (a wavefront whose share of the list is one short repeats the list's last piece: the same bytes to the same
+        // place, and every wavefront then has exactly NJ loads per tile in flight, which the wait below counts on)
+        const int idx = min(wave + PW_WAVES * jj, NIK + NIV - 1);
+        const bool is_k = idx < NIK;
+        const int i = is_k ? idx : idx - NIK;
+        const int pos = 1024 * i + 16 * lane;
+        const int pitch = is_k ? KP : VP, bytes = is_k ? K_BYTES : V_BYTES;
+        const int r = pos / pitch, cbyte = pos % pitch;
+        const bool active = pos < bytes && cbyte < 2 * D;
+        piece_voff[jj] = active ? r * (is_k ? krow_bytes : vrow_bytes) + cbyte : 0x7ffffff0;
+        piece_lds[jj] = (is_k ? 0 : V_AT) + 1024 * i;
     }
-    const uint32_t kstep = RSTEP * (uint32_t)p.ks[2] * 2, vstep = RSTEP * (uint32_t)p.vs[2] * 2;
-    auto goff = [&](int u) __attribute__((always_inline)) -> uint32_t {
-        if constexpr (AFFINE) return u < NLD / 2 ? goff_[0] + u * kstep : goff_[1] + (u - NLD / 2) * vstep;
-        else return goff_[u];
-    };
-    auto loff = [&](int u) __attribute__((always_inline)) -> uint32_t {
-        if constexpr (AFFINE)
-            return u < NLD / 2 ? loff_[0] + u * RSTEP * KP : loff_[1] + (u - NLD / 2) * RSTEP * VP;
-        else return loff_[u];
-    };
-    auto load_tile = [&](int j0) __attribute__((always_inline)) {
-        const char *kt = (const char *)(kbase + (int64_t)j0 * p.ks[2]);
-        const char *vt = (const char *)(vbase + (int64_t)j0 * p.vs[2]);
-        if (j0 + PW_KEYS <= p.Skv) {
+    auto issue_tile = [&](int j0, int stage_base) __attribute__((always_inline)) {
+        // (uniform values; pinned to scalar registers, which is what the instruction takes.  A tile that starts beyond the
+        // key axis is never used: the offset is clamped so that it stays inside 32 bits.)
+        const int key0 = min(j0, p.Skv);
+        const int lbase = (int)(uint32_t)(uintptr_t)lds_base + stage_base;
 #pragma unroll
-            for (int u = 0; u < NLD; u++) {
-                const bool is_v = tid + 64 * PW_WAVES * u >= CHUNKS;  // known at compile time except for the mixed piece
-                if (has_piece(u)) st[u] = *(const uint4_t *)((is_v ? vt : kt) + goff(u));
-            }
-            return;
-        }
-        // the last tile of a cache whose length is no multiple of the tile: rows past the end repeat the last key
-        const int last = p.Skv - 1 - j0;
-#pragma unroll
-        for (int u = 0; u < NLD; u++) {
-            const int cid = tid + 64 * PW_WAVES * u;
-            const bool is_v = cid >= CHUNKS;
-            const int r = (is_v ? cid - CHUNKS : cid) / CPR, c = (is_v ? cid - CHUNKS : cid) % CPR;
-            const int64_t row_stride = is_v ? p.vs[2] : p.ks[2];
-            if (has_piece(u)) st[u] = *(const uint4_t *)((is_v ? vt : kt) + (min(r, last) * row_stride + c * 8) * 2);
+        for (int jj = 0; jj < NJ; jj++) {
+            const bool is_k = min(wave + PW_WAVES * jj, NIK + NIV - 1) < NIK;  // the same for the whole wavefront
+            const uint4_t rs = is_k ? krs : vrs;
+            const int soff = __builtin_amdgcn_readfirstlane(key0 * (is_k ? krow_bytes : vrow_bytes));
+            const int m0 = __builtin_amdgcn_readfirstlane(lbase + piece_lds[jj]);
+            // written as assembly on purpose: the compiler would otherwise make every later LDS read of this wavefront
+            // wait for these loads, whose data is not due before the next barrier
+            // (no branch around it for the lanes without data: every wavefront must have the same number of loads in
+            // flight per tile, which the waits count on)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                             :
+                             : "s"(m0), "v"(piece_voff[jj]), "s"(rs), "s"(soff)
+                             : "memory", "m0");
         }
     };
-    auto store_tile = [&](int stage_base) __attribute__((always_inline)) {
-#pragma unroll
-        for (int u = 0; u < NLD; u++)
-            if (has_piece(u)) *PWLDS_PTR(uint4_t, stage_base + loff(u)) = st[u];
+    // all direct loads of this wavefront have landed but those of the `newer` most recent tiles (NJ loads each; lanes
+    // without a piece are masked off, the instruction is still issued and counted)
+    auto wait_tiles = [&](int newer) __attribute__((always_inline)) {
+        static_assert(2 * NJ <= 63, "vmcnt");
+        if (newer == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else if (newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NJ) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NJ) : "memory");
     };
 
     const int j_begin = (lo_wg / PW_KEYS) * PW_KEYS;
     const int ntiles = hi_wg > j_begin ? (hi_wg - j_begin + PW_KEYS - 1) / PW_KEYS : 0;
-    if (ntiles > 0) load_tile(j_begin);  // issued first so the Q fetch below overlaps it
+    if (ntiles > 0) issue_tile(j_begin, 0);  // issued first so the Q fetch below overlaps them
+    if (NSTAGE > 2 && ntiles > 1) issue_tile(j_begin + PW_KEYS, STAGE);
 
     // Q^T operand: column j of block cb, dims 32 kb + 8 q4 .. +8 (rows beyond Sq repeat the last row; never stored)
     vec8 qreg[CB][KB];
@@ -257,10 +250,11 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     // which costs more than the few such tiles on the diagonal of a causal mask.)
     auto tile_front = [&](int t) __attribute__((always_inline)) -> bool {  // true: move the reference first
         const int j0 = j_begin + t * PW_KEYS;
-        sbase = (t & 1) * STAGE;
-        store_tile(sbase);
-        __syncthreads();  // tile t is in LDS; every wavefront is done with tile t - 1, whose stage the next store takes
-        if (t + 1 < ntiles) load_tile(j0 + PW_KEYS);
+        sbase = (t % NSTAGE) * STAGE;
+        // tile t has landed: all of this wavefront's loads but those of the tiles issued after it
+        wait_tiles(min(ntiles - 1 - t, NSTAGE - 2));
+        __syncthreads();  // tile t is in LDS; every wavefront is done with tile t - 1, whose stage the next issue takes
+        if (t + NSTAGE - 1 < ntiles) issue_tile(j0 + (NSTAGE - 1) * PW_KEYS, ((t + NSTAGE - 1) % NSTAGE) * STAGE);
         const bool all_visible = j0 >= full_lo_w && j0 + PW_KEYS <= full_hi_w;  // no element test needed
 
         // S^T[key][col] = K . Q^T : two 16-key halves, every K operand read serves both column blocks
@@ -342,9 +336,9 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
             const short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                PWLDS_PTR(short4_t, sbase + K_BYTES + trow * VP + nb * 32 + tcol));
+                PWLDS_PTR(short4_t, sbase + V_AT + trow * VP + nb * 32 + tcol));
             const short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                PWLDS_PTR(short4_t, sbase + K_BYTES + (16 + trow) * VP + nb * 32 + tcol));
+                PWLDS_PTR(short4_t, sbase + V_AT + (16 + trow) * VP + nb * 32 + tcol));
             const uint2w_t u0 = __builtin_bit_cast(uint2w_t, a0), u1 = __builtin_bit_cast(uint2w_t, a1);
             const uint4_t araw = {u0[0], u0[1], u1[0], u1[1]};
 #pragma unroll
@@ -392,11 +386,13 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     }
 }
 
-// Wavefronts per workgroup.  Eight wavefronts of 16 rows (two per SIMD, half the register file each) hide each other's
-// dependent phases but read every K and V operand from LDS for half as many matrix instructions: measured (f16,
-// 4096 x 4096 causal) +15 % at head_dim 160, +16 % at 192, +6 % at 224 and -5 % at 256, where the eight-wavefront form
-// leaves 7 of its 256 registers free.
-constexpr int wide_waves(int d) { return d == 256 ? 4 : 8; }
+// Wavefronts per workgroup: eight wavefronts of 16 rows (two per SIMD, half the register file each), which hide each
+// other's dependent phases but read every K and V operand from LDS for half as many matrix instructions as four
+// wavefronts of 32 rows would.  Measured (f16, 4096 x 4096 causal) while the tiles still went through staging registers:
+// +15 % at head_dim 160, +16 % at 192, +6 % at 224 and -5 % at 256 (249 of 256 registers); with the tiles loaded
+// straight into LDS (218 registers at 256) eight are ahead there too, 535 against 501 TFLOP/s.  The four-wavefront
+// form <4, 2> is kept in the template for such measurements.
+constexpr int wide_waves(int) { return 8; }
 
 template <typename T, int D>
 void launch_wide_d(const AttnParams &p, int bm, const dim3 &grid, int nqb, hipStream_t stream) {
