@@ -824,6 +824,34 @@ def test_wide_head_dims_on_a_grid_that_fills_the_chip(device, dtype, D, case):
         assert_parity(out[b:b + 1], ref, tol, f"D{D} {case}, sequence {b}")
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
+@pytest.mark.parametrize("D", [64, 128, 160, 256])
+def test_memory_behind_a_cache_view_is_never_used(device, dtype, D):
+    """K and V are views of the first 333 rows of a 512-row cache allocation whose other rows hold NaN.  The tiled kernels
+    fetch whole 32- or 64-key tiles; the rows of the last tile that lie beyond the view must not reach the result (the
+    16-bit kernels fetch them through a buffer descriptor that ends with the view and get zeros; a NaN there would
+    survive the masking as 0 x NaN in P . V)."""
+    B, H, Hkv, Sq, Skv, cap = 1, 4, 2, 200, 333, 512
+    rng = np.random.default_rng(12)
+    q = rng.normal(0, 1, (B, H, Sq, D)).astype(np.float32)
+    kbuf = np.full((B, Hkv, cap, D), np.nan, np.float32)
+    vbuf = np.full((B, Hkv, cap, D), np.nan, np.float32)
+    kbuf[:, :, :Skv] = rng.normal(0, 1, (B, Hkv, Skv, D))
+    vbuf[:, :, :Skv] = rng.normal(0, 1, (B, Hkv, Skv, D))
+    tq = fa.Tensor.from_numpy(device, q, dtype)
+    tk = fa.Tensor.from_numpy(device, kbuf, dtype).narrow(2, 0, Skv)
+    tv = fa.Tensor.from_numpy(device, vbuf, dtype).narrow(2, 0, Skv)
+    for analytic in ((True, Skv - Sq, 0), None):
+        kw = {} if analytic is None else {"analytic": analytic}
+        assert tq.selected_kernel(tk, tv, D ** -0.5, **kw) == (fa.KERNEL_PREFILL_F32 if dtype == fa.F32 else fa.KERNEL_PREFILL_MFMA)
+        out = tq.flash_attention(tk, tv, D ** -0.5, **kw).to_numpy()
+        mask = None if analytic is None else _analytic_mask(Sq, Skv, *analytic)
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(kbuf[:, :, :Skv], dtype), rounded(vbuf[:, :, :Skv], dtype),
+                                     D ** -0.5, mask, None if mask is None else "qk")
+        tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+        assert_parity(out, ref, tol, f"D{D}, mask {analytic}")
+
+
 @pytest.mark.parametrize("dtype,tol", [(fa.F16, 2e-3), (fa.BF16, 8e-3)])
 @pytest.mark.parametrize("D", [160, 256])
 @pytest.mark.parametrize("growth", [0.02, 0.3, 3.0, 40.0])
