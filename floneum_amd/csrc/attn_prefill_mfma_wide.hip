@@ -78,7 +78,7 @@ __device__ __forceinline__ float pw_quad_sum(float x) {
 // PW_WAVES wavefronts of 16 * CB query rows: <4, 2> and <8, 1> are one workgroup per CU, <4, 1> (64-row workgroups
 // for grids that would leave CUs idle) two.
 template <typename T, int D, int PW_WAVES, int CB>
-__global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
+__global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
     typedef typename WideMma<T>::vec8 vec8;
     constexpr int KP = D * 2 + 16;           // K tile row pitch (bytes): rows 4 banks apart
     constexpr int VP = D * 2 + 32;           // V tile row pitch (bytes): rows 8 banks apart
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB == 8 ? 1 : 2) void pre
     constexpr int NB = D / 16;               // 16-dim blocks of the output
     constexpr int BM = 16 * CB * PW_WAVES;   // query rows per workgroup (CB 16-column blocks per wavefront)
     // tiles in LDS: the one in use and the next two on their way; the two-per-CU form has room for one on its way only
-    constexpr int NSTAGE = PW_WAVES * CB == 8 ? 3 : 2;
+    constexpr int NSTAGE = PW_WAVES * CB >= 8 ? 3 : 2;
     __shared__ __attribute__((aligned(16))) char smem[NSTAGE * STAGE];
     auto lds_base = (__attribute__((address_space(3))) char *)smem;
 
@@ -398,6 +398,8 @@ template <typename T, int D>
 void launch_wide_d(const AttnParams &p, int bm, const dim3 &grid, int nqb, hipStream_t stream) {
     if (bm == 64) {
         FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, D, 4, 1>), grid, dim3(256), stream, p, p, nqb);
+    } else if (bm == 256) {
+        if constexpr (D <= 192) FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, D, 8, 2>), grid, dim3(512), stream, p, p, nqb);
     } else {
         constexpr int W = wide_waves(D);
         FHIP_LAUNCH_MAIN((prefill_mfma_wide_kernel<T, D, W, 8 / W>), grid, dim3(64 * W), stream, p, p, nqb);
@@ -417,7 +419,17 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // (With the keys split, up to 64 rows are one row block either way: the 64-row form computes half as much per tile
     // and runs two workgroups per CU: f16, head_dim 256, B8 x 16 heads, 64 rows on 8192 keys 271 -> 181 us.)
     const bool small = p.pf_nsplit <= 1 ? wgs128 < 2 * p.cus : p.Sq <= 64;
-    const int bm = (!p.pf_pack && small) ? 64 : PW_BM;
+    int bm = (!p.pf_pack && small) ? 64 : PW_BM;
+    // Up to head_dim 192 a wavefront can hold 32 rows (two column blocks: every K and V operand read from LDS then feeds
+    // two matrix instructions): 256-row workgroups where those still give every CU one (f16, 4096 x 4096 causal:
+    // head_dim 160 497 -> 559 TFLOP/s, 192 450 -> 511; at 224 and 256 the registers do not suffice)
+    const long wgs256 = (long)p.B * p.H * ((p.Sq + 255) / 256);
+#ifdef PW_FORCE_256
+    const bool big = true;
+#else
+    const bool big = wgs256 >= p.cus;
+#endif
+    if (!p.pf_pack && !small && p.pf_nsplit <= 1 && p.D <= 192 && big) bm = 256;
     const int nqb = p.pf_pack ? 1 : (p.Sq + bm - 1) / bm;
     const long blocks = (long)nqb * p.B * (p.pf_pack ? p.H / 4 : p.H) * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {

@@ -795,10 +795,10 @@ def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype,
 @pytest.mark.parametrize("D", [160, 192, 224, 256])
 @pytest.mark.parametrize("case", ["causal", "chunk_window", "ragged"])
 def test_wide_head_dims_on_a_grid_that_fills_the_chip(device, dtype, D, case):
-    """The wide-head kernel has two workgroup shapes: 128 query rows (one workgroup per CU) when those fill the chip
-    twice over or the keys are split, 64 rows (two per CU) otherwise.  The other tests of these head dims are small
-    grids; here 4 x 64 heads x 2 row blocks reach twice the CU count, so the 128-row form runs (its second row block
-    holds two rows)."""
+    """The wide-head kernel has three workgroup shapes: 64 query rows (two workgroups per CU) on small grids, and where
+    128-row workgroups fill the chip twice over 128 rows (head dims 224 and 256; also every split or packed call) or
+    256 rows (32 rows per wavefront, up to head_dim 192).  The other tests of these head dims are small grids; here
+    4 x 64 heads x 130 rows reach twice the CU count in 128-row blocks (the second block holds two rows)."""
     B, H, Hkv, Sq = 4, 64, 16, 130
     assert B * H * ((Sq + 127) // 128) >= 2 * device.compute_units
     Skv = {"causal": 130, "chunk_window": 400, "ragged": 333}[case]
