@@ -75,8 +75,9 @@ __device__ __forceinline__ float pw_quad_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// PW_WAVES wavefronts of 16 * CB query rows: <4, 2> and <8, 1> are one workgroup per CU, <4, 1> (64-row workgroups
-// for grids that would leave CUs idle) two.
+// PW_WAVES wavefronts of 16 * CB query rows.  <8, 1>: 128-row workgroups, one per CU; <8, 2>: 256-row workgroups (up to
+// head_dim 192, where 32 rows fit a wavefront's half of the register file); <4, 1>: 64-row workgroups, two per CU, for
+// grids that would leave CUs idle; <4, 2> (four wavefronts with the whole register file each) is not launched any more.
 template <typename T, int D, int PW_WAVES, int CB>
 __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void prefill_mfma_wide_kernel(AttnParams p, int nqb) {
     typedef typename WideMma<T>::vec8 vec8;
