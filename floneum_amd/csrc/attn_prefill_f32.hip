@@ -131,6 +131,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     int h = rem % p.H;
     if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
+    // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
+    // allocation) are never fetched: what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
+    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
 
     const int q0 = qb * BM;
     const int qw0 = q0 + 32 * wig;
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
         }
         float4_t st[NCH];
         auto load_rows = [&](const T *base, int64_t stride, int j0) __attribute__((always_inline)) {
-            if (AFFINE && whole_rows && j0 + PF32_BN <= p.Skv) {
+            if (AFFINE && whole_rows && j0 + PF32_BN <= key_end) {
                 // a tile inside the key axis with rows as wide as the kernel's: one address per thread, the
                 // chunks a fixed number of rows apart, no clamp and no branch per chunk
                 const T *p0 = base + (int64_t)(j0 + lane / CPR) * stride + (lane % CPR) * 4;
@@ -294,7 +297,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             for (int i = 0; i < NCH; i++) {
                 const int cid = lane + 64 * i;
                 const int row = cid / CPR, col = cid % CPR;
-                const int key = min(j0 + row, p.Skv - 1);
+                const int key = min(j0 + row, key_end - 1);
                 st[i] = col * 4 < p.D ? load4(base + (int64_t)key * stride + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
             }
         };
@@ -321,7 +324,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     } else {
         float4_t kst[NCH], vst[NCH];
         auto load_tile = [&](int j0) {
-            if (AFFINE && whole_rows && j0 + PF32_BN <= p.Skv) {  // see load_rows above
+            if (AFFINE && whole_rows && j0 + PF32_BN <= key_end) {  // see load_rows above
                 const T *pk = kg + (int64_t)(j0 + gtid / CPR) * p.ks[2] + (gtid % CPR) * 4;
                 const T *pv = vg + (int64_t)(j0 + gtid / CPR) * p.vs[2] + (gtid % CPR) * 4;
                 const int64_t kstep = (int64_t)RSTEP * p.ks[2], vstep = (int64_t)RSTEP * p.vs[2];
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
             for (int i = 0; i < NCH; i++) {
                 const int cid = gtid + GT * i;
                 const int row = cid / CPR, col = cid % CPR;
-                const int key = min(j0 + row, p.Skv - 1);
+                const int key = min(j0 + row, key_end - 1);
                 const bool in_row = col * 4 < p.D;  // a head_dim below D is padded with zeros
                 kst[i] = in_row ? load4(kg + (int64_t)key * p.ks[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
                 vst[i] = in_row ? load4(vg + (int64_t)key * p.vs[2] + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
@@ -533,6 +536,9 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     if (pack) h = 2 * h + pr;
     else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
+    // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
+    // allocation) are never fetched: what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
+    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
 
     const int q0 = pack ? 0 : qb * BM;
     const int qw0 = pack ? 0 : q0 + 32 * pr;
@@ -577,7 +583,7 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
         for (int i = 0; i < NCH; i++) {
             const int cid = tid + 64 * PF32_WAVES * i;
             const int row = cid / CPR, col = cid % CPR;
-            const int key = min(j0 + row, p.Skv - 1);
+            const int key = min(j0 + row, key_end - 1);
             st[i] = col * 4 < p.D ? load4(base + (int64_t)key * row_stride + col * 4) : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     };

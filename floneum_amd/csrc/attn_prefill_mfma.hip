@@ -165,6 +165,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     if (pack) h = 4 * h + (wave & 3);
     else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
+    // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
+    // allocation) read as zero (the buffers end there): what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
+    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
 
     const int q0 = pack ? 0 : qb * BM;
     const int qw0 = pack ? 0 : q0 + 32 * (KS ? (wave & 3) : wave);  // KS: both groups own the same 128 rows
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int wv = wave & 3;
     auto descriptor = [&](const uint16_t *base, int row_bytes) __attribute__((always_inline)) {
         const uint64_t ptr = (uint64_t)base;
-        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((p.Skv - 1) * row_bytes + D * 2),
+        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((key_end - 1) * row_bytes + D * 2),
                        0x00020000u};
     };
     const uint4_t krs = descriptor(kg, krow_bytes), vrs = descriptor(vg, vrow_bytes);

@@ -124,6 +124,9 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     if (pack) h = 4 * h + (wave & 3);
     else if ((p.H & 7) == 0) h = (h & 7) * (p.H >> 3) + (h >> 3);
     const int g = h / p.G;
+    // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
+    // allocation) read as zero (the buffers end there): what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
+    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
     const int q0 = pack ? 0 : qb * BM, qw0 = pack ? 16 * CB * (wave >> 2) : q0 + 16 * CB * wave;
 
     // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     const int krow_bytes = (int)p.ks[2] * 2, vrow_bytes = (int)p.vs[2] * 2;
     auto descriptor = [&](const uint16_t *base, int row_bytes) __attribute__((always_inline)) {
         const uint64_t ptr = (uint64_t)base;
-        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((p.Skv - 1) * row_bytes + D * 2),
+        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((key_end - 1) * row_bytes + D * 2),
                        0x00020000u};
     };
     const uint4_t krs = descriptor(kbase, krow_bytes), vrs = descriptor(vbase, vrow_bytes);

@@ -852,6 +852,33 @@ def test_memory_behind_a_cache_view_is_never_used(device, dtype, D):
         assert_parity(out, ref, tol, f"D{D}, mask {analytic}")
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
+@pytest.mark.parametrize("D", [64, 80, 128, 160, 256])
+@pytest.mark.parametrize("Sq", [1, 4, 40, 200])
+def test_rows_beyond_a_sequence_s_own_keys_are_never_used(device, dtype, D, Sq):
+    """A ragged batch in one cache allocation: kv_lens below the view's length, and NaN in the rows between a
+    sequence's own keys and the end of the view (what an uninitialised cache holds there is the caller's business).
+    Decode and prefill kernels fetch whole steps or tiles; none of it may reach the result."""
+    B, H, Hkv, Skv = 2, 4, 2, 700
+    lens = np.array([333, 401], np.int32)
+    rng = np.random.default_rng(13)
+    q = rng.normal(0, 1, (B, H, Sq, D)).astype(np.float32)
+    k = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    v = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    kn, vn = k.copy(), v.copy()
+    for b in range(B):
+        kn[b, :, lens[b]:] = np.nan
+        vn[b, :, lens[b]:] = np.nan
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, kn, vn))
+    out = tq.flash_attention(tk, tv, D ** -0.5, kv_lens=fa.IntTensor(device, lens)).to_numpy()
+    tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+    for b in range(B):
+        n = int(lens[b])
+        ref = oracle.flash_attention(rounded(q[b:b + 1], dtype), rounded(k[b:b + 1, :, :n], dtype),
+                                     rounded(v[b:b + 1, :, :n], dtype), D ** -0.5)
+        assert_parity(out[b:b + 1], ref, tol, f"D{D} Sq{Sq}, sequence {b} of length {n}")
+
+
 @pytest.mark.parametrize("dtype,tol", [(fa.F16, 2e-3), (fa.BF16, 8e-3)])
 @pytest.mark.parametrize("D", [160, 256])
 @pytest.mark.parametrize("growth", [0.02, 0.3, 3.0, 40.0])
