@@ -133,7 +133,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_kernel(AttnPar
     const int g = h / p.G;
     // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
     // allocation) are never fetched: what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
-    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    // (likewise the rows behind the last query's own position when the call says where its rows stand inside a longer
+    // cache view: a causal descriptor with q_pos_offset + Sq below the view's length)
+    int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    if (p.analytic && p.causal) key_end = (int)min((int64_t)key_end, max(p.q_pos_offset + p.Sq, (int64_t)1));
 
     const int q0 = qb * BM;
     const int qw0 = q0 + 32 * wig;
@@ -538,7 +541,10 @@ __global__ __launch_bounds__(64 * PF32_WAVES, 2) void prefill_f32_wide_kernel(At
     const int g = h / p.G;
     // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
     // allocation) are never fetched: what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
-    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    // (likewise the rows behind the last query's own position when the call says where its rows stand inside a longer
+    // cache view: a causal descriptor with q_pos_offset + Sq below the view's length)
+    int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    if (p.analytic && p.causal) key_end = (int)min((int64_t)key_end, max(p.q_pos_offset + p.Sq, (int64_t)1));
 
     const int q0 = pack ? 0 : qb * BM;
     const int qw0 = pack ? 0 : q0 + 32 * pr;

@@ -126,7 +126,10 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     const int g = h / p.G;
     // Rows of a tile beyond the sequence's own keys (kv_lens below the view's length: a ragged batch in one cache
     // allocation) read as zero (the buffers end there): what such rows hold, NaN included, must not reach the result as 0 x NaN in P . V.
-    const int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    // (likewise the rows behind the last query's own position when the call says where its rows stand inside a longer
+    // cache view: a causal descriptor with q_pos_offset + Sq below the view's length)
+    int key_end = p.kv_lens ? min(p.Skv, max(p.kv_lens[b], 1)) : p.Skv;
+    if (p.analytic && p.causal) key_end = (int)min((int64_t)key_end, max(p.q_pos_offset + p.Sq, (int64_t)1));
     const int q0 = pack ? 0 : qb * BM, qw0 = pack ? 16 * CB * (wave >> 2) : q0 + 16 * CB * wave;
 
     // visible keys: of the workgroup's rows (tiles to move), of the wavefront's rows (tiles to compute), of this

@@ -879,6 +879,31 @@ def test_rows_beyond_a_sequence_s_own_keys_are_never_used(device, dtype, D, Sq):
         assert_parity(out[b:b + 1], ref, tol, f"D{D} Sq{Sq}, sequence {b} of length {n}")
 
 
+@pytest.mark.parametrize("dtype", [fa.F16, fa.BF16, fa.F32])
+@pytest.mark.parametrize("D", [64, 80, 128, 160, 256])
+@pytest.mark.parametrize("Sq", [1, 4, 40, 200])
+def test_rows_behind_the_last_query_position_are_never_used(device, dtype, D, Sq):
+    """The view is the whole cache allocation (700 rows), the new rows stand at positions 300 ... inside it (a causal
+    descriptor with q_pos_offset + Sq below the view's length) and the rows behind them hold NaN: causality hides them,
+    and no kernel may fetch them into a tile either."""
+    B, H, Hkv, Skv, pos = 2, 4, 2, 700, 300
+    rng = np.random.default_rng(14)
+    q = rng.normal(0, 1, (B, H, Sq, D)).astype(np.float32)
+    k = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    v = rng.normal(0, 1, (B, Hkv, Skv, D)).astype(np.float32)
+    kn, vn = k.copy(), v.copy()
+    kn[:, :, pos + Sq:] = np.nan
+    vn[:, :, pos + Sq:] = np.nan
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, kn, vn))
+    for window in (0, 100):
+        out = tq.flash_attention(tk, tv, D ** -0.5, analytic=(True, pos, window)).to_numpy()
+        n = pos + Sq
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k[:, :, :n], dtype), rounded(v[:, :, :n], dtype), D ** -0.5,
+                                     _analytic_mask(Sq, n, True, pos, window), "qk")
+        tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=2e-2, rel_l2=1e-2) if dtype == fa.BF16 else TOL_16)
+        assert_parity(out, ref, tol, f"D{D} Sq{Sq} window {window}")
+
+
 @pytest.mark.parametrize("dtype,tol", [(fa.F16, 2e-3), (fa.BF16, 8e-3)])
 @pytest.mark.parametrize("D", [160, 256])
 @pytest.mark.parametrize("growth", [0.02, 0.3, 3.0, 40.0])
