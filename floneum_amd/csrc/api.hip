@@ -218,8 +218,10 @@ static bool decode_eligible(const fhip_attn_args *a) {
 static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     if (a->dtype == FHIP_F32) return false;
     const uint32_t D = a->q.shape[3];
-    const bool wide = D == 160 || D == 192 || D == 224 || D == 256;  // attn_prefill_mfma_wide.hip
-    if (!(D == 64 || D == 96 || D == 128 || wide)) return false;
+    // 64 / 96 / 128: attn_prefill_mfma.hip; every other multiple of 8 up to 256 (padded to the next multiple of 32):
+    // attn_prefill_mfma_wide.hip
+    const bool wide = !(D == 64 || D == 96 || D == 128);
+    if (D % 8 != 0 || D < 8 || D > 256) return false;
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
     // the kernel for 64 / 96 / 128 folds scale * log2(e) into Q (rounded back to the input type): the factor must not
     // be able to push a finite element out of range (the wide-head kernel scales the scores in f32)
@@ -291,7 +293,7 @@ static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratc
 static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
     const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
     const int Hkv = (int)a->k.shape[1];
-    if (a->q.shape[3] > 128)  // the wide-head form: 128-row query blocks
+    if (!(a->q.shape[3] == 64 || a->q.shape[3] == 96 || a->q.shape[3] == 128))  // the wide-head form: 128-row query blocks
         prefill_mfma_wide_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
                                (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
     else
@@ -742,7 +744,7 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
 
 // the 16-bit tiled prefill kernels: 64 / 96 / 128, and the wide-head form above
 static int launch_mfma_by_head_dim(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
-    return p.D > 128 ? launch_prefill_mfma_wide(p, dtype, stream) : launch_prefill_mfma(p, dtype, stream);
+    return (p.D == 64 || p.D == 96 || p.D == 128) ? launch_prefill_mfma(p, dtype, stream) : launch_prefill_mfma_wide(p, dtype, stream);
 }
 
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {

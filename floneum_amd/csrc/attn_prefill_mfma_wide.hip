@@ -1,5 +1,6 @@
 // Prefill attention for f16 / bf16 at head dims 160, 192, 224 and 256 (Gemma-3's key length is 256) on the gfx950
-// matrix cores.
+// matrix cores, and at every other multiple of 8 up to 256 that the 256-row kernel (64 / 96 / 128) does not take: the
+// kernel's D is the head dim rounded up to a multiple of 32, the padding dims read as zero and are not written.
 //
 // The 256-row kernel of attn_prefill_mfma.hip keeps Q and O^T of 32 rows in a wavefront's registers with two wavefronts
 // per SIMD; at these head dims that is 192 registers and more for the two alone.  Here a workgroup is eight wavefronts
@@ -103,6 +104,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     const int lane = tid & 63;
     const int j = lane & 15;   // column inside a block
     const int q4 = lane >> 4;  // key group
+    const int hd = p.D;        // the head dim itself: a multiple of 8, padded with zeros up to the kernel's D
 
     // workgroup -> (share of the keys, query block, batch, head): long (late) query blocks first
     // Packed form (at most 32 query rows, GQA group a multiple of 4; not for the 64-row workgroups): the workgroup's
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     const int krow_bytes = (int)p.ks[2] * 2, vrow_bytes = (int)p.vs[2] * 2;
     auto descriptor = [&](const uint16_t *base, int row_bytes) __attribute__((always_inline)) {
         const uint64_t ptr = (uint64_t)base;
-        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((key_end - 1) * row_bytes + D * 2),
+        return uint4_t{(uint32_t)ptr, (uint32_t)(ptr >> 32) & 0xffffu, (uint32_t)((key_end - 1) * row_bytes + hd * 2),
                        0x00020000u};
     };
     const uint4_t krs = descriptor(kbase, krow_bytes), vrs = descriptor(vbase, vrow_bytes);
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
         const int pos = 1024 * i + 16 * lane;
         const int pitch = is_k ? KP : VP, bytes = is_k ? K_BYTES : V_BYTES;
         const int r = pos / pitch, cbyte = pos % pitch;
-        const bool active = pos < bytes && cbyte < 2 * D;
+        const bool active = pos < bytes && cbyte < 2 * hd;  // (the dims that pad the head up to D read as zero)
         piece_voff[jj] = active ? r * (is_k ? krow_bytes : vrow_bytes) + cbyte : 0x7ffffff0;
         piece_lds[jj] = (is_k ? 0 : V_AT) + 1024 * i;
     }
@@ -231,8 +233,11 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
     for (int cb = 0; cb < CB; cb++) {
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)min(row[cb], p.Sq - 1) * p.qs[2];
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++)
-            qreg[cb][kb] = __builtin_bit_cast(vec8, *(const uint4_t *)(qp + 32 * kb + 8 * q4));
+        for (int kb = 0; kb < KB; kb++) {
+            uint4_t raw = {0, 0, 0, 0};
+            if (32 * kb + 8 * q4 < hd) raw = *(const uint4_t *)(qp + 32 * kb + 8 * q4);
+            qreg[cb][kb] = __builtin_bit_cast(vec8, raw);
+        }
     }
 
     float4_t o[CB][NB];
@@ -373,10 +378,11 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
             // this share's state: O unnormalised, then (m, l); the merge kernel normalises
             float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + row[cb]) * nks + ksplit) * p.pf_pitch;
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) *(float4_t *)(ws + 16 * nb + 4 * q4) = o[cb][nb];
+            for (int nb = 0; nb < NB; nb++)
+                if (16 * nb + 4 * q4 < hd) *(float4_t *)(ws + 16 * nb + 4 * q4) = o[cb][nb];
             if (q4 == 0) {
-                ws[D] = m[cb];
-                ws[D + 1] = l_col;
+                ws[hd] = m[cb];
+                ws[hd + 1] = l_col;
             }
             continue;
         }
@@ -387,6 +393,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, PW_WAVES * CB >= 8 ? 1 : 2) void pre
             for (int r = 0; r < 4; r++) {
                 const float val = o[cb][nb][r] / l_col;
                 const int64_t oi = ob + (int64_t)(16 * nb + 4 * q4 + r) * p.os[3];
+                if (16 * nb + 4 * q4 >= hd) continue;
                 if (p.out_f32) ((float *)p.out)[oi] = val;
                 else ((T *)p.out)[oi] = from_float<T>(val);
             }
@@ -444,12 +451,19 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     const dim3 grid((unsigned)blocks);
-    switch (p.D) {
+    if (p.D % 8 != 0 || p.D < 8 || p.D > 256) {
+        set_error("wide prefill MFMA kernel: head_dim %d is not a multiple of 8 up to 256", p.D);
+        return FHIP_ERR_UNSUPPORTED;
+    }
+    switch ((p.D + 31) / 32 * 32) {  // the kernel's D is head_dim rounded up to a multiple of 32
+        case 32: launch_wide_d<T, 32>(p, bm, grid, nqb, stream); break;
+        case 64: launch_wide_d<T, 64>(p, bm, grid, nqb, stream); break;
+        case 96: launch_wide_d<T, 96>(p, bm, grid, nqb, stream); break;
+        case 128: launch_wide_d<T, 128>(p, bm, grid, nqb, stream); break;
         case 160: launch_wide_d<T, 160>(p, bm, grid, nqb, stream); break;
         case 192: launch_wide_d<T, 192>(p, bm, grid, nqb, stream); break;
         case 224: launch_wide_d<T, 224>(p, bm, grid, nqb, stream); break;
-        case 256: launch_wide_d<T, 256>(p, bm, grid, nqb, stream); break;
-        default: set_error("wide prefill MFMA kernel: head_dim %d not in {160, 192, 224, 256}", p.D); return FHIP_ERR_UNSUPPORTED;
+        default: launch_wide_d<T, 256>(p, bm, grid, nqb, stream); break;
     }
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.pf_nsplit > 1) return launch_prefill_merge(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);

@@ -136,8 +136,9 @@ typedef struct {
 typedef enum {
     FHIP_KERNEL_AUTO = 0,
     FHIP_KERNEL_GENERIC = 1,     /* any dtype, any strides, any mask; one wavefront per query row   */
-    FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim in {64,96,128} and {160,192,224,256}, LDS-tiled MFMA; masks by
-                                    interval (analytic, kv_lens, or a mask tensor reduced on the device) */
+    FHIP_KERNEL_PREFILL_MFMA = 2,/* f16/bf16, head_dim a multiple of 8 up to 256, LDS-tiled MFMA (64 / 96 / 128 on
+                                    256-row workgroups, the others on the wide-head form); masks by interval
+                                    (analytic, kv_lens, or a mask tensor reduced on the device) */
     FHIP_KERNEL_PREFILL_F32 = 3, /* f32 arithmetic on the f32 MFMA, LDS-tiled: f32 tensors, and 16-bit tensors
                                     (widened on load) the kernel above does not take; head_dim multiple of
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */

@@ -165,11 +165,15 @@ def test_kernel_selection():
     a.mask.shape[:] = [64, 64]
     a.mask.stride[:] = [64, 1]
     assert selected(a)[1] == fa.KERNEL_GENERIC
-    # 16-bit head dims their own matrix-core kernel does not take run on the f32-arithmetic kernel
-    assert selected(make_args(Sq=64, Skv=64, D=80))[1] == fa.KERNEL_PREFILL_F32
-    assert selected(make_args(Sq=64, Skv=64, D=200, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_F32
-    # ... and 160 / 192 / 224 / 256 on the wide-head form of the 16-bit kernel
+    # 16-bit head dims: every multiple of 8 up to 256 runs on the 16-bit matrix cores (64 / 96 / 128 on the 256-row kernel,
+    # the others, padded with zeros to the next multiple of 32, on the wide-head one) ...
+    assert selected(make_args(Sq=64, Skv=64, D=80))[1] == fa.KERNEL_PREFILL_MFMA
+    assert selected(make_args(Sq=64, Skv=64, D=200, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_MFMA
+    assert selected(make_args(Sq=64, Skv=64, D=8))[1] == fa.KERNEL_PREFILL_MFMA
     assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_MFMA
+    # ... and the other multiples of 4 on the f32-arithmetic kernel (rows widened on load)
+    assert selected(make_args(Sq=64, Skv=64, D=100))[1] == fa.KERNEL_PREFILL_F32
+    assert selected(make_args(Sq=64, Skv=64, D=12, dtype=fa.BF16))[1] == fa.KERNEL_PREFILL_F32
     assert selected(make_args(Sq=64, Skv=64, D=256, dtype=fa.F32))[1] == fa.KERNEL_PREFILL_F32
     assert selected(make_args(Sq=64, Skv=64, D=264))[1] == fa.KERNEL_GENERIC
     # innermost stride != 1 or a misaligned base pointer -> generic

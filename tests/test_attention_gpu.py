@@ -317,11 +317,12 @@ def test_prefill_f32_wide_heads(device, D, case):
 
 
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
-@pytest.mark.parametrize("D,case", [(80, "causal"), (144, "causal"), (200, "window_offset"), (32, "full_ragged"), (40, "causal"),
+@pytest.mark.parametrize("D,case", [(84, "causal"), (148, "causal"), (204, "window_offset"), (36, "full_ragged"), (44, "causal"),
                                     (128, "bias"), (64, "bias"), (96, "bias_batch_key")])
 def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
-    """Head dims and mask tensors the 16-bit matrix-core kernel does not take run on the tiled kernel that computes
-    in f32: rows are widened on their way into LDS, the result is rounded to the tensors' type."""
+    """Head dims (multiples of 4 that are not multiples of 8) and mask tensors the 16-bit matrix-core kernels do not take
+    run on the tiled kernel that computes in f32: rows are widened on their way into LDS, the result is rounded to the
+    tensors' type."""
     B, H, Hkv = 2, 4, 2
     Sq, Skv = {"causal": (150, 150), "window_offset": (97, 400), "full_ragged": (70, 333), "bias": (90, 200),
                "bias_batch_key": (90, 200)}[case]
@@ -358,10 +359,11 @@ def test_16_bit_tensors_on_the_f32_arithmetic_kernel(device, dtype, D, case):
 
 
 @pytest.mark.parametrize("dtype", [fa.F16, fa.BF16])
-@pytest.mark.parametrize("D", [160, 192, 224, 256])
+@pytest.mark.parametrize("D", [160, 192, 224, 256, 8, 40, 80, 144, 200, 32])
 @pytest.mark.parametrize("case", ["causal", "chunk_window", "ragged", "mask_tensor", "bias", "padding_mask", "cache_views", "full"])
 def test_wide_head_dims_on_the_16_bit_matrix_cores(device, dtype, D, case):
-    """Head dims 160 ... 256 (Gemma-3's key length is 256) in 16-bit: the four-wavefront tiled kernel, 128 query rows per
+    """Head dims 160 ... 256 (Gemma-3's key length is 256), and every other multiple of 8 that is not 64 / 96 / 128 (80 in
+    Qwen-VL's vision blocks), padded with zeros to the next multiple of 32, in 16-bit: the four-wavefront tiled kernel, 128 query rows per
     workgroup and 32-key tiles; every way of masking, rows and keys that do not fill their last block or tile, K and V
     as narrowed views of a larger cache allocation, GQA, and the output in f32 as well."""
     B, H, Hkv = 2, 6, 2
@@ -720,7 +722,7 @@ def test_few_query_rows_on_a_long_cache_split_the_keys(device, dtype, D, case):
 
 
 @pytest.mark.parametrize("dtype,D,G,Sq", [(fa.F32, 256, 4, 20), (fa.F32, 256, 2, 32), (fa.F32, 160, 4, 17), (fa.F32, 200, 6, 17),
-                                          (fa.F16, 144, 2, 30), (fa.F32, 256, 3, 20)])
+                                          (fa.F16, 148, 2, 30), (fa.F32, 256, 3, 20)])
 @pytest.mark.parametrize("case", ["causal_offset", "window", "mask_tensor", "kv_lens", "full"])
 def test_few_rows_above_head_dim_128_in_f32_arithmetic_pair_two_heads(device, dtype, D, G, Sq, case):
     """Up to 32 new rows on a long cache above head_dim 128 on the f32-arithmetic kernel (Gemma-3's key length in the
