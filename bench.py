@@ -6,12 +6,14 @@
 A step is one attention call through the C ABI on synthetic, seeded inputs that are resident in
 HBM before the timed region.  The default workload is C2 (Llama-3-8B-shaped decode, batch 16, 4096
 f16 KV tokens per sequence): `value` is its KV-streaming rate in GB/s (algorithmic bytes per call /
-time per call, combine pass included).  The same JSON line also carries the C3 prefill figure
-(TFLOP/s, MFMA roofline) under "prefill" and, under "configs", the other three benchmark configurations
-(C1, C4, C5) plus two decode workloads beside C2 (F2: the same batch with an f32 cache, M1: four new rows per
-sequence), each with the HBM/MFMA roofline of its dominant kernel (the kernel's own
-duration from HIP events carried by its dispatch on the launch stream) and the CPU checker timed on
-the host cores ("cpu_baseline").
+time per call, combine pass included).
+
+Output: one JSON object per line.  Lines that start with {"detail": ...} come first and hold every workload's
+complete record (roofline of its dominant kernel from HIP events carried by that kernel's dispatch on the launch
+stream, the CPU checker timed on the host cores as "cpu_baseline", a spot check against it) and the two
+calibrations.  The LAST line is the result line: C2 in full contract form with "roofline" and "cpu_baseline",
+the C3 prefill figure (TFLOP/s, MFMA roofline, its own cpu_baseline) under "prefill", and one short entry per
+other workload under "configs" (C1, C1M, C4, C5, F2, M1, L1, L2, W2, W3); it stays under 4 KB.
 """
 import argparse
 import ctypes
@@ -573,45 +575,95 @@ def main():
     main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
     if a.calibration_copy:
         calibration_copy()
-    line = {"metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": a.steps,
-            "warmup": a.warmup, "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (seeded SplitMix64 normals)",
-            "config": main_res["config"], "roofline": main_res["roofline"],
-            "frac_of_roofline": main_res["frac_of_roofline"],
-            "spot_check_max_abs_err": main_res["spot_check_max_abs_err"]}
-    if "cpu_baseline" in main_res:
-        line["cpu_baseline"] = main_res["cpu_baseline"]
-    if "imbalance" in main_res:
-        line["imbalance"] = main_res["imbalance"]
+    detail("workload", dict(main_res, steps=a.steps, warmup=a.warmup))
+    read_cal = pre = mfma_cal = None
+    others = {}
     if not a.no_extra and a.config == "C2":
         # beside the nominal 8 TB/s the roofline is priced against: what a kernel that only reads the same number of
         # bytes per launch reaches on this chip
-        line["roofline"]["read_calibration"] = calibration_read()
+        read_cal = calibration_read()
+        detail("read_calibration", read_cal)
         # the other half of the metric: C3 prefill on the matrix cores
         # the shader clock needs some tens of milliseconds of matrix load to settle: warm the prefill
         # leg up for longer than the (much shorter) decode steps need
         pre = run_config("C3", max(20, a.steps // 2), max(100, a.warmup), with_cpu=not a.no_cpu)
-        line["prefill"] = {k: pre[k] for k in ("value", "unit", "ms_per_step", "roofline", "config", "dtype",
-                                               "frac_of_roofline", "spot_check_max_abs_err") if k in pre}
-        if "cpu_baseline" in pre:
-            line["prefill"]["cpu_baseline"] = pre["cpu_baseline"]
+        detail("workload", dict(pre, steps=max(20, a.steps // 2), warmup=max(100, a.warmup)))
         # beside the nominal peak the roofline is priced against: what a register-only loop of the same matrix
         # instruction reaches on this chip under its power limit, and the clock it holds
-        line["prefill"]["mfma_calibration"] = calibration_mfma()
-        # the remaining benchmark configurations, each a line of its own in miniature
-        line["configs"] = {}
-        # (F2: C2's batch with the f32 cache kalosm-llama keeps; M1: C2's batch with four new rows per sequence)
-        for name, (steps, warmup) in (("C1", (200, 20)), ("C4", (100, 100)), ("C5", (20, 3)), ("F2", (100, 10)),
-                                      ("M1", (100, 10))):
-            r = run_config(name, steps, warmup, with_cpu=not a.no_cpu)
+        mfma_cal = calibration_mfma()
+        detail("mfma_calibration", mfma_cal)
+        # the remaining benchmark configurations (C1M: C1 with the mask as the tensor kalosm-llama passes; F2: C2's batch
+        # with the f32 cache kalosm-llama keeps; M1: C2's batch with four new rows per sequence; L1 / L2: a whole
+        # attention layer step around the call; W2 / W3: Gemma-3's key length 256 in f16, no CPU leg)
+        for name, (steps, warmup, cpu) in EXTRA_WORKLOADS.items():
+            r = run_config(name, steps, warmup, with_cpu=cpu and not a.no_cpu)
             r["steps"], r["warmup"] = steps, warmup
-            line["configs"][name] = r
-        # (W2 / W3: a decode step and a 4096-token prompt at Gemma-3's key length 256 in f16; no CPU leg)
-        for name, (steps, warmup) in (("W2", (100, 10)), ("W3", (50, 100))):
-            r = run_config(name, steps, warmup, with_cpu=False)
-            r["steps"], r["warmup"] = steps, warmup
-            line["configs"][name] = r
-    print(json.dumps(line))
+            detail("workload", r)
+            others[name] = r
+    print(json.dumps(final_line(main_res, a.steps, a.warmup, read_cal, pre, mfma_cal, others)), flush=True)
+
+
+# workloads beside C2 and C3 on the default run: name -> (steps, warm-up steps, CPU leg)
+EXTRA_WORKLOADS = {"C1": (200, 20, True), "C1M": (200, 20, False), "C4": (100, 100, True), "C5": (20, 3, True),
+                   "F2": (100, 10, True), "M1": (100, 10, True), "W2": (100, 10, False), "W3": (50, 100, False)}
+
+
+def detail(kind, obj):
+    """One complete record per line, ahead of the final line (which stays short enough for any log tail)."""
+    print(json.dumps({"detail": kind, **(obj if isinstance(obj, dict) else {"rows": obj})}), flush=True)
+
+
+def _r(x, digits=5):
+    return float(f"{x:.{digits}g}") if isinstance(x, float) else x
+
+
+def _short_roofline(roof, keys=("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "kernel_ms_mean")):
+    return {k: _r(roof[k]) for k in keys if k in roof}
+
+
+def _short_config(cfg):
+    keep = ("workload", "kind", "batch", "q_heads", "kv_heads", "q_len", "kv_len", "head_dim", "causal", "window",
+            "ragged_lens", "kv_sets_rotated", "algorithmic_flops", "algorithmic_bytes")
+    return {k: cfg[k] for k in keep if cfg.get(k) is not None}
+
+
+def _short_cpu(cpu):
+    return dict(value=_r(cpu["value"]), unit=cpu["unit"], cores=cpu["cores"], kind=cpu["kind"], sample=cpu["sample"][:100])
+
+
+def final_line(main_res, steps, warmup, read_cal=None, pre=None, mfma_cal=None, others=None):
+    """The last line of stdout: the headline workload in full contract form, C3 under "prefill", one short entry per other
+    workload.  Everything else went out earlier as "detail" lines.  Kept under 4 KB."""
+    line = {"metric": METRIC, "value": _r(main_res["value"], 6), "unit": main_res["unit"], "n_gpus": 1, "steps": steps,
+            "warmup": warmup, "ms_per_step": _r(main_res["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": main_res["dtype"], "data": "synthetic (seeded SplitMix64 normals)",
+            "config": _short_config(main_res["config"]), "roofline": _short_roofline(main_res["roofline"]),
+            "frac_of_roofline": _r(main_res["frac_of_roofline"]),
+            "spot_check_max_abs_err": _r(main_res["spot_check_max_abs_err"])}
+    if read_cal:
+        line["roofline"]["read_calibration_gbps"] = _r(read_cal["gbps"])
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = _short_cpu(main_res["cpu_baseline"])
+    if "imbalance" in main_res:
+        line["imbalance"] = {k: _r(v) for k, v in main_res["imbalance"].items() if k != "note"}
+    if pre:
+        line["prefill"] = dict(value=_r(pre["value"], 6), unit=pre["unit"], ms_per_step=_r(pre["ms_per_step"], 6), dtype=pre["dtype"],
+                               frac_of_roofline=_r(pre["frac_of_roofline"]), config=_short_config(pre["config"]),
+                               roofline=_short_roofline(pre["roofline"]),
+                               spot_check_max_abs_err=_r(pre["spot_check_max_abs_err"]))
+        if "cpu_baseline" in pre:
+            line["prefill"]["cpu_baseline"] = _short_cpu(pre["cpu_baseline"])
+        if mfma_cal:
+            row = next((r for r in mfma_cal if r["dtype"] == "f16" and r["operands"] == "random" and r["duty_percent"] == 100), None)
+            if row:
+                line["prefill"]["mfma_calibration"] = {k: _r(row[k]) for k in ("dtype", "operands", "duty_percent", "tflops",
+                                                                               "sclk_ghz_median")}
+    if others:
+        # value = per step by the wall clock; kernel_frac = the dominant kernel's own duration against its roofline
+        line["configs"] = {name: dict(value=_r(r["value"]), unit=r["unit"], ms_per_step=_r(r["ms_per_step"]),
+                                      step_frac=_r(r["frac_of_roofline"], 4), kernel_frac=_r(r["roofline"]["frac"], 4),
+                                      err=_r(r["spot_check_max_abs_err"], 3)) for name, r in others.items()}
+    return line
 
 
 if __name__ == "__main__":

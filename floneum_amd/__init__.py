@@ -227,11 +227,14 @@ class Device:
         self._workspace = None
         self._workspace_bytes = 0
         self._pool, self._sizes, self._pooled = {}, {}, 0  # cached free blocks by size, block sizes, bytes cached
-        # A recorded graph keeps the POINTERS of the buffers and of the workspace its calls used, not the buffers:
-        # while a capture is open or a Graph of this device is alive, freed blocks are parked instead of being
-        # handed out again (a replay would overwrite their new owner's data), and the workspace is neither
-        # recycled nor grown under a capture.
+        # A recorded graph keeps the POINTERS of the buffers and of the workspace its calls used, not the buffers.
+        # The blocks a capture may have recorded (those alive when it opened or allocated while it was open) are
+        # `_pinned`: freed while a capture is open or a Graph of this device is alive, they are parked instead of
+        # being handed out again (a replay would overwrite their new owner's data).  Blocks allocated after the
+        # capture closed are not pinned and return to the cache as usual.  The workspace is neither recycled nor
+        # grown under a capture.
         self._capturing, self._graphs_alive, self._parked = False, 0, []
+        self._live, self._pinned = set(), set()
 
     @classmethod
     def default(cls):
@@ -261,16 +264,22 @@ class Device:
         free_list = self._pool.get(size)
         if free_list:
             self._pooled -= size
-            return free_list.pop()
-        p = ctypes.c_void_p()
-        check(lib().fhip_malloc(self.handle, size, ctypes.byref(p)))
-        self._sizes[p.value] = size
-        return p.value
+            ptr = free_list.pop()
+        else:
+            p = ctypes.c_void_p()
+            check(lib().fhip_malloc(self.handle, size, ctypes.byref(p)))
+            self._sizes[p.value] = size
+            ptr = p.value
+        self._live.add(ptr)
+        if self._capturing:
+            self._pinned.add(ptr)
+        return ptr
 
     def free(self, ptr):
-        if self._capturing or self._graphs_alive > 0:
+        if self._capturing or (self._graphs_alive > 0 and ptr in self._pinned):
             self._parked.append(ptr)
             return
+        self._live.discard(ptr)
         size = self._sizes.get(ptr)
         if size is not None and self._pooled + size <= self._CACHE_LIMIT:
             self._pool.setdefault(size, []).append(ptr)
@@ -283,6 +292,7 @@ class Device:
         self._graphs_alive -= 1
         if self._graphs_alive == 0 and not self._capturing:
             parked, self._parked = self._parked, []
+            self._pinned = set()
             for ptr in parked:
                 self.free(ptr)
 
@@ -344,6 +354,7 @@ class _Capture:
     def __enter__(self):
         check(lib().fhip_stream_begin_capture(self.device.stream))
         self.device._capturing = True
+        self.device._pinned |= self.device._live
         return self
 
     def __exit__(self, exc_type, exc, tb):

@@ -16,14 +16,13 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-EXTRA = os.environ.get("FHIP_EXTRA_FLAGS", "").split()  # e.g. -D switches while tuning
 # the rotary embedding must round every product and sum on its own (bit parity with the reference's CPU path)
 PER_FILE = {"rope.hip": ["-ffp-contract=off"]}
 
 
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + PER_FILE.get(src, []) + EXTRA + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + PER_FILE.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

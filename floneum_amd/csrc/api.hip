@@ -223,9 +223,9 @@ static bool prefill_mfma_eligible(const fhip_attn_args *a) {
     const bool wide = !(D == 64 || D == 96 || D == 128);
     if (D % 8 != 0 || D < 8 || D > 256) return false;
     if (!rows_vectorizable(a->q, 2) || !rows_vectorizable(a->k, 2) || !rows_vectorizable(a->v, 2)) return false;
-    // the kernel for 64 / 96 / 128 folds scale * log2(e) into Q (rounded back to the input type): the factor must not
-    // be able to push a finite element out of range (the wide-head kernel scales the scores in f32)
-    if (!wide && (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f <= 1.0f))) return false;
+    // the kernel for 64 / 96 / 128 multiplies Q by the power-of-two part of scale * log2(e): that power must be at most
+    // 1 so that no finite element can leave the type's range (the wide-head kernel scales the scores in f32 only)
+    if (!wide && (!(a->scale > 0.0f) || !(a->scale * 1.4426950408889634f < 2.0f))) return false;
     // K/V rows are fetched through 32-bit buffer offsets: rows must not overlap and one (batch, kv
     // head) slice must span less than 2 GiB
     const uint64_t Skv = a->k.shape[2];
@@ -299,6 +299,18 @@ static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *
     else
         prefill_mfma_plan((int)a->q.shape[0], (int)a->q.shape[1], Hkv ? (int)a->q.shape[1] / Hkv : 1, (int)a->q.shape[2],
                           (int)a->k.shape[2], causal_square, cus > 0 ? cus : 256, nsplit, chunk);
+}
+
+// A workspace too small for the planned key split still takes the largest split that fits (shares stay multiples of 64
+// keys, which every tiled kernel's tile size divides); below two shares the call runs unsplit.
+static void fit_split(int Skv, size_t bytes_per_share, size_t avail, int *nsplit, int *chunk) {
+    if (*nsplit <= 1 || bytes_per_share == 0 || bytes_per_share * (size_t)*nsplit <= avail) return;
+    const long fit = (long)(avail / bytes_per_share);
+    long c = fit >= 2 ? ((long)Skv + fit - 1) / fit : Skv;
+    c = (c + 63) / 64 * 64;
+    *chunk = (int)c;
+    *nsplit = (int)((Skv + c - 1) / c);
+    if (*nsplit <= 1) *nsplit = 1, *chunk = Skv;
 }
 
 // assume_workspace: answer as if the caller had provided the scratch a masked tiled call needs
@@ -430,9 +442,13 @@ int fhip_device_create(int32_t ordinal, fhip_device **out) {
         return FHIP_ERR_UNSUPPORTED;
     }
     // this device's copy of the static workspace (the lookup is per device: it must be the current one)
+    // (the calling thread's current device is put back afterwards)
     d->scratch_ptr = nullptr;
+    int previous = -1;
+    (void)hipGetDevice(&previous);
     e = hipSetDevice(ordinal);
     if (e == hipSuccess) e = hipGetSymbolAddress((void **)&d->scratch_ptr, HIP_SYMBOL(scratch));
+    if (previous >= 0 && previous != ordinal) (void)hipSetDevice(previous);
     if (e != hipSuccess || !d->scratch_ptr) {
         delete d;
         return hip_fail(e, "hipGetSymbolAddress(scratch)");
@@ -764,6 +780,8 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
             rc = launch_fill_zero_rows(out, args->out.stride, args->out.shape, elem_bytes(args->out_dtype), s->s);
             if (rc) return rc;
         }
+        // no attention kernel runs: the hooks still hold a valid (empty) interval
+        if (args->main_kernel_start && args->main_kernel_done) FHIP_HIP_CHECK(hipEventRecord(args->main_kernel_start->e, s->s));
         if (args->main_kernel_done) FHIP_HIP_CHECK(hipEventRecord(args->main_kernel_done->e, s->s));
         return FHIP_OK;
     }
@@ -771,14 +789,25 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
     fill_params(args, &p);
     p.main_done = args->main_kernel_done ? args->main_kernel_done->e : nullptr;
     p.main_start = args->main_kernel_start && p.main_done ? args->main_kernel_start->e : nullptr;
+    if (p.main_start) {
+        // a dispatch that carries its own events cannot be recorded into a graph
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        FHIP_HIP_CHECK(hipStreamIsCapturing(s->s, &capturing));
+        if (capturing != hipStreamCaptureStatusNone) {
+            set_error("main_kernel_start cannot be used while the stream is being captured (use main_kernel_done alone)");
+            return FHIP_ERR_UNSUPPORTED;
+        }
+    }
     p.cus = s->dev->prop.multiProcessorCount;
     if (id == FHIP_KERNEL_PREFILL_F32) {
         // few query rows on a long cache: split the keys over workgroups if the caller brought the scratch for it
         int ns, chunk;
         f32_split_plan(args, s->dev->prop.multiProcessorCount, &ns, &chunk);
         const size_t off = f32_partials_offset(args);
+        const bool usable = args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes > off;
+        if (usable) fit_split(p.Skv, prefill_f32_workspace_bytes(p.B, p.H, p.Sq, p.D, 2) / 2, args->workspace_bytes - off, &ns, &chunk);
         const size_t part = prefill_f32_workspace_bytes(p.B, p.H, p.Sq, p.D, ns);
-        if (part && args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes >= off + part) {
+        if (part && usable && args->workspace_bytes >= off + part) {
             p.pf_nsplit = ns;
             p.pf_chunk = chunk;
             p.pf_pitch = p.D + 2;
@@ -789,8 +818,10 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         int ns, chunk;
         mfma_split_plan(args, s->dev->prop.multiProcessorCount, &ns, &chunk);
         const size_t off = f32_partials_offset(args);
+        const bool usable = args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes > off;
+        if (usable) fit_split(p.Skv, prefill_mfma_workspace_bytes(p.B, p.H, p.Sq, p.D, 2) / 2, args->workspace_bytes - off, &ns, &chunk);
         const size_t part = prefill_mfma_workspace_bytes(p.B, p.H, p.Sq, p.D, ns);
-        if (part && args->workspace && ((uintptr_t)args->workspace & 15) == 0 && args->workspace_bytes >= off + part) {
+        if (part && usable && args->workspace_bytes >= off + part) {
             p.pf_nsplit = ns;
             p.pf_chunk = chunk;
             p.pf_pitch = p.D + 4;  // rows of the partials are written in 16-byte pieces
@@ -882,8 +913,9 @@ int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_opera
         set_error("calibration: NULL stream or scratch");
         return FHIP_ERR_INVALID_ARG;
     }
-    if (duty_percent < 40 || duty_percent > 100 || rounds < 1) {
-        set_error("calibration: duty_percent %d must be in 40..100 and rounds %d positive", duty_percent, rounds);
+    if (duty_percent < 40 || duty_percent > 100 || rounds < 1 || rounds > FHIP_CALIBRATION_MFMA_MAX_ROUNDS) {
+        set_error("calibration: duty_percent %d must be in 40..100 and rounds %d in 1..%d", duty_percent, rounds,
+                  FHIP_CALIBRATION_MFMA_MAX_ROUNDS);
         return FHIP_ERR_INVALID_ARG;
     }
     const int cus = s->dev->prop.multiProcessorCount;
@@ -919,6 +951,14 @@ int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args) {
     size_t need = 0;
     int rc = fhip_flash_attention_workspace_bytes(args, s->dev->prop.multiProcessorCount, &need);
     if (rc) return rc;
+    // What a call cannot do without: the split-KV partials of a decode step, the interval table of a mask tensor.  The
+    // partials of a tiled prefill call's key split are optional: fhip_flash_attention takes the largest split that fits
+    // the workspace it is given (none, if not even two shares fit).
+    int32_t id;
+    rc = select_kernel(args, &id, true);
+    if (rc) return rc;
+    if ((id == FHIP_KERNEL_PREFILL_MFMA || id == FHIP_KERNEL_PREFILL_F32) && !output_is_empty(args) && !no_keys(args))
+        need = mask_scratch_bytes(args);
     if (need > STATIC_WORKSPACE_BYTES) {
         set_error("this call needs a workspace of %zu bytes; fhip_flash_attention_noalloc holds %zu (use "
                   "fhip_flash_attention with a workspace of your own)", need, STATIC_WORKSPACE_BYTES);

@@ -4,10 +4,9 @@
 // Keys/values are walked in tiles of 64 rows that go from global memory straight into a three-stage
 // LDS ring (direct-to-LDS buffer loads, no staging registers).  Per tile and wavefront:
 //   S^T (64 keys x 32 queries)  = K_tile . Q^T      v_mfma_f32_32x32x16  (A = K from LDS, B = Q in registers)
-//   Q is multiplied by scale * log2(e) once (f16; for bf16 only by its power-of-two part, the rest multiplies
-//   the scores in f32), and the first MFMA of a tile takes -m (the running row maximum) as its C operand, so
-//   the accumulators come out as base-2 exponents relative to the maximum and go straight into exp2: no
-//   multiply or subtract per score in f16
+//   Q is multiplied once by the power-of-two part of scale * log2(e) (exact); the rest, a factor in [1, 2),
+//   multiplies the scores in f32.  The first MFMA of a tile takes -m (the running row maximum) as its C
+//   operand, so the accumulators come out relative to the maximum: one multiply per score, then exp2
 //   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of
 //   it per 32-key block, so the row max / row sum are in-lane folds plus one exchange with the
 //   lane 32 away (v_permlane32_swap); the running maximum is only moved (and O rescaled) when a
@@ -46,12 +45,6 @@ constexpr int PF_WAVES = 8;
 constexpr int PF_BM = 32 * PF_WAVES;  // query rows per workgroup
 constexpr int PF_BN = 64;             // key rows per tile
 constexpr float PF_LOG2E = 1.4426950408889634f;
-
-// Sensitivity switches for measurements only; never defined in a shipped build (`FHIP_EXTRA_FLAGS=-D... python -m
-// floneum_amd.build`).  Both give WRONG RESULTS on purpose: they take away half of one kind of work while the matrix
-// instructions stay the same, to see how much of the run time (i.e. of the power budget) that work costs.
-//   FHIP_EXP_HALF_LDS  every second LDS operand read is skipped (the registers keep what they held)
-//   FHIP_EXP_HALF_EXP  every second exponential is skipped
 
 #define LDS_PTR(type, byte_off) ((__attribute__((address_space(3))) type *)(lds_base + (byte_off)))
 
@@ -188,19 +181,16 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     const int qrow = min(query, p.Sq - 1);
     const bool wave_has_rows = qw0 < p.Sq;
 
-    // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel, already
-    // multiplied by scale * log2(e) (rounded back to the input type): the S^T accumulators then hold
-    // base-2 exponents and the softmax needs no multiply per score
+    // Q^T operand: Q[query][16 kb + 8 h2 .. +8], kept in registers for the whole kernel
     // (the loads are issued here, the scaling waits until the first K/V tiles are on their way too)
     const float scale2 = p.scale * PF_LOG2E;
-    // f16: Q takes the whole factor scale2 (one rounding to 11 bits per element of Q: a score is off by about
-    // 2^-11.5 of the root sum of squares of its terms, 5e-4 of an exponent for unit-variance inputs; it grows in
-    // proportion to the scores).  bf16 would keep 8 bits only, so there scale2 = pw * rr with pw a power of two and rr
-    // in [1, 2): Q takes pw, which is exact, and rr multiplies every score in f32 right before exp2 (one more vector
-    // instruction per score, 4 % of an 8192 x 8192 call); the S^T accumulators, m and negm are then in units of 1 / rr.
-    constexpr bool EXACT_SCALE = std::is_same<T, bf16_t>::value;
-    const float pw = EXACT_SCALE ? __uint_as_float(__float_as_uint(scale2) & 0x7F800000u) : scale2;
-    const float rr = EXACT_SCALE ? scale2 / pw : 1.0f;
+    // scale2 = pw * rr with pw a power of two and rr in [1, 2).  Q takes pw, which is exact in f16 and bf16 alike, and
+    // rr multiplies every score in f32 right before exp2: the scores are then the f32 dot product times the scale, one
+    // rounding, as the reference computes them (fusor-ml/fusor/src/composite/flash_attention.rs:145).  Folding all of
+    // scale2 into Q instead would save that multiply but round Q's elements a second time (11 bits in f16, 8 in bf16),
+    // an error that grows in proportion to the scores.  The S^T accumulators, m and negm are in units of 1 / rr.
+    const float pw = __uint_as_float(__float_as_uint(scale2) & 0x7F800000u);
+    const float rr = scale2 / pw;
     const float slack_u = PF_RESCALE_SLACK / rr;
     vec8 qreg[D / 16];
     {
@@ -369,12 +359,6 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         auto read_v = [&](int gq, uint4_t (&a)[NDB]) {  // gq = 2 t + kk: rows 32 t + 16 kk (+8)
 #pragma unroll
             for (int db = 0; db < NDB; db++) {
-#ifdef FHIP_EXP_HALF_LDS
-                if (db & 1) {
-                    a[db] = a[db - 1];
-                    continue;
-                }
-#endif
                 const int addr = vbase + gq * C::ROWB + db * 64;
                 short4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr));
                 short4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, addr + 8 * C::VG));
@@ -390,9 +374,6 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
             for (int db = 0; db < NDB; db++) o[db] = Mma<T>::mfma(__builtin_bit_cast(vec8, a[db]), bop, o[db]);
         };
         auto read_k = [&](int kb, uint4_t (&a)[2]) {
-#ifdef FHIP_EXP_HALF_LDS
-            if (kb & 1) return;
-#endif
 #pragma unroll
             for (int t = 0; t < 2; t++) a[t] = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
         };
@@ -480,12 +461,8 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(EXACT_SCALE ? s[t][r] * rr : s[t][r]);
-#ifdef FHIP_EXP_HALF_EXP
-                const float p1 = p0;
-#else
-                const float p1 = __builtin_amdgcn_exp2f(EXACT_SCALE ? s[t][r + 1] * rr : s[t][r + 1]);
-#endif
+                const float p0 = __builtin_amdgcn_exp2f(s[t][r] * rr);
+                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1] * rr);
                 pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
                 l += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
             }

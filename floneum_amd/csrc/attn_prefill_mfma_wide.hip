@@ -438,11 +438,7 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // two matrix instructions): 256-row workgroups where those still give every CU one (f16, 4096 x 4096 causal:
     // head_dim 160 497 -> 559 TFLOP/s, 192 450 -> 511; at 224 and 256 the registers do not suffice)
     const long wgs256 = (long)p.B * p.H * ((p.Sq + 255) / 256);
-#ifdef PW_FORCE_256
-    const bool big = true;
-#else
     const bool big = wgs256 >= p.cus;
-#endif
     if (!p.pf_pack && !small && p.pf_nsplit <= 1 && p.D <= 192 && big) bm = 256;
     const int nqb = p.pf_pack ? 1 : (p.Sq + bm - 1) / bm;
     const long blocks = (long)nqb * p.B * (p.pf_pack ? p.H / 4 : p.H) * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);

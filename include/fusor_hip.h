@@ -119,8 +119,8 @@ typedef struct {
                         padding mask, has that form) and then runs the tiled kernel; a mask that is
                         not of that form, or a call that brings no workspace, is served by a kernel
                         that adds the mask values like the reference.  A prefill call of few query rows
-                        on a long cache uses it to split the keys over workgroups; without it the call
-                        runs unsplit.  Same results either way.                                       */
+                        on a long cache uses it to split the keys over workgroups (the largest split
+                        whose partial results fit); without it the call runs unsplit.                                       */
     size_t workspace_bytes;
     int32_t force_kernel; /* 0 = choose; otherwise a fhip_kernel_id (testing / benchmarking)       */
     /* Optional profiling hook: when non-NULL the event is recorded on the stream right after the
@@ -129,7 +129,10 @@ typedef struct {
     fhip_event *main_kernel_done;
     /* With main_kernel_done: when non-NULL too, the main kernel's dispatch itself carries the two events
      * and they hold its begin and end as the command processor stamps them; fhip_event_elapsed_ms(start,
-     * done) is then the kernel's own duration, the figure a profiler's kernel trace gives. */
+     * done) is then the kernel's own duration, the figure a profiler's kernel trace gives.  A call that runs
+     * no attention kernel (no output element, or no key) records start and then done on the stream.  Such a
+     * dispatch cannot be recorded into a graph: with main_kernel_start set, a call on a stream that is being
+     * captured fails with FHIP_ERR_UNSUPPORTED (main_kernel_done alone may be captured). */
     fhip_event *main_kernel_start;
 } fhip_attn_args;
 
@@ -237,13 +240,17 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
 
 /* fhip_flash_attention for callers that cannot allocate: code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels and
- * the same results bit for bit, but the workspace is a fixed array of FHIP_NOALLOC_WORKSPACE_BYTES of device
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and same kernels,
+ * but the workspace is a fixed array of FHIP_NOALLOC_WORKSPACE_BYTES of device
  * memory that the library holds on every GPU it is used on until the process ends; args->workspace and
  * args->workspace_bytes are ignored.  Neither this function nor anything it calls allocates or frees memory.
- * A call whose fhip_flash_attention_workspace_bytes exceeds the array fails with FHIP_ERR_WORKSPACE and does
- * nothing.  All calls on one GPU share that GPU's array: two of them must not overlap in time (one stream, or
- * ordered by events); nothing in it has to be cleared between calls. */
+ * Only what a call cannot do without must fit the array: the split-KV partials of a decode call and the interval
+ * table of a mask tensor (otherwise FHIP_ERR_WORKSPACE, and nothing runs).  The key split of a tiled prefill call
+ * (few query rows on a long cache) is optional: it takes the largest split whose partial results fit, so such a call
+ * may run with fewer shares than fhip_flash_attention_workspace_bytes plans, or unsplit (same results to the
+ * stated tolerance).  Results are bit for bit those of fhip_flash_attention with a workspace of
+ * FHIP_NOALLOC_WORKSPACE_BYTES.  All calls on one GPU share that GPU's array: two of them must not overlap in time
+ * (one stream, or ordered by events); nothing in it has to be cleared between calls. */
 #define FHIP_NOALLOC_WORKSPACE_BYTES (32u << 20)
 int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
 
@@ -255,7 +262,9 @@ int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
  * (the wavefront sleeps in between).  FLOPs per launch = 4 * compute_units * rounds * 32 * 32768.  `scratch`
  * (device, 16-byte aligned, compute_units * 1040 bytes) receives compute_units * 256 floats nobody needs and then,
  * per compute unit, two uint64: the shader-clock cycles and the 100 MHz wall-clock ticks its workgroup ran (their
- * ratio * 0.1 = the clock in GHz the chip held under this load).  Asynchronous on `s`. */
+ * ratio * 0.1 = the clock in GHz the chip held under this load).  `rounds` is at most
+ * FHIP_CALIBRATION_MFMA_MAX_ROUNDS (about a second of matrix work).  Asynchronous on `s`. */
+#define FHIP_CALIBRATION_MFMA_MAX_ROUNDS 2000000
 int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
                           void *scratch, size_t scratch_bytes);
 

@@ -66,6 +66,8 @@ pub const FHIP_KERNEL_DECODE_SPLITKV: fhip_kernel_id = 4;
 
 /// Size of the per-GPU array `fhip_flash_attention_noalloc` uses as its workspace.
 pub const FHIP_NOALLOC_WORKSPACE_BYTES: usize = 32 << 20;
+/// Most `rounds` `fhip_calibration_mfma` accepts (about a second of matrix work).
+pub const FHIP_CALIBRATION_MFMA_MAX_ROUNDS: i32 = 2000000;
 
 // ---- structs -----------------------------------------------------------------------------------
 /// Rank-4 strided view `[batch, heads, seq, head_dim]`; offset and strides in elements

@@ -935,26 +935,32 @@ def test_wide_head_prefill_when_the_row_maximum_keeps_rising(device, dtype, tol,
         assert rl <= tol, f"rel-L2 {rl:.2e} at growth {growth}, D{D}, mask {analytic}"
 
 
-@pytest.mark.parametrize("dtype,std,tol", [(fa.BF16, 8.0, dict(max_abs=None, rel_l2=8e-3)), (fa.BF16, 30.0, dict(max_abs=None, rel_l2=8e-3)),
-                                           (fa.F16, 3.0, dict(max_abs=None, rel_l2=1e-3)), (fa.F16, 8.0, dict(max_abs=None, rel_l2=3e-3))])
+@pytest.mark.parametrize("dtype,std,rel_gate,abs_gate", [(fa.BF16, 8.0, 8e-3, None), (fa.BF16, 30.0, 8e-3, None),
+                                                        (fa.F16, 3.0, 1e-3, 2e-3), (fa.F16, 8.0, 1e-3, 2e-3), (fa.F16, 30.0, 1e-3, 2e-3)])
 @pytest.mark.parametrize("D,Sq,Skv", [(128, 300, 300), (64, 200, 1500), (96, 260, 260)])
-def test_tiled_16bit_prefill_at_large_score_magnitudes(device, dtype, std, tol, D, Sq, Skv):
-    """Inputs far wider than the unit-variance benchmark tensors: scaled scores of standard deviation std^2 (9 ... 900),
-    softmax rows close to one-hot.  bf16: the kernel multiplies the scores by the non-power-of-two part of
-    scale * log2(e) in f32 (Q takes only the power of two), so the error does not grow with the scores.  f16: Q takes
-    the whole factor, rounded to 11 bits; the error grows in proportion to the scores and stays inside the gate for
-    scores of standard deviation 9, about three times the gate at 64."""
+def test_tiled_16bit_prefill_at_large_score_magnitudes(device, dtype, std, rel_gate, abs_gate, D, Sq, Skv):
+    """Queries and keys far wider than the unit-variance benchmark tensors: scaled scores of standard deviation std^2
+    (9 ... 900), softmax rows close to one-hot.  The kernel multiplies Q by the power-of-two part of scale * log2(e)
+    only (exact) and the scores by the rest in f32, as the reference multiplies the f32 dot product by the scale, so
+    the error does not grow with the scores: f16 stays inside the gate of the benchmark configurations (rel-L2 1e-3,
+    max-abs 2e-3 on the f32 output) at every magnitude.  Values are unit-variance in the gated run, so that the absolute
+    gate means what it means for the benchmark tensors; a second run with values as wide as the keys checks rel-L2.
+    bf16 is an extension over the reference's types and is held to 8e-3."""
     B, H, Hkv = 1, 4, 2
     rng = np.random.default_rng(77)
     q = rng.normal(0, std, (B, H, Sq, D)).astype(np.float32)
     k = rng.normal(0, std, (B, Hkv, Skv, D)).astype(np.float32)
-    v = rng.normal(0, std, (B, Hkv, Skv, D)).astype(np.float32)
-    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    v1 = rng.normal(0, 1.0, (B, Hkv, Skv, D)).astype(np.float32)
     analytic = (True, Skv - Sq, 0)
-    assert tq.selected_kernel(tk, tv, D ** -0.5, analytic=analytic) == fa.KERNEL_PREFILL_MFMA
-    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out_dtype=fa.F32).to_numpy()
-    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
-                                 _analytic_mask(Sq, Skv, True, Skv - Sq, 0), "qk")
-    assert np.isfinite(out).all()
-    rl = rel_l2(out, ref)
-    assert rl <= tol["rel_l2"], f"rel-L2 {rl:.2e} at std {std}, D{D}"
+    mask = _analytic_mask(Sq, Skv, True, Skv - Sq, 0)
+    for v in (v1, v1 * np.float32(std)):
+        tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+        assert tq.selected_kernel(tk, tv, D ** -0.5, analytic=analytic) == fa.KERNEL_PREFILL_MFMA
+        out = tq.flash_attention(tk, tv, D ** -0.5, analytic=analytic, out_dtype=fa.F32).to_numpy()
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask, "qk")
+        assert np.isfinite(out).all()
+        rl = rel_l2(out, ref)
+        assert rl <= rel_gate, f"rel-L2 {rl:.2e} at std {std}, D{D}"
+        if abs_gate is not None and v is v1:
+            err = float(np.abs(out - ref).max())
+            assert err <= abs_gate, f"max-abs {err:.2e} at std {std}, D{D}"

@@ -176,6 +176,15 @@ def test_blocks_freed_after_capture_are_not_reused_while_the_graph_lives(device)
     host = np.empty((B, H, 1, D), np.float16)
     fa.check(fa.lib().fhip_memcpy_d2h(device.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(out_ptr), host.nbytes))
     assert np.array_equal(host.view(np.uint8), first.view(np.uint8))
+    # a block allocated AND freed after the capture was never recorded: it goes back to the cache and is handed out again
+    # (a serving loop that keeps one recorded step alive must not grow by what it allocates eagerly per step)
+    late = fa.Tensor.empty(device, (3, 5, 7, 64), fa.F16)
+    late_ptr, parked_before = late.buffer.ptr, len(device._parked)
+    del late
+    assert len(device._parked) == parked_before
+    again = fa.Tensor.empty(device, (3, 5, 7, 64), fa.F16)
+    assert again.buffer.ptr == late_ptr
+    del again
     # a larger call while the graph lives: the old workspace is parked, not reused; the replay still works
     k2, v2 = (fa.Tensor.from_numpy(device, np.concatenate([a, a, a, a], 2), fa.F16) for a in (k, v))
     _ = tq.flash_attention(k2, v2, D ** -0.5).to_numpy()

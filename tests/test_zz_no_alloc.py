@@ -83,6 +83,40 @@ def test_noalloc_few_rows_on_a_long_cache_two_calls_in_a_row(device):
               what=f"key shares {Sq} rows on {Skv} keys")
 
 
+def test_noalloc_prefill_whose_planned_key_split_exceeds_the_array_still_runs(device):
+    """A chat turn of 256 new rows on a 16384-key cache (f16, 32/8 heads, head_dim 128) plans 66 MiB of partial rows,
+    twice the array.  Those are optional: the call takes the largest key split that fits, bit for bit what
+    fhip_flash_attention does with a workspace of the array's size, and close to the unsplit call (workspace NULL);
+    then a smaller call whose split fits."""
+    D, H, Hkv = 128, 32, 8
+    for seed, (Sq, Skv, beyond) in enumerate([(256, 16384, True), (64, 4096, False)]):
+        q, k, v = _normal_qkv(330 + seed, 1, H, Hkv, Sq, Skv, D)
+        tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))
+        analytic = (True, Skv - Sq, 0)
+        args = tq._attn_args(tk, tv, D ** -0.5, None, analytic, None, None, fa.KERNEL_AUTO, None)
+        need = ctypes.c_size_t()
+        fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+        assert (need.value > fa.NOALLOC_WORKSPACE_BYTES) == beyond, need.value
+        fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))  # workspace NULL: unsplit
+        unsplit = args._out_tensor.to_numpy()
+        ws = fa.Buffer(device, fa.NOALLOC_WORKSPACE_BYTES)
+        args.workspace, args.workspace_bytes = ws.ptr, fa.NOALLOC_WORKSPACE_BYTES
+        fa.check(fa.lib().fhip_flash_attention(device.stream, ctypes.byref(args)))
+        want = args._out_tensor.to_numpy()
+        out = fa.Tensor.from_numpy(device, np.full(q.shape, 7.0, np.float32), fa.F16)
+        args2 = tq._attn_args(tk, tv, D ** -0.5, None, analytic, None, None, fa.KERNEL_AUTO, out)
+        fa.check(fa.lib().fhip_flash_attention_noalloc(device.stream, ctypes.byref(args2)))
+        got = out.to_numpy()
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), f"{Sq} rows on {Skv}: differs from fhip_flash_attention"
+        assert not np.array_equal(got.view(np.uint8), unsplit.view(np.uint8)), "the keys were not split at all"
+        # the CPU checker on the first KV head's group of query heads
+        G = H // Hkv
+        ref = oracle.flash_attention(rounded(q[:, :G], fa.F16), rounded(k[:, :1], fa.F16), rounded(v[:, :1], fa.F16), D ** -0.5,
+                                     _analytic_mask(Sq, Skv, *analytic), "qk")
+        assert_parity(got[:, :G], ref, TOL_16, f"{Sq} rows on {Skv} keys, largest split that fits")
+        assert_parity(unsplit[:, :G], ref, TOL_16, f"{Sq} rows on {Skv} keys, unsplit")
+
+
 def test_noalloc_rejects_a_call_beyond_its_workspace(device):
     """64 x 64 rows over 65536 keys would park 136 MB of partial results: refused, nothing runs, the output is
     untouched.  (K and V are stride-0 views of a single row: the shape is large, the memory is not.)"""
