@@ -70,6 +70,11 @@ class CAttnArgs(ctypes.Structure):
                 ("main_kernel_start", ctypes.c_void_p)]
 
 
+class CDecodePlanInfo(ctypes.Structure):
+    _fields_ = [("is_decode", ctypes.c_int32), ("nsplit", ctypes.c_int32), ("chunk", ctypes.c_int32),
+                ("wavefronts", ctypes.c_int32), ("kernels", ctypes.c_int32)]
+
+
 class CDeviceInfo(ctypes.Structure):
     _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 64), ("compute_units", ctypes.c_int32),
                 ("wavefront_size", ctypes.c_int32), ("clock_khz", ctypes.c_int32),
@@ -114,6 +119,7 @@ SYMBOLS = {
     "fhip_flash_attention_select": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.POINTER(ctypes.c_int32)]),
     "fhip_flash_attention_workspace_bytes": (ctypes.c_int, [ctypes.POINTER(CAttnArgs), ctypes.c_int32,
                                                             ctypes.POINTER(ctypes.c_size_t)]),
+    "fhip_flash_attention_decode_plan": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs), ctypes.POINTER(CDecodePlanInfo)]),
     "fhip_flash_attention": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
     "fhip_flash_attention_noalloc": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
     "fhip_calibration_mfma": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P, ctypes.c_size_t]),
@@ -603,6 +609,15 @@ class Tensor:
         kid = ctypes.c_int32()
         check(lib().fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
         return kid.value
+
+
+    def decode_plan(self, k, v, scale, mask=None, **kw):
+        """How the call would run on the split-KV decode kernels: dict(is_decode, nsplit, chunk, wavefronts, kernels)."""
+        args = self._attn_args(k, v, scale, mask, kw.get("analytic"), kw.get("kv_lens"), kw.get("out_dtype"),
+                               kw.get("force_kernel", KERNEL_AUTO), kw.get("out"))
+        info = CDecodePlanInfo()
+        check(lib().fhip_flash_attention_decode_plan(self.buffer.device.stream, ctypes.byref(args), ctypes.byref(info)))
+        return {name: getattr(info, name) for name, _ in CDecodePlanInfo._fields_}
 
 
 class IntTensor:

@@ -26,7 +26,37 @@ struct fhip_device {
     // Source of the per-call marks of masked prefill calls (AttnParams::bad_tag): the one piece of state a device
     // handle changes after its creation.
     std::atomic<uint32_t> next_tag;
+    // The fused split-KV merge needs workgroups L of a one-dimensional launch with the same L % 8 to share an XCD (and
+    // with it an L2).  Probed once per handle.  `trip` is a word of pinned host memory the decode kernels set when the
+    // workgroups of a unit find themselves on different XCDs all the same: the next decode call then fails once and the
+    // form stays off for the handle.
+    std::atomic<bool> xcd_grouped;
+    int32_t *trip_host, *trip_dev;
 };
+
+// Do workgroups with the same number modulo 8 run on one XCD?  (The hardware deals the workgroups of a launch to its
+// XCDs round-robin in launch order, starting wherever the previous launch of the queue left off: true for 8, 4, 2 or 1
+// XCDs per device.)
+static void probe_xcd_grouping(fhip_device *d) {
+    d->xcd_grouped.store(false);
+    d->trip_host = d->trip_dev = nullptr;
+    constexpr int N = 4096;
+    uint8_t *dev_ids = nullptr;
+    uint8_t ids[N];
+    if (hipMalloc((void **)&dev_ids, N) != hipSuccess) return;
+    bool ok = fhip::launch_xcd_probe(dev_ids, N, nullptr) == FHIP_OK && hipMemcpy(ids, dev_ids, N, hipMemcpyDeviceToHost) == hipSuccess;
+    (void)hipFree(dev_ids);
+    for (int i = 0; ok && i < N; i++) ok = ids[i] < 16 && ids[i] == ids[i & 7];
+    if (!ok) return;
+    if (hipHostMalloc((void **)&d->trip_host, sizeof(int32_t), hipHostMallocMapped) != hipSuccess) return;
+    *d->trip_host = 0;
+    if (hipHostGetDevicePointer((void **)&d->trip_dev, d->trip_host, 0) != hipSuccess) {
+        (void)hipHostFree(d->trip_host);
+        d->trip_host = nullptr;
+        return;
+    }
+    d->xcd_grouped.store(true);
+}
 struct fhip_stream {
     fhip_device *dev;
     hipStream_t s;
@@ -448,6 +478,7 @@ int fhip_device_create(int32_t ordinal, fhip_device **out) {
     (void)hipGetDevice(&previous);
     e = hipSetDevice(ordinal);
     if (e == hipSuccess) e = hipGetSymbolAddress((void **)&d->scratch_ptr, HIP_SYMBOL(scratch));
+    if (e == hipSuccess && d->scratch_ptr) probe_xcd_grouping(d);
     if (previous >= 0 && previous != ordinal) (void)hipSetDevice(previous);
     if (e != hipSuccess || !d->scratch_ptr) {
         delete d;
@@ -458,6 +489,7 @@ int fhip_device_create(int32_t ordinal, fhip_device **out) {
 }
 
 int fhip_device_destroy(fhip_device *dev) {
+    if (dev && dev->trip_host) (void)hipHostFree(dev->trip_host);
     delete dev;
     return FHIP_OK;
 }
@@ -758,9 +790,56 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
     return FHIP_OK;
 }
 
+// The plan of a split-KV decode call: the visible stretch of the cache, the split, and whether the splits are merged
+// inside the main kernel (when the device's workgroups are grouped by XCD as that form needs, see probe_xcd_grouping).
+static void plan_decode_call(fhip_device *dev, const fhip_attn_args *args, AttnParams *p) {
+    int lo0, vis_len;
+    decode_visible_range(args, &lo0, &vis_len);
+    if (lo0 > 0 || vis_len < p->Skv) {  // the kernels see keys lo0 .. lo0 + vis_len as keys 0 .. vis_len
+        const int64_t eb = elem_bytes(args->dtype);
+        p->k = (const char *)p->k + lo0 * p->ks[2] * eb;
+        p->v = (const char *)p->v + lo0 * p->vs[2] * eb;
+        p->Skv = vis_len;
+        p->q_pos_offset -= lo0;
+    }
+    decode_plan(p->B, p->Hkv, p->G * p->Sq, p->Skv, p->D, dev->prop.multiProcessorCount, p->kv_lens != nullptr,
+                args->dtype == FHIP_F32, &p->chunk, &p->nsplit, &p->dec_waves);
+    int stride;
+    size_t ctr_off;
+    p->dec_fused = 0;
+    if (dev->xcd_grouped.load() && decode_fused_layout(*p, args->dtype == FHIP_F32, &stride, &ctr_off)) {
+        p->dec_fused = 1;
+        p->dec_unit_stride = stride;
+        p->dec_counters_offset = ctr_off;
+    }
+}
+
 // the 16-bit tiled prefill kernels: 64 / 96 / 128, and the wide-head form above
 static int launch_mfma_by_head_dim(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
     return (p.D == 64 || p.D == 96 || p.D == 128) ? launch_prefill_mfma(p, dtype, stream) : launch_prefill_mfma_wide(p, dtype, stream);
+}
+
+int fhip_flash_attention_decode_plan(fhip_stream *s, const fhip_attn_args *args, fhip_decode_plan_info *info) {
+    if (!s || !info) {
+        set_error("stream/info is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    memset(info, 0, sizeof(*info));
+    int rc = validate(args);
+    if (rc) return rc;
+    int32_t id;
+    rc = select_kernel(args, &id);
+    if (rc) return rc;
+    if (id != FHIP_KERNEL_DECODE_SPLITKV || output_is_empty(args) || no_keys(args)) return FHIP_OK;
+    AttnParams p;
+    fill_params(args, &p);
+    plan_decode_call(s->dev, args, &p);
+    info->is_decode = 1;
+    info->nsplit = p.nsplit;
+    info->chunk = p.chunk;
+    info->wavefronts = p.dec_waves;
+    info->kernels = p.nsplit > 1 && !p.dec_fused ? 2 : 1;
+    return FHIP_OK;
 }
 
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
@@ -875,17 +954,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         case FHIP_KERNEL_PREFILL_MFMA: rc = launch_mfma_by_head_dim(p, args->dtype, s->s); break;
         case FHIP_KERNEL_PREFILL_F32: rc = launch_prefill_f32(p, args->dtype, s->s); break;
         case FHIP_KERNEL_DECODE_SPLITKV: {
-            int lo0, vis_len;
-            decode_visible_range(args, &lo0, &vis_len);
-            if (lo0 > 0 || vis_len < p.Skv) {  // the kernels see keys lo0 .. lo0 + vis_len as keys 0 .. vis_len
-                const int64_t eb = elem_bytes(args->dtype);
-                p.k = (const char *)p.k + lo0 * p.ks[2] * eb;
-                p.v = (const char *)p.v + lo0 * p.vs[2] * eb;
-                p.Skv = vis_len;
-                p.q_pos_offset -= lo0;
-            }
-            decode_plan(p.B, p.Hkv, p.G * p.Sq, p.Skv, p.D, s->dev->prop.multiProcessorCount, p.kv_lens != nullptr,
-                        args->dtype == FHIP_F32, &p.chunk, &p.nsplit, &p.dec_waves);
+            plan_decode_call(s->dev, args, &p);
             const size_t need = decode_workspace_bytes(p.B, p.H * p.Sq, p.Hkv, p.D, p.nsplit);
             if (need > 0 && (!args->workspace || args->workspace_bytes < need)) {
                 set_error("decode needs a workspace of %zu bytes, got %zu", need,
@@ -898,6 +967,20 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
                     return FHIP_ERR_WORKSPACE;
                 }
                 p.partials = (float *)args->workspace;
+                fhip_device *dev = s->dev;
+                if (dev->xcd_grouped.load() && *(volatile int32_t *)dev->trip_host != 0) {
+                    dev->xcd_grouped.store(false);
+                    set_error("the workgroups of one split-KV unit ran on different XCDs, which the device's probe had ruled out: "
+                              "the result of an earlier decode call on this device may be wrong; later calls merge with a "
+                              "second kernel");
+                    return FHIP_ERR_HIP;
+                }
+                if (p.dec_fused) {
+                    p.dec_counters = (uint32_t *)((char *)args->workspace + p.dec_counters_offset);
+                    p.dec_trip = dev->trip_dev;
+                    do p.dec_tag = dev->next_tag.fetch_add(1, std::memory_order_relaxed) & 0xfffffu;
+                    while (p.dec_tag == 0);
+                }
             }
             return launch_decode(p, args->dtype, s->s);  // records main_done itself, before the combine
         }

@@ -108,11 +108,34 @@ void decode_plan(int B, int Hkv, int G, int Skv, int D, int compute_units, bool 
     *nsplit = (int)((Skv + c - 1) / c);
 }
 
-// Workspace: the partials, B * H * nsplit * (D + 2) floats.
+// Workspace: the partials, B * H * nsplit * (D + 2) floats (H counts (head, row) pairs), plus what the fused merge adds:
+// every split's partials start on a 128-byte line, and one arrival counter per unit behind them.
 size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit) {
-    (void)Hkv;
     if (nsplit <= 1) return 0;
-    return (size_t)B * H * nsplit * (size_t)(D + 2) * sizeof(float);
+    // columns of a KV head, padded to whole column blocks of 16 or 32 where there is more than one block
+    const size_t cols = (size_t)H / Hkv;
+    size_t padded = cols;
+    for (size_t gt = 16; gt <= 32; gt *= 2)
+        if (cols > gt && (cols + gt - 1) / gt * gt > padded) padded = (cols + gt - 1) / gt * gt;
+    const size_t units = (size_t)B * Hkv * ((cols + 15) / 16);
+    const size_t partials = (size_t)B * Hkv * padded * nsplit * (size_t)(D + 2) * sizeof(float);
+    if (nsplit > 8) return partials;  // never merged inside the main kernel
+    return partials + units * ((size_t)nsplit * 128 + sizeof(uint32_t)) + 256;
+}
+
+// The fused merge (the matrix-core variants with p.dec_fused): 2 to 8 splits, equal lengths.
+// *unit_stride: floats between the partials of consecutive units; *counters_offset: bytes from the workspace's start
+// to the arrival counters.
+bool decode_fused_layout(const AttnParams &p, bool f32, int *unit_stride, size_t *counters_offset) {
+    const int cols = p.G * p.Sq;
+    if (!decode_use_mfma(p.D, f32, cols) || p.nsplit < 2 || p.nsplit > 8 || p.kv_lens) return false;
+    const int gt = decode_gt(cols, p.D, f32);
+    const long units = (long)p.B * p.Hkv * ((cols + gt - 1) / gt);
+    const long stride = p.nsplit * (((long)(cols < gt ? cols : gt) * (p.D + 2) + 31) / 32 * 32);
+    if ((units + 7) / 8 * 8 * p.nsplit > 0x7fffffffL || stride > 0x7fffffffL) return false;
+    *unit_stride = (int)stride;
+    *counters_offset = ((size_t)units * stride * sizeof(float) + 255) & ~(size_t)255;
+    return true;
 }
 
 // ---- element helpers ---------------------------------------------------------------------------
@@ -458,6 +481,113 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// ---- fused merge of the matrix-core variants ----------------------------------------------------------------------
+// With p.dec_fused the launch is one-dimensional and the workgroups of a (batch, kv head, column block) unit are
+// numbered so that they run on ONE XCD: the hardware deals the workgroups of a launch to its XCDs round-robin in launch
+// order (workgroup L + 1 runs on the XCD after workgroup L's; where workgroup 0 lands depends on what the queue ran
+// before), so workgroups with the same L % 8 share an XCD whether the device has 8, 4, 2 or 1 of them (checked per
+// device before the form is ever chosen).  Their partials then meet in that XCD's L2 and the last workgroup of the unit
+// to arrive merges them: no second kernel, whose dependent launch costs a few microseconds (batch 16 x 4096 keys, f16:
+// 47.1 -> 46.3 us per step; head_dim 256: 54.3 -> 52.2).  The arrival counter itself is kept coherent over the whole
+// device (with partials AND counter device-coherent the form is slower than two kernels) and carries the XCC id of the
+// first workgroup to arrive: a workgroup that arrives from another XCD sets the host-visible word p.dec_trip, which
+// fails the device's next decode call and switches the form off.
+__device__ __forceinline__ uint32_t xcc_id() {
+    uint32_t x;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+    return x & 15u;
+}
+
+__global__ void xcd_probe_kernel(uint8_t *out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = (uint8_t)xcc_id();
+}
+
+int launch_xcd_probe(uint8_t *out, int workgroups, hipStream_t stream) {
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3((unsigned)workgroups), dim3(64), 0, stream, out);
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
+// unit and split of this workgroup (false: the launch is padded to a multiple of 8 units and this one is beyond the end)
+__device__ __forceinline__ bool decode_unit_of_workgroup(const AttnParams &p, int units, int *unit, int *split) {
+    if (p.dec_fused) {
+        const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+        *split = (int)(slot % (unsigned)p.nsplit);
+        *unit = (int)(slot / (unsigned)p.nsplit) * 8 + (int)xcd;
+        return *unit < units;
+    }
+    // spread the splits over the XCDs, see decode_vec_kernel
+    *split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);
+    *unit = blockIdx.y;
+    return true;
+}
+
+// where a workgroup parks column hh of its split in the fused form: a unit's partials are [split][column][D + 2], and
+// every split's part starts on a 128-byte line of its own (no line is written by two workgroups)
+__device__ __forceinline__ float *fused_partial_row(const AttnParams &p, int unit, int split, int hh, int D) {
+    return (float *)p.partials + (int64_t)unit * p.dec_unit_stride + split * (p.dec_unit_stride / p.nsplit) + hh * (D + 2);
+}
+
+// After every thread of the workgroup has stored its part of the unit's partials: count the arrival; the last
+// workgroup of the unit merges the splits in order with the arithmetic of decode_combine_kernel (same bits) and
+// writes the output rows.  Every access is served by this XCD's L2: the stores have been acknowledged by it before
+// the arrival is counted (an atomic in the same L2), and the last workgroup reads lines nobody on its CU has read in
+// this launch (every split's partials have whole lines to themselves, one writer and one reader).  Nothing spins: a workgroup that
+// is not the last leaves.  The counter holds (tag << 8) | arrivals with a tag unique to the call, so it needs no
+// clearing: whatever else it holds (another call's count, the finished count of a replay of this call) restarts it.
+template <typename T, int THREADS>
+__device__ __forceinline__ void fused_merge_tail(const AttnParams &p, int unit, int nh, int D, int b, int g, int c0, int rows) {
+    __shared__ int is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        // word: tag (20 bits) | XCC id of the first workgroup to arrive (4) | arrivals (8)
+        uint32_t *ctr = p.dec_counters + unit;
+        const uint32_t tag = p.dec_tag & 0xfffffu, xcc = xcc_id();
+        const uint32_t fresh = (tag << 12) | (xcc << 8) | 1u;
+        uint32_t cur = (tag << 12) | (xcc << 8), want;
+        do {
+            want = ((cur >> 12) == tag && (cur & 255u) < (uint32_t)p.nsplit) ? cur + 1 : fresh;
+        } while (!__hip_atomic_compare_exchange_strong(ctr, &cur, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT));
+        // the count is kept coherent over the whole device, so a unit whose workgroups are NOT on one XCD is seen here
+        if (((want >> 8) & 15u) != xcc) __hip_atomic_store(p.dec_trip, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        is_last = (want & 255u) == (uint32_t)p.nsplit;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    const float *wu = (const float *)p.partials + (int64_t)unit * p.dec_unit_stride;
+    const int split_stride = p.dec_unit_stride / p.nsplit;
+    for (int idx = threadIdx.x; idx < nh * D; idx += THREADS) {
+        const int hh = idx / D, d = idx % D;
+        float ms[8], ls[8], as[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const bool ok = u < p.nsplit;
+            const float *src = wu + (ok ? u : 0) * split_stride + hh * (D + 2);
+            ms[u] = ok ? src[D] : -INFINITY;
+            ls[u] = ok ? src[D + 1] : 0.0f;
+            as[u] = ok ? src[d] : 0.0f;
+        }
+        float Mn = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 8; u++) Mn = fmaxf(Mn, ms[u]);
+        const float Ms = (Mn == -INFINITY) ? 0.0f : Mn;
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float w = __builtin_amdgcn_exp2f(ms[u] - Ms);
+            L += w * ls[u];
+            A += w * as[u];
+        }
+        const int h = g * p.G + (c0 + hh) / rows, qr = (c0 + hh) % rows;
+        const float val = A / L;  // no visible key: 0/0 = NaN like the reference
+        const int64_t oi = b * p.os[0] + h * p.os[1] + qr * p.os[2] + d * p.os[3];
+        if (p.out_f32) ((float *)p.out)[oi] = val;
+        else ((T *)p.out)[oi] = from_float<T>(val);
+    }
+}
+
 constexpr int DM_KEYS = 32;  // keys per wavefront step
 constexpr int DM_DEPTH = 1;  // tiles in flight per wavefront beside the one in LDS (2 measured no faster: the stream
                              // is not latency-bound with eight wavefronts per CU)
@@ -493,14 +623,15 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
     const int q4 = lane >> 4; // key group
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
-    const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
     // The MFMA columns are the (query head, query row) pairs that share this KV head: column c is head c / rows,
     // row c % rows of the group (one row per head in a plain decode step, a few in a multi-token step).
     const int rows = p.Sq;
     const int NC = p.G * rows;
     const int HB = (NC + COLS - 1) / COLS;
-    const int hb = blockIdx.y % HB;
-    const int bg = blockIdx.y / HB;
+    int split, unit;
+    if (!decode_unit_of_workgroup(p, p.B * p.Hkv * HB, &unit, &split)) return;
+    const int hb = unit % HB;
+    const int bg = unit / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
     const int c0 = hb * COLS;
@@ -741,7 +872,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
             if (p.out_f32) ((float *)p.out)[oi] = val;
             else ((T *)p.out)[oi] = from_float<T>(val);
         } else {
-            float *ws = (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
+            float *ws = p.dec_fused
+                            ? fused_partial_row(p, unit, split, hh, D)
+                            : (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
             ws[d] = A;
             if (d == 0) {
                 ws[D] = M;
@@ -749,6 +882,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void decode_mf
             }
         }
     }
+    if (p.dec_fused && p.nsplit > 1) fused_merge_tail<T, 64 * WAVES>(p, unit, nh, D, b, g, c0, rows);
 }
 
 // ---- pass 1, matrix-core variant for f32 tensors -------------------------------------------------------
@@ -788,12 +922,13 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
     const int q4 = lane >> 4; // key group
     auto lds_base = (__attribute__((address_space(3))) char *)smem + wave * WAVE_BYTES;
 
-    const int split = (int)((blockIdx.x + blockIdx.y) % (unsigned)p.nsplit);  // spread over the XCDs, see decode_vec_kernel
     const int rows = p.Sq;  // columns are (query head, query row) pairs, see decode_mfma_kernel
     const int NC = p.G * rows;
     const int HB = (NC + COLS - 1) / COLS;
-    const int hb = blockIdx.y % HB;
-    const int bg = blockIdx.y / HB;
+    int split, unit;
+    if (!decode_unit_of_workgroup(p, p.B * p.Hkv * HB, &unit, &split)) return;
+    const int hb = unit % HB;
+    const int bg = unit / HB;
     const int g = bg % p.Hkv;
     const int b = bg / p.Hkv;
     const int c0 = hb * COLS;
@@ -1012,7 +1147,9 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
         if (p.nsplit == 1) {
             ((float *)p.out)[b * p.os[0] + h * p.os[1] + qr * p.os[2] + d * p.os[3]] = A / L;  // no visible key: 0/0 = NaN
         } else {
-            float *ws = (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
+            float *ws = p.dec_fused
+                            ? fused_partial_row(p, unit, split, hh, D)
+                            : (float *)p.partials + ((((int64_t)b * p.H + h) * rows + qr) * p.nsplit + split) * (D + 2);
             ws[d] = A;
             if (d == 0) {
                 ws[D] = M;
@@ -1020,6 +1157,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES, D > 128 ? 1 : 2) void decode_mfma_f
             }
         }
     }
+    if (p.dec_fused && p.nsplit > 1) fused_merge_tail<float, 64 * DEC_WAVES>(p, unit, nh, D, b, g, c0, rows);
 }
 
 // ---- pass 2 -------------------------------------------------------------------------------------
@@ -1237,13 +1375,14 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
         return FHIP_ERR_UNSUPPORTED;
     }
     dim3 grid((unsigned)p.nsplit, (unsigned)gy);
+    if (p.dec_fused) grid = dim3((unsigned)((gy + 7) / 8 * 8 * p.nsplit));  // see the kernel's unit numbering
     if constexpr (F32) {
         if (decode_use_mfma(p.D, true, p.G * p.Sq)) {
             if (gt == 32) launch_mfma_f32<2>(p, grid, stream);
             else launch_mfma_f32<1>(p, grid, stream);
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);
-            if (p.nsplit > 1) {
+            if (p.nsplit > 1 && !p.dec_fused) {
                 launch_combine<T>(p, stream);
                 FHIP_HIP_CHECK(hipGetLastError());
             }
@@ -1261,7 +1400,7 @@ static int launch_decode_t(const AttnParams &p, hipStream_t stream) {
             }
             FHIP_HIP_CHECK(hipGetLastError());
             FHIP_MARK_MAIN_DONE(p, stream);
-            if (p.nsplit > 1) {
+            if (p.nsplit > 1 && !p.dec_fused) {
                 launch_combine<T>(p, stream);
                 FHIP_HIP_CHECK(hipGetLastError());
             }

@@ -29,6 +29,14 @@ struct AttnParams {
     int32_t chunk;          // keys per split
     int32_t nsplit;         // splits per (batch, kv head) over Skv
     int32_t dec_waves;      // wavefronts per workgroup of the 16-bit matrix-core decode variant (4 or 8)
+    // Fused merge of the 16-bit matrix-core decode variant (no second kernel): the workgroups of a (batch, kv head)
+    // unit run on one XCD, park their partials in that XCD's L2 and the last one to arrive merges them.
+    int32_t dec_fused;        // 0: two kernels
+    int32_t dec_unit_stride;  // floats between the partials of consecutive units (a multiple of 32: 128-byte lines)
+    uint32_t dec_tag;         // unique to the call (20 bits are used): arrival counters need no clearing
+    uint32_t *dec_counters;   // [units] arrival counters: tag | XCC id of the first arrival | arrivals
+    size_t dec_counters_offset;  // host side: bytes from the workspace's start to the counters
+    int32_t *dec_trip;        // host-visible word set when the workgroups of a unit turn out to run on different XCDs
     // host-side only (profiling hook).  Both set: the dispatch of the main kernel carries the two events, which then
     // hold its own begin and end timestamps.  Only main_done: recorded on the stream after the main kernel.
     hipEvent_t main_start, main_done;
@@ -79,6 +87,11 @@ int launch_mask_intervals(const AttnParams &p, fhip_dtype dtype, int2 *iv, int32
 // writes get_mask's [rows, cols] tensor (0 / -inf bit patterns of `dtype`) into device memory; off = cols - rows
 int launch_mask_build(void *out, fhip_dtype dtype, uint32_t rows, uint64_t cols, uint64_t off, int has_window,
                       uint64_t window, hipStream_t stream);
+
+// layout of the fused split-KV merge in the workspace (false: the call takes the two-kernel form)
+bool decode_fused_layout(const AttnParams &p, bool f32, int *unit_stride, size_t *counters_offset);
+// writes the XCC id each of `workgroups` workgroups of a one-dimensional launch runs on
+int launch_xcd_probe(uint8_t *out, int workgroups, hipStream_t stream);
 
 // thread-local error text
 void set_error(const char *fmt, ...);

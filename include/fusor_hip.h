@@ -239,6 +239,21 @@ int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t com
  * is what the reference's [Sq, 0] x [0, D] product gives (fusor flash_attention.rs:141-199). */
 int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args);
 
+/* How a call would run on the split-KV decode kernels (for tests and benchmarks; no counterpart in the reference).
+ * is_decode 0: another kernel takes the call and the other fields are 0.  Otherwise: the cache is streamed by
+ * `nsplit` workgroups of `wavefronts` wavefronts per (batch, kv head, column block), `chunk` keys each, and the call
+ * is `kernels` launches: 1 when nothing is split or the splits are merged inside the main kernel (equal-length
+ * batches with 2 to 8 splits on the matrix-core variants, when the device deals the workgroups of a launch to its
+ * XCDs round-robin so that the splits of a unit can share an XCD's L2), else 2 (a log-sum-exp merge kernel follows). */
+typedef struct {
+    int32_t is_decode;
+    int32_t nsplit;
+    int32_t chunk;
+    int32_t wavefronts;
+    int32_t kernels;
+} fhip_decode_plan_info;
+int fhip_flash_attention_decode_plan(fhip_stream *s, const fhip_attn_args *args, fhip_decode_plan_info *info);
+
 /* fhip_flash_attention for callers that cannot allocate: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and same kernels,
  * but the workspace is a fixed array of FHIP_NOALLOC_WORKSPACE_BYTES of device

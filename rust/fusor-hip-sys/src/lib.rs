@@ -123,6 +123,17 @@ pub struct fhip_attn_args {
     pub main_kernel_start: *mut fhip_event,
 }
 
+/// How a call would run on the split-KV decode kernels (`fhip_flash_attention_decode_plan`).
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default, PartialEq, Eq)]
+pub struct fhip_decode_plan_info {
+    pub is_decode: i32,
+    pub nsplit: i32,
+    pub chunk: i32,
+    pub wavefronts: i32,
+    pub kernels: i32,
+}
+
 #[repr(C)]
 #[derive(Clone, Copy)]
 pub struct fhip_device_info {
@@ -200,6 +211,11 @@ unsafe extern "C" {
         args: *const fhip_attn_args,
         compute_units: i32,
         bytes: *mut usize,
+    ) -> c_int;
+    pub fn fhip_flash_attention_decode_plan(
+        s: *mut fhip_stream,
+        args: *const fhip_attn_args,
+        info: *mut fhip_decode_plan_info,
     ) -> c_int;
     pub fn fhip_flash_attention(s: *mut fhip_stream, args: *const fhip_attn_args) -> c_int;
     pub fn fhip_flash_attention_noalloc(s: *mut fhip_stream, args: *const fhip_attn_args) -> c_int;
@@ -345,6 +361,7 @@ const _: () = {
     assert!(core::mem::size_of::<fhip_analytic_mask>() == 24);
     assert!(core::mem::size_of::<fhip_attn_args>() == 384);
     assert!(core::mem::size_of::<fhip_device_info>() == 240);
+    assert!(core::mem::size_of::<fhip_decode_plan_info>() == 20);
     assert!(core::mem::size_of::<fhip_rope_tables>() == 40);
     assert!(core::mem::size_of::<fhip_rms_norm>() == 24);
 };

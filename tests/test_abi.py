@@ -199,9 +199,11 @@ def test_workspace_bytes():
     L = fa.lib()
     a = make_args(B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128)
     assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
-    assert need.value > 0 and need.value % (16 * 32 * (128 + 2) * 4) == 0
-    nsplit = need.value // (16 * 32 * (128 + 2) * 4)
-    assert 2 <= nsplit <= 16
+    # (partials of D + 2 floats per (batch, head, split); up to 8 splits a little more: every split's partials start on a
+    # 128-byte line and every (batch, kv head) has an arrival counter, for the merge inside the main kernel)
+    per = 16 * 32 * (128 + 2) * 4
+    nsplit = need.value // per
+    assert 2 <= nsplit <= 16 and need.value - nsplit * per <= 16 * 8 * (nsplit * 128 + 4) + 256
     a = make_args(Sq=512, Skv=512, D=128)
     assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK and need.value == 0
     # a decode call without the workspace it needs must fail before any launch (stream is checked first)
@@ -219,8 +221,10 @@ def test_decode_split_planning_on_256_cus():
         a = make_args(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D, dtype=dtype)
         assert L.fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK
         per = B * H * (D + 2) * 4
-        assert need.value % per == 0
-        return need.value // per
+        ns = need.value // per
+        # more than 8 splits: the partials exactly; up to 8 the padding and counters of the merge inside the main kernel
+        assert need.value == ns * per if ns > 8 or ns == 0 else need.value - ns * per <= B * Hkv * (ns * 128 + 4) + 256
+        return ns
 
     assert splits(16, 32, 8, 4096, 128, fa.F16) == 4     # C2
     assert splits(1, 32, 8, 4096, 128, fa.F16) == 32     # one stream, 128-key steps

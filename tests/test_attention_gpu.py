@@ -771,11 +771,15 @@ def test_decode_with_a_unit_per_cu_takes_the_eight_wavefront_form(device, dtype,
     q, k, v = _normal_qkv(47, B, H, Hkv, Sq, Skv, D, 0.5)
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
     assert tq.selected_kernel(tk, tv, 0.1) == fa.KERNEL_DECODE_SPLITKV
-    # three splits of 2048 keys per (batch, head, row): that is what the workspace is sized for
+    # three splits of 2048 keys per (batch, head, row) on eight wavefronts; the workspace holds their partials (and, up to
+    # 8 splits, the padding and counters of the merge inside the main kernel)
+    plan = tq.decode_plan(tk, tv, 0.1)
+    assert (plan["nsplit"], plan["chunk"], plan["wavefronts"]) == (3, 2048, 8), plan
     need = ctypes.c_size_t()
     args = tq._attn_args(tk, tv, 0.1, None, None, None, None, fa.KERNEL_AUTO, None)
     fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
-    assert need.value == B * H * Sq * 3 * (D + 2) * 4
+    partials = B * H * Sq * 3 * (D + 2) * 4
+    assert partials <= need.value <= partials + B * Hkv * (3 * 128 + 4) + 256
     tol = TOL_F32 if dtype == fa.F32 else (dict(max_abs=1e-2, rel_l2=5e-3) if dtype == fa.BF16 else TOL_16)
     analytic = (True, Skv - Sq, 0) if Sq > 1 else None
     mask = _analytic_mask(Sq, Skv, True, Skv - Sq, 0) if Sq > 1 else None
