@@ -4,13 +4,14 @@
 // Keys/values are walked in tiles of 64 rows that go from global memory straight into a three-stage
 // LDS ring (direct-to-LDS buffer loads, no staging registers).  Per tile and wavefront:
 //   S^T (64 keys x 32 queries)  = K_tile . Q^T      v_mfma_f32_32x32x16  (A = K from LDS, B = Q in registers)
-//   Q is multiplied once by the power-of-two part of scale * log2(e) (exact); the rest, a factor in [1, 2),
-//   multiplies the scores in f32.  The first MFMA of a tile takes -m (the running row maximum) as its C
-//   operand, so the accumulators come out relative to the maximum: one multiply per score, then exp2
-//   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of
-//   it per 32-key block, so the row max / row sum are in-lane folds plus one exchange with the
-//   lane 32 away (v_permlane32_swap); the running maximum is only moved (and O rescaled) when a
-//   tile exceeds it by more than 2^8
+//   Q is multiplied once by the power-of-two part of scale * log2(e) (exact); the rest, a factor rr in [1, 2),
+//   multiplies the scores in f32: a probability is exp2(fma(s, rr, -m * rr)), one fused multiply-add and one
+//   exponential per score, with m the row's reference exponent
+//   online softmax down the key axis: with S^T every lane owns ONE query column and 16 keys of it per 32-key
+//   block, so row sums are in-lane folds (the two half-rows are added once, at the end).  No maximum is taken
+//   per tile: the reference m is the maximum the row had when it was last set, and it is moved (and l and O
+//   rescaled) only when a lane's probabilities of a tile sum to more than 2^15, i.e. before one of them could
+//   leave the 16-bit type's range; on random data that is the first tile and almost never again
 //   O^T (D x 32 queries)       += V_tile^T . P^T    A = V^T read from row-major LDS with the
 //   transposing LDS load ds_read_b64_tr_b16, B = P^T taken straight from the S^T accumulator
 //   registers (the contraction index is permuted identically on both operands)
@@ -118,11 +119,6 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// Rows whose running maximum is stale by at most this much (log2 domain) keep it: probabilities
-// then reach 2^8 at most, well inside f16/bf16 range, and the 64-register rescale of O is skipped
-// on almost every tile.
-constexpr float PF_RESCALE_SLACK = 8.0f;
-
 template <typename T, int D, bool KS>
 __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnParams p, int nqb, int out_vec) {
     typedef PfCfg<D, KS> C;
@@ -188,10 +184,9 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     // rr multiplies every score in f32 right before exp2: the scores are then the f32 dot product times the scale, one
     // rounding, as the reference computes them (fusor-ml/fusor/src/composite/flash_attention.rs:145).  Folding all of
     // scale2 into Q instead would save that multiply but round Q's elements a second time (11 bits in f16, 8 in bf16),
-    // an error that grows in proportion to the scores.  The S^T accumulators, m and negm are in units of 1 / rr.
+    // an error that grows in proportion to the scores.  The S^T accumulators and m are in units of 1 / rr.
     const float pw = __uint_as_float(__float_as_uint(scale2) & 0x7F800000u);
     const float rr = scale2 / pw;
-    const float slack_u = PF_RESCALE_SLACK / rr;
     vec8 qreg[D / 16];
     {
         const uint16_t *qp = (const uint16_t *)p.q + b * p.qs[0] + h * p.qs[1] + (int64_t)qrow * p.qs[2];
@@ -214,13 +209,13 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
     for (int db = 0; db < D / 32; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[db][r] = 0.0f;
-    // m: running row maximum (base-2 exponent units); negm = -m in every element (0 while m is still
-    // -inf): it is the C operand of the first S^T MFMA of every tile, so the accumulators come out as
-    // s - m and go straight into exp2
-    float m = -INFINITY, l = 0.0f;
-    float16_t negm;
+    // m: the row's reference exponent, in units of the S^T accumulators (1 / rr of a base-2 exponent): probabilities are
+    // exp2((s - m) * rr), formed as exp2(fma(s, rr, nmr)) with nmr = -m * rr.  While the row has seen no key m is -inf and
+    // nmr +inf, which sends the first tile with a visible key through the branch that sets m (see softmax below).
+    float m = -INFINITY, l = 0.0f, nmr = INFINITY;
+    float16_t zero16;
 #pragma unroll
-    for (int r = 0; r < 16; r++) negm[r] = 0.0f;
+    for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
 
     using std::integral_constant;
     // ---- tile movement: global -> LDS directly (no registers) --------------------------------------
@@ -306,7 +301,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
 #pragma unroll
             for (int t = 0; t < 2; t++) {
                 uint4_t raw = *LDS_PTR(uint4_t, kbase + t * 2 * C::ROWB + kb * 32);
-                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], kb == 0 ? negm : s[t]);
+                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, raw), qreg[kb], kb == 0 ? zero16 : s[t]);
             }
         }
     };
@@ -385,7 +380,7 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
             for (int t = 0; t < 2; t++)
-                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, ka[kb % PFK][t]), qreg[kb], kb == 0 ? negm : s[t]);
+                s[t] = Mma<T>::mfma(__builtin_bit_cast(vec8, ka[kb % PFK][t]), qreg[kb], kb == 0 ? zero16 : s[t]);
             if (kb + PFK < NKB) read_k(kb + PFK, ka[kb % PFK]);
             if (PV && kb >= NKB - 4 && kb < NKB - 2) read_v(kb + 4 - NKB, va[kb + 4 - NKB]);
         }
@@ -431,41 +426,47 @@ __global__ __launch_bounds__(64 * PF_WAVES, 2) void prefill_mfma_kernel(AttnPara
                     s[t][r] = (key >= klo && key < khi) ? s[t][r] : -INFINITY;
                 }
         }
-        // s holds (score - m) already; mx is the tile maximum relative to the running maximum
-        float mx = s[0][0];
+        // Probabilities against the reference the row already has; no maximum is taken.  The reference is whatever maximum
+        // the row had when it was last set, so a probability may exceed 1: harmless while it stays inside the 16-bit
+        // type's range (P is rounded to it for the second product; l and O are f32), and that is what the check below
+        // guarantees: a lane's 32 probabilities are positive, so while their sum is at most 2^15 each of them is.
+        auto probabilities = [&](float nm) __attribute__((always_inline)) {
+            float ts = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+            for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-        mx = half_swap_max(mx);
-        const bool first = (m == -INFINITY);  // no visible key so far (negm is 0 then)
-        const bool grow = first ? (mx > -INFINITY) : (mx > slack_u);
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float delta = grow ? mx : 0.0f;
-            const float corr = first ? 0.0f : __builtin_amdgcn_exp2f(-delta * rr);
-            m = grow ? (first ? mx : m + mx) : m;
+                for (int r = 0; r < 16; r += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], rr, nm));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], rr, nm));
+                    pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
+                    ts += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
+                }
+            return ts;
+        };
+        float ts = probabilities(nmr);
+        // Not at most 2^15 (which also catches the +inf and NaN a row without a reference produces): some row of the
+        // wavefront needs its reference moved.  Take the tile's maximum, move every row's reference to at least that,
+        // rescale what the row has accumulated, and form the tile's probabilities again.
+        if (__builtin_amdgcn_ballot_w64(!(ts <= 32768.0f)) != 0) {
+            float mx = s[0][0];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+            mx = half_swap_max(mx);
+            const float m_new = fmaxf(m, mx);
+            const float corr = (m == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m - m_new) * rr);
+            m = m_new;
             l *= corr;
 #pragma unroll
             for (int db = 0; db < D / 32; db++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[db][r] *= corr;
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) s[t][r] -= delta;
-            const float nm = (m == -INFINITY) ? 0.0f : -m;
-#pragma unroll
-            for (int r = 0; r < 16; r++) negm[r] = nm;
+            // still no visible key: the tile's probabilities are exp2(-inf) = 0 and the row stays without a reference
+            nmr = (m == -INFINITY) ? INFINITY : -m * rr;
+            ts = probabilities((m == -INFINITY) ? 0.0f : nmr);
         }
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[t][r] * rr);
-                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1] * rr);
-                pk[t][r >> 1] = Mma<T>::pack2(p0, p1);
-                l += p0 + p1;  // plain f32 adds: a dot-product instruction here would queue behind the MFMAs
-            }
+        l += ts;
     };
 
     // ---- slot schedule ---------------------------------------------------------------------------------
