@@ -406,6 +406,185 @@ def run_config(name, steps, warmup, with_cpu=True):
     return res
 
 
+# ---- a whole attention layer step around the call -----------------------------------------------------------------
+# What kalosm-llama runs per layer (models/kalosm-llama/src/raw/attention_layer.rs:217-280,400-455, raw/mod.rs:618-620):
+# q / k RMS-norm (blocks that have them), rotary embedding, KvCache::append, the mask tensor of the step from
+# MaskCache::get_mask, attention, output as [b, seq, heads * hd].  Here: fhip_kv_cache_qkv_rope_append (one launch) and
+# fhip_flash_attention with the mask TENSOR, through the C ABI, everything but the two calls prepared outside the clock.
+LAYER_STEPS = {
+    # one decode step at batch 1 on the f32 cache kalosm-llama keeps, about 4096 keys (the cache grows by one per step)
+    "L1": dict(kind="layer_decode", B=1, H=32, Hkv=8, n=1, start=4090, D=128, dtype="f32", norm=False),
+    # a 512-token prompt (C1's shape) into an empty cache, with q / k norms
+    "L2": dict(kind="layer_prompt", B=1, H=32, Hkv=8, n=512, start=0, D=64, dtype="f32", norm=True),
+}
+
+
+def run_layer_step(name, steps, warmup, with_cpu=True):
+    import floneum_amd as fa
+    from floneum_amd import synth
+    import oracle
+
+    c = LAYER_STEPS[name]
+    L = fa.lib()
+    dev = fa.Device.default()
+    B, H, Hkv, n, D = c["B"], c["H"], c["Hkv"], c["n"], c["D"]
+    decode = c["kind"] == "layer_decode"
+    seed = SEED + 0x100 + int(name[1])
+    eb = 4
+    # the projections as the reference holds them: [b, seq, heads, hd], viewed as [b, heads, seq, hd]
+    qh = synth.normal(seed, 0, (B, n, H, D), 1.0, np.float32)
+    kh = synth.normal(seed, 1, (B, n, Hkv, D), 1.0, np.float32)
+    vh = synth.normal(seed, 2, (B, n, Hkv, D), 1.0, np.float32)
+    tq, tk, tv = (fa.Tensor.from_numpy(dev, a, fa.F32).transpose(1, 2) for a in (qh, kh, vh))
+    ctx = 8192
+    rope = fa.RopeCache(D, ctx, 10000.0, dev)
+    qw = kw = None
+    qn = kn = None
+    if c["norm"]:
+        qw = synth.normal(seed, 3, (D,), 0.2, np.float32) + np.float32(1.0)
+        kw = synth.normal(seed, 4, (D,), 0.2, np.float32) + np.float32(1.0)
+        qn, kn = fa.RmsNorm(qw, None, 1e-6, fa.F32, dev), fa.RmsNorm(kw, None, 1e-6, fa.F32, dev)
+    cache = fa.KvCache(2, ctx, fa.F32, dev)
+    k0 = v0 = None
+    if decode:  # the context the step runs on: `start` cached positions (already rotated keys, as the cache holds them)
+        k0 = synth.normal(seed, 5, (B, Hkv, c["start"], D), 1.0, np.float32)
+        v0 = synth.normal(seed, 6, (B, Hkv, c["start"], D), 1.0, np.float32)
+        cache.append(dev, fa.Tensor.from_numpy(dev, k0, fa.F32), fa.Tensor.from_numpy(dev, v0, fa.F32))
+    q_out = fa.Tensor.empty(dev, (B, H, n, D), fa.F32)
+    out_buf = fa.Tensor.empty(dev, (B, n, H, D), fa.F32)  # what attention_wo multiplies, as [b, seq, heads * hd]
+    if decode:  # get_mask(1, pos, None): a [1, pos + 1] row of zeros; one row long enough for every step, narrowed per step
+        mask_t = fa.Tensor.from_numpy(dev, np.zeros((1, ctx), np.float32), fa.F32)
+    else:       # get_mask(n, 0, None), which MaskCache keeps per (seq_len, window)
+        mask_t = fa.MaskCache(fa.F32).get_mask_on_device(n, 0, None, dev).mask()
+    # argument blocks, filled once; per step only the position, the cache views and the mask width change
+    tables = rope._tables(c["start"], False)
+    cq, co, ck, cv = tq._c4(), q_out._c4(), tk._c4(), tv._c4()
+    ka, va = fa.CTensor4(), fa.CTensor4()
+    cqn, ckn = (qn._c(), kn._c()) if c["norm"] else (None, None)
+    pqn, pkn = (ctypes.byref(cqn), ctypes.byref(ckn)) if c["norm"] else (None, None)
+    last_len = c["start"] + n * (warmup + 2 * steps + 2) if decode else n
+    dummy = fa.Tensor(q_out.buffer, fa.F32, (B, Hkv, last_len, D), (0, 0, 0, 1))  # stands in for the cache views below
+    args = q_out._attn_args(dummy, dummy, D ** -0.5, (mask_t.narrow(1, 0, last_len) if decode else mask_t, fa.MaskKind.QKMask),
+                            None, None, None, fa.KERNEL_AUTO, out_buf.transpose(1, 2))
+    # one workspace for every step: the split-KV plan, and with it the size, changes with the cache length
+    need, most = ctypes.c_size_t(), 16
+    for length in (range(c["start"] + n, last_len + 1, n) if decode else [n]):
+        args.k.shape[2] = args.v.shape[2] = args.mask.shape[1] = length
+        fa.check(L.fhip_flash_attention_workspace_bytes(ctypes.byref(args), dev.compute_units, ctypes.byref(need)))
+        most = max(most, need.value)
+    ws = fa.Buffer(dev, most)
+    args.workspace, args.workspace_bytes = ws.ptr, ws.nbytes
+    pos = [c["start"]]
+
+    def step():
+        if not decode:
+            fa.check(L.fhip_kv_cache_reset(cache.handle))  # a new sequence; the cache keeps its memory
+            pos[0] = 0
+        tables.start_pos = pos[0]
+        fa.check(L.fhip_kv_cache_qkv_rope_append(cache.handle, dev.stream, pqn, pkn, ctypes.byref(tables), ctypes.byref(cq),
+                                                 fa.F32, ctypes.byref(co), fa.F32, ctypes.byref(ck), ctypes.byref(cv), fa.F32,
+                                                 ctypes.byref(ka), ctypes.byref(va)))
+        pos[0] += n
+        args.k, args.v = ka, va
+        if decode:
+            args.mask.shape[1] = pos[0]
+        fa.check(L.fhip_flash_attention(dev.stream, ctypes.byref(args)))
+
+    for _ in range(warmup):
+        step()
+    dev.synchronize()
+    len0 = pos[0]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    dev.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    keys_mean = (len0 + n * (steps + 1) / 2.0) if decode else float(n)  # keys the attention call of a step sees
+    # the attention kernel's own duration (events carried by its dispatch), in a second pass
+    starts = [Event(fa, dev) for _ in range(steps)]
+    dones = [Event(fa, dev) for _ in range(steps)]
+    for i in range(steps):
+        args.main_kernel_start, args.main_kernel_done = starts[i].h, dones[i].h
+        step()
+    args.main_kernel_start = args.main_kernel_done = None
+    dev.synchronize()
+    kernel_ms = np.array([dones[i].ms_since(starts[i]) for i in range(steps)])
+    for e in starts + dones:
+        L.fhip_event_destroy(e.h)
+    kid = ctypes.c_int32()
+    fa.check(L.fhip_flash_attention_select(ctypes.byref(args), ctypes.byref(kid)))
+
+    # algorithmic bytes of a step: every tensor a stage must read or write, once
+    # (rotation: q in, q out, new k / v in, new k / v into the cache, cos / sin rows; attention: q, K, V, mask tensor, out)
+    rot = eb * (2 * B * H * n * D + 4 * B * Hkv * n * D + 2 * n * (D // 2))
+    attn_of = lambda keys: eb * (2 * B * H * n * D + 2 * B * Hkv * keys * D + n * keys)  # noqa: E731
+    byts = rot + attn_of(keys_mean)
+    flops = 4 * D * H * B * (n * keys_mean if decode else n * (n + 1) / 2.0)
+
+    # spot check of one more step against the CPU checker's pieces
+    step()
+    dev.synchronize()
+    f32 = lambda t: np.asarray(t.to_numpy(), np.float32)  # noqa: E731
+    view = lambda cten: fa.Tensor(fa._View(dev, cten.ptr, cache), fa.F32, tuple(cten.shape), tuple(cten.stride), cten.offset)  # noqa: E731
+    k_all, v_all, q_rot = f32(view(ka)), f32(view(va)), f32(q_out)
+    p0 = pos[0] - n
+    q_in, k_in = qh.transpose(0, 2, 1, 3), kh.transpose(0, 2, 1, 3)
+    if c["norm"]:
+        q_in, k_in = oracle.rms_norm(q_in, qw, None, 1e-6), oracle.rms_norm(k_in, kw, None, 1e-6)
+    q_ref = oracle.rope(q_in, rope.cos_host, rope.sin_host, p0)
+    k_ref = oracle.rope(k_in, rope.cos_host, rope.sin_host, p0)
+    bit_exact = bool(np.array_equal(q_rot, q_ref) and np.array_equal(k_all[:, :, -n:], k_ref)
+                     and np.array_equal(v_all[:, :, -n:], vh.transpose(0, 2, 1, 3)))
+    mask = oracle.get_mask(n, p0, None)
+    ref = oracle.flash_attention(q_ref, np.ascontiguousarray(k_all), np.ascontiguousarray(v_all), D ** -0.5, mask, "qk")
+    got = f32(out_buf).reshape(B, n, H, D).transpose(0, 2, 1, 3)
+    err = float(np.abs(got - ref).max())
+
+    value = byts / (wall_ms * 1e-3) / 1e9
+    kmean = float(kernel_ms.mean())
+    roof = dict(bound="hbm", achieved=attn_of(keys_mean) / (kmean * 1e-3) / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"], roof["traffic_note"] = measured_traffic(name, fa.KERNEL_NAMES[kid.value])
+    roof.update(kernel=fa.KERNEL_NAMES[kid.value], kernel_ms_mean=kmean, kernel_ms_median=float(np.median(kernel_ms)),
+                kernel_ms_min=float(kernel_ms.min()),
+                note="the attention call's main kernel against the attention call's own algorithmic bytes")
+    res = dict(value=value, unit="GB/s", ms_per_step=wall_ms, roofline=roof,
+               config=dict(workload=name, kind=c["kind"], batch=B, q_heads=H, kv_heads=Hkv, q_len=n,
+                           kv_len=int(round(keys_mean)), head_dim=D, causal=True, q_norm_k_norm=c["norm"],
+                           calls_per_step="fhip_kv_cache_qkv_rope_append + fhip_flash_attention (mask tensor, output as "
+                                          "[b, seq, heads * hd])" + ("" if decode else ", after fhip_kv_cache_reset"),
+                           algorithmic_flops=int(flops), algorithmic_bytes=int(byts)),
+               dtype=c["dtype"], frac_of_roofline=value / PEAK_HBM_GBS, spot_check_max_abs_err=err,
+               rope_and_cache_rows_bit_exact=bit_exact)
+    if with_cpu:
+        # the same step on the CPU checker's restatements (rotation, cache append by concatenation as the reference does,
+        # mask, attention), a few steps
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        reps = 5 if decode else 3
+        ocache = oracle.KvCache(2, ctx)
+        if decode:
+            ocache.append(k0, v0)
+        dts = []
+        p = c["start"]
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            if not decode:
+                ocache, p = oracle.KvCache(2, ctx), 0
+            qi, ki = qh.transpose(0, 2, 1, 3), kh.transpose(0, 2, 1, 3)
+            if c["norm"]:
+                qi, ki = oracle.rms_norm(qi, qw, None, 1e-6), oracle.rms_norm(ki, kw, None, 1e-6)
+            qr = oracle.rope(qi, rope.cos_host, rope.sin_host, p)
+            kr = oracle.rope(ki, rope.cos_host, rope.sin_host, p)
+            kall, vall = ocache.append(kr, vh.transpose(0, 2, 1, 3))
+            m = oracle.get_mask(n, p, None)
+            oracle.flash_attention(qr, np.ascontiguousarray(kall), np.ascontiguousarray(vall), D ** -0.5, m, "qk")
+            p += n
+            dts.append(time.perf_counter() - t0)
+        res["cpu_baseline"] = dict(value=byts / float(np.median(dts)) / 1e9, unit="GB/s", cores=threads, kind="port",
+                                   sample=f"{reps} whole steps (norm, rotation, cache append by concatenation, mask, attention), median")
+    return res
+
+
 def calibration_copy(mib=256, reps=3):
     """A first KvCache.append is a plain copy of the appended tensor: reads `mib` MiB, writes `mib` MiB."""
     import floneum_amd as fa
@@ -538,7 +717,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="C2", choices=sorted(configs()))
+    ap.add_argument("--config", default="C2", choices=sorted(configs()) + sorted(LAYER_STEPS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the other configurations (C3 under \"prefill\"; C1, C4, C5 under \"configs\")")
@@ -572,7 +751,7 @@ def main():
         print(json.dumps({"mfma_calibration": calibration_mfma(a.calibration_mfma), "nominal_peak_tflops": PEAK_MFMA_F16_TFLOPS}))
         return
 
-    main_res = run_config(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
+    main_res = (run_layer_step if a.config in LAYER_STEPS else run_config)(a.config, a.steps, a.warmup, with_cpu=not a.no_cpu)
     if a.calibration_copy:
         calibration_copy()
     detail("workload", dict(main_res, steps=a.steps, warmup=a.warmup))
@@ -596,7 +775,8 @@ def main():
         # with the f32 cache kalosm-llama keeps; M1: C2's batch with four new rows per sequence; L1 / L2: a whole
         # attention layer step around the call; W2 / W3: Gemma-3's key length 256 in f16, no CPU leg)
         for name, (steps, warmup, cpu) in EXTRA_WORKLOADS.items():
-            r = run_config(name, steps, warmup, with_cpu=cpu and not a.no_cpu)
+            run = run_layer_step if name in LAYER_STEPS else run_config
+            r = run(name, steps, warmup, with_cpu=cpu and not a.no_cpu)
             r["steps"], r["warmup"] = steps, warmup
             detail("workload", r)
             others[name] = r
@@ -605,7 +785,8 @@ def main():
 
 # workloads beside C2 and C3 on the default run: name -> (steps, warm-up steps, CPU leg)
 EXTRA_WORKLOADS = {"C1": (200, 20, True), "C1M": (200, 20, False), "C4": (100, 100, True), "C5": (20, 3, True),
-                   "F2": (100, 10, True), "M1": (100, 10, True), "W2": (100, 10, False), "W3": (50, 100, False)}
+                   "F2": (100, 10, True), "M1": (100, 10, True), "L1": (200, 20, True), "L2": (200, 20, True),
+                   "W2": (100, 10, False), "W3": (50, 100, False)}
 
 
 def detail(kind, obj):

@@ -1153,6 +1153,12 @@ int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has
 
 struct fhip_tensor_cache_side {
     void *buf = nullptr;  // [B, Hkv, rows, D] contiguous; rows = allocated while growing, 2 * max_len once full
+    size_t bytes = 0;     // size of buf
+    // What a reset leaves behind: the sequence's buffer, kept for the next sequence's first buffers (the reference's
+    // device recycles freed buffers through an allocation cache, fusor-ml/core/src/device.rs:305-354; hipMalloc and
+    // hipFree cost more than a short prompt's whole attention call, and hipFree waits for the device).
+    void *spare = nullptr;
+    size_t spare_bytes = 0;
 };
 
 // Once the cache is full (max_sequence_len rows) it slides: the buffer holds 2 * max_len rows per (batch, head), the
@@ -1248,12 +1254,23 @@ int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequen
     return FHIP_OK;
 }
 
-static int kv_release(fhip_kv_cache *c) {
+// keep_memory: the larger of the current buffer and the spare stays with the cache as its spare
+static int kv_release(fhip_kv_cache *c, bool keep_memory) {
     int rc = FHIP_OK;
     if (hipSetDevice(c->dev->ordinal) != hipSuccess) rc = FHIP_ERR_HIP;
     for (int s = 0; s < 2; s++) {
-        if (c->side[s].buf && hipFree(c->side[s].buf) != hipSuccess) rc = FHIP_ERR_HIP;
-        c->side[s].buf = nullptr;
+        fhip_tensor_cache_side &S = c->side[s];
+        if (keep_memory && S.buf && S.bytes > S.spare_bytes) {
+            void *smaller = S.spare;
+            S.spare = S.buf, S.spare_bytes = S.bytes;
+            S.buf = smaller;
+        }
+        if (S.buf && hipFree(S.buf) != hipSuccess) rc = FHIP_ERR_HIP;
+        S.buf = nullptr, S.bytes = 0;
+        if (!keep_memory) {
+            if (S.spare && hipFree(S.spare) != hipSuccess) rc = FHIP_ERR_HIP;
+            S.spare = nullptr, S.spare_bytes = 0;
+        }
     }
     c->current = c->allocated = 0;
     c->sliding = false;
@@ -1265,18 +1282,18 @@ static int kv_release(fhip_kv_cache *c) {
 
 int fhip_kv_cache_destroy(fhip_kv_cache *c) {
     if (!c) return FHIP_OK;
-    int rc = kv_release(c);
+    int rc = kv_release(c, false);
     delete c;
     return rc;
 }
 
-// TensorCache::reset (tensor_cache.rs:39-43): drops the data, keeps the limits.
+// TensorCache::reset (tensor_cache.rs:39-43): drops the data, keeps the limits (and the memory, for the next sequence).
 int fhip_kv_cache_reset(fhip_kv_cache *c) {
     if (!c) {
         set_error("cache is NULL");
         return FHIP_ERR_INVALID_ARG;
     }
-    return kv_release(c);
+    return kv_release(c, true);
 }
 
 int fhip_kv_cache_current_seq_len(const fhip_kv_cache *c, uint64_t *len) {
@@ -1342,18 +1359,27 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
     // install them only after every launch into them was accepted: a failure on the way frees them and leaves the
     // cache (buffers, lengths, strides) exactly as it was.
     void *nb[2] = {nullptr, nullptr};
+    size_t nb_bytes[2] = {0, 0};
     auto drop_new = [&]() {
         for (int sd = 0; sd < 2; sd++)
             if (nb[sd]) (void)hipFree(nb[sd]);
     };
     auto alloc_new = [&](size_t bytes) -> int {
         for (int sd = 0; sd < 2; sd++) {
+            fhip_tensor_cache_side &S = c->side[sd];
+            if (S.spare && S.spare_bytes >= bytes) {  // what the last reset left (work queued on this stream before the
+                nb[sd] = S.spare;                      // reset is done with it before anything queued now writes to it)
+                nb_bytes[sd] = S.spare_bytes;
+                S.spare = nullptr, S.spare_bytes = 0;
+                continue;
+            }
             const hipError_t e = hipMalloc(&nb[sd], bytes);
             if (e != hipSuccess) {
                 nb[sd] = nullptr;
                 drop_new();
                 return fhip::hip_fail(e, "hipMalloc (KV cache buffers)");
             }
+            nb_bytes[sd] = bytes;
         }
         return FHIP_OK;
     };
@@ -1361,6 +1387,7 @@ static int kv_append_core(fhip_kv_cache *c, fhip_stream *s, const fhip_tensor4 *
         for (int sd = 0; sd < 2; sd++) {
             if (c->side[sd].buf) (void)hipFree(c->side[sd].buf);  // waits for the copies out of it
             c->side[sd].buf = nb[sd];
+            c->side[sd].bytes = nb_bytes[sd];
         }
     };
 

@@ -325,6 +325,10 @@ int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has
 typedef struct fhip_kv_cache fhip_kv_cache;
 int fhip_kv_cache_create(fhip_device *dev, fhip_dtype dtype, uint64_t max_sequence_len, fhip_kv_cache **out);
 int fhip_kv_cache_destroy(fhip_kv_cache *c);
+/* TensorCache::reset (tensor_cache.rs:39-43): the cache is empty again.  Its buffers stay with it and serve the next
+ * sequence's first buffers if they are large enough (no hipMalloc / hipFree per sequence); fhip_kv_cache_destroy frees
+ * them.  Views returned before the reset are dead, and the next append must be ordered after the work that read them
+ * (the same stream, or an event), as that work may still be running when reset returns. */
 int fhip_kv_cache_reset(fhip_kv_cache *c);
 int fhip_kv_cache_current_seq_len(const fhip_kv_cache *c, uint64_t *len);
 int fhip_kv_cache_allocated_seq_len(const fhip_kv_cache *c, uint64_t *len);
