@@ -92,8 +92,12 @@ def configs():
         "S2": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False),
         "S3": dict(kind="decode", B=1, H=32, Hkv=8, Sq=1, Skv=32768, D=128, dtype="f16", std=0.5, causal=False),
         # C1 as kalosm-llama really calls it: the mask comes as the [512, 512] tensor MaskCache::get_mask builds, not as
-        # a formula (interval scan + tiled kernel + the kernel for masks that are not intervals, which exits at once)
+        # a formula.  Timed as a model calls it layer after layer: the mask tensor comes with the interval table its owner computed
+        # when it built the mask (fhip_mask_intervals; MaskCache keeps both), so the calls run no scan of the mask.
+        # C1S: the same call without the table (scan of the mask in every call).
         "C1M": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True,
+                    mask_tensor=True, mask_table=True),
+        "C1S": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True,
                     mask_tensor=True),
         # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the f32 matrix-core
         # variant of the decode kernel; and a 16-bit cache with Gemma-3's key length 256 (the 16-bit matrix-core variant
@@ -197,7 +201,8 @@ def prepare(fa, dev, c, sets, lens_t):
         # the tensor the reference's MaskCache builds for this call, written on the device
         dt = {"f32": fa.F32, "f16": fa.F16}[c["dtype"]]
         off = c.get("q_pos_offset", c["Skv"] - c["Sq"])
-        mask = (fa.MaskCache(dt).get_mask_on_device(c["Sq"], off, c.get("window") or None, dev).mask(), fa.MaskKind.QKMask)
+        am = fa.MaskCache(dt).get_mask_on_device(c["Sq"], off, c.get("window") or None, dev)
+        mask = (am.mask(), fa.MaskKind.QKMask, am.intervals()) if c.get("mask_table") else (am.mask(), fa.MaskKind.QKMask)
     for (q, k, v) in sets:
         analytic = None
         if c["causal"] and mask is None:

@@ -67,7 +67,7 @@ class CAttnArgs(ctypes.Structure):
                 ("mask_kind", ctypes.c_int), ("mask", CTensor2), ("analytic", CAnalyticMask),
                 ("kv_lens", ctypes.c_void_p), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
                 ("force_kernel", ctypes.c_int32), ("main_kernel_done", ctypes.c_void_p),
-                ("main_kernel_start", ctypes.c_void_p)]
+                ("main_kernel_start", ctypes.c_void_p), ("mask_intervals", ctypes.c_void_p)]
 
 
 class CDecodePlanInfo(ctypes.Structure):
@@ -130,6 +130,8 @@ SYMBOLS = {
                                                 ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint64)]),
     "fhip_mask_get_mask": (ctypes.c_int, [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int32,
                                           ctypes.c_uint64, _P]),
+    "fhip_mask_intervals_bytes": (ctypes.c_int, [ctypes.c_uint32, ctypes.POINTER(ctypes.c_size_t)]),
+    "fhip_mask_intervals": (ctypes.c_int, [_P, ctypes.POINTER(CTensor2), ctypes.c_int, _P, ctypes.c_size_t]),
     "fhip_mask_get_analytic": (ctypes.c_int, [ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int32, ctypes.c_uint64,
                                               ctypes.POINTER(CAnalyticMask)]),
     "fhip_kv_cache_create": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_uint64, _PP]),
@@ -577,7 +579,10 @@ class Tensor:
         args.scale = float(np.float32(scale))
         keep = [out]
         if mask is not None:
-            m, kind = mask
+            m, kind, *table = mask  # (tensor, kind) or (tensor, kind, MaskIntervals of that tensor)
+            if table:
+                args.mask_intervals = table[0].buffer.ptr
+                keep.append(table[0])
             if m.device is not self.device:
                 raise AssertionError("Mask must be on the same device as other tensors")  # fusor :64
             if m.dtype != self.dtype:
@@ -641,6 +646,20 @@ def _host_mask(fn, dtype, rows, cols, *a):
     return host
 
 
+class MaskIntervals:
+    """The interval form of a mask tensor (fhip_mask_intervals), computed once for a mask that does not change and
+    passed with it as the third element of flash_attention's mask tuple: the call then skips its scan of the mask."""
+
+    def __init__(self, mask):
+        need = ctypes.c_size_t()
+        check(lib().fhip_mask_intervals_bytes(mask.shape[0], ctypes.byref(need)))
+        self.buffer = Buffer(mask.device, need.value)
+        cm = mask._c2()
+        check(lib().fhip_mask_intervals(mask.device.stream, ctypes.byref(cm), mask.dtype, ctypes.c_void_p(self.buffer.ptr),
+                                        need.value))
+        self.mask = mask  # the table describes this view and lives no longer than it
+
+
 class AttentionMask:
     """fusor::cache::AttentionMask (attention_mask.rs:9-83): wraps the 2-D additive mask tensor."""
 
@@ -648,6 +667,13 @@ class AttentionMask:
         self._mask = mask
         self.host = host          # the same values on the host (numpy), kept for inspection
         self.analytic = analytic  # CAnalyticMask equal to this mask, when it was built by MaskCache
+        self._intervals = None
+
+    def intervals(self):
+        """The mask's interval table, computed on first use and kept with the mask (which never changes)."""
+        if self._intervals is None:
+            self._intervals = MaskIntervals(self._mask)
+        return self._intervals
 
     @classmethod
     def causal(cls, device, seq_len, dtype=F32):

@@ -149,6 +149,10 @@ static int validate(const fhip_attn_args *a) {
             set_error("output stride %d is 0 (overlapping writes)", i);
             return FHIP_ERR_INVALID_ARG;
         }
+    if (a->mask_intervals && (a->mask_kind == FHIP_MASK_NONE || ((uintptr_t)a->mask_intervals & 15) != 0)) {
+        set_error("mask_intervals needs a mask tensor and a 16-byte aligned table");
+        return FHIP_ERR_INVALID_ARG;
+    }
     if (!std::isfinite(a->scale)) {
         set_error("scale must be finite");
         return FHIP_ERR_INVALID_ARG;
@@ -277,14 +281,17 @@ static bool prefill_f32_eligible(const fhip_attn_args *a) {
     return true;
 }
 
+// what fhip_mask_intervals leaves in the first word of its table when some row of the mask is not an interval
+constexpr int32_t MASK_TABLE_BAD = 1;
+
 // A dense mask reaches the tiled prefill kernels in interval form (mask_intervals.hip), which needs
 // device scratch: 16 bytes for the mark of a mask whose rows are not all intervals, then {lo, hi} per row.
 static size_t mask_scratch_bytes(const fhip_attn_args *a) {
-    if (a->mask_kind == FHIP_MASK_NONE) return 0;
+    if (a->mask_kind == FHIP_MASK_NONE || a->mask_intervals) return 0;  // no mask, or its interval form comes with the call
     return mask_intervals_bytes(a->mask_kind == FHIP_MASK_QK ? (int)a->q.shape[2] : (int)a->q.shape[0]);
 }
 static bool mask_scratch_ok(const fhip_attn_args *a, bool assume_workspace) {
-    if (a->mask_kind == FHIP_MASK_NONE || assume_workspace) return true;
+    if (a->mask_kind == FHIP_MASK_NONE || assume_workspace || a->mask_intervals) return true;
     return a->workspace && ((uintptr_t)a->workspace & 15) == 0 && a->workspace_bytes >= mask_scratch_bytes(a);
 }
 
@@ -920,19 +927,27 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         // f32-arithmetic kernel's mask-adding form (up to head_dim 128), else the general kernel.
         int32_t *bad = (int32_t *)args->workspace;
         int2 *iv = (int2 *)((char *)args->workspace + 16);
-        do p.bad_tag = (int32_t)s->dev->next_tag.fetch_add(1, std::memory_order_relaxed);
-        while (p.bad_tag == 0);
-        // A recorded call is replayed with the mark it was recorded with: a replay whose mask is not made of intervals
-        // would leave that mark behind for every later replay.  Under capture the word is therefore cleared first
-        // (by a kernel, which is what a graph may hold); an eager call's mark is new every time and needs no clearing.
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        FHIP_HIP_CHECK(hipStreamIsCapturing(s->s, &capturing));
-        if (capturing == hipStreamCaptureStatusActive) {
-            rc = launch_fill_zero_bytes(bad, 16, s->s);
+        if (args->mask_intervals) {
+            // the interval form came with the call (fhip_mask_intervals, computed once for a mask that does not change):
+            // no scan
+            bad = (int32_t *)args->mask_intervals;
+            iv = (int2 *)((char *)args->mask_intervals + 16);
+            p.bad_tag = MASK_TABLE_BAD;
+        } else {
+            do p.bad_tag = (int32_t)s->dev->next_tag.fetch_add(1, std::memory_order_relaxed);
+            while (p.bad_tag == 0);
+            // A recorded call is replayed with the mark it was recorded with: a replay whose mask is not made of intervals
+            // would leave that mark behind for every later replay.  Under capture the word is therefore cleared first
+            // (by a kernel, which is what a graph may hold); an eager call's mark is new every time and needs no clearing.
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            FHIP_HIP_CHECK(hipStreamIsCapturing(s->s, &capturing));
+            if (capturing == hipStreamCaptureStatusActive) {
+                rc = launch_fill_zero_bytes(bad, 16, s->s);
+                if (rc) return rc;
+            }
+            rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
             if (rc) return rc;
         }
-        rc = launch_mask_intervals(p, args->dtype, iv, bad, s->s);
-        if (rc) return rc;
         AttnParams pt = p;
         pt.iv = iv;
         pt.iv_bad = bad;
@@ -1127,6 +1142,44 @@ int fhip_mask_get_mask_device(fhip_stream *s, fhip_dtype dtype, uint32_t seq_len
     const uint64_t off = mask_offset(seq_len, seqlen_offset, has_window, window);
     FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
     return launch_mask_build(out_device, dtype, seq_len, off + seq_len, off, has_window ? 1 : 0, window, s->s);
+}
+
+int fhip_mask_intervals_bytes(uint32_t rows, size_t *bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    *bytes = mask_intervals_bytes((int)rows);
+    return FHIP_OK;
+}
+
+int fhip_mask_intervals(fhip_stream *s, const fhip_tensor2 *mask, fhip_dtype dtype, void *table, size_t table_bytes) {
+    if (!s || !mask || !dtype_ok(dtype) || !table) {
+        set_error("mask_intervals: NULL argument or bad dtype");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (mask->shape[0] > 0x7fffffffu || mask->shape[1] > 0x7fffffffu || (mask->shape[0] && mask->shape[1] && !mask->ptr)) {
+        set_error("mask_intervals: mask of [%u, %u] without a device pointer, or too large", mask->shape[0], mask->shape[1]);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (((uintptr_t)table & 15) != 0 || table_bytes < mask_intervals_bytes((int)mask->shape[0])) {
+        set_error("mask_intervals: the table must be 16-byte aligned and hold %zu bytes (got %zu)",
+                  mask_intervals_bytes((int)mask->shape[0]), table_bytes);
+        return FHIP_ERR_WORKSPACE;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    int rc = launch_fill_zero_bytes(table, 16, s->s);
+    if (rc) return rc;
+    AttnParams p;
+    memset(&p, 0, sizeof(p));
+    p.mask = (const char *)mask->ptr + mask->offset * (uint64_t)elem_bytes(dtype);
+    p.ms0 = mask->stride[0];
+    p.ms1 = mask->stride[1];
+    p.mask_kind = FHIP_MASK_QK;  // rows of the table = rows of the tensor, whichever kind it is used as
+    p.Sq = (int)mask->shape[0];
+    p.Skv = (int)mask->shape[1];
+    p.bad_tag = MASK_TABLE_BAD;
+    return launch_mask_intervals(p, dtype, (int2 *)((char *)table + 16), (int32_t *)table, s->s);
 }
 
 int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window, uint64_t window,

@@ -134,6 +134,12 @@ typedef struct {
      * dispatch cannot be recorded into a graph: with main_kernel_start set, a call on a stream that is being
      * captured fails with FHIP_ERR_UNSUPPORTED (main_kernel_done alone may be captured). */
     fhip_event *main_kernel_start;
+    /* Optional, with a mask tensor: the table fhip_mask_intervals computed for exactly this mask view.  The tiled
+     * prefill kernels then skip the scan of the mask (one launch and one pass over the tensor per call) and need no
+     * workspace for it.  For masks that do not change between calls: one mask tensor serves every layer of a forward
+     * pass, and MaskCache keeps its tensors for its lifetime.  The caller vouches that the mask's contents are what
+     * they were when the table was computed; decode calls ignore it. */
+    const void *mask_intervals;
 } fhip_attn_args;
 
 typedef enum {
@@ -309,6 +315,16 @@ int fhip_mask_get_mask(fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offse
 int fhip_mask_get_mask_device(fhip_stream *s, fhip_dtype dtype, uint32_t seq_len, uint64_t seqlen_offset,
                               int32_t has_window, uint64_t window, void *out_device);
 /* The analytic descriptor equal to get_mask(seq_len, seqlen_offset, window) (no tensor built). */
+/* The interval form of a mask tensor: for every row the run of keys where the mask is 0, if the row is zeros on one run
+ * of keys and -inf elsewhere (every mask MaskCache::get_mask builds, padding masks, block-diagonal masks), and a mark
+ * in the table's first word if some row is anything else (then calls that carry the table add the mask values like
+ * the reference, as they would have without it).  What fhip_flash_attention computes per call from a mask tensor and
+ * its workspace, computed once here: `table` is device memory of fhip_mask_intervals_bytes(mask->shape[0]) bytes,
+ * 16-byte aligned, to be passed as fhip_attn_args.mask_intervals together with the same mask view.  No counterpart in
+ * the reference.  Asynchronous on `s`. */
+int fhip_mask_intervals_bytes(uint32_t rows, size_t *bytes);
+int fhip_mask_intervals(fhip_stream *s, const fhip_tensor2 *mask, fhip_dtype dtype, void *table, size_t table_bytes);
+
 int fhip_mask_get_analytic(uint32_t seq_len, uint64_t seqlen_offset, int32_t has_window,
                            uint64_t window, fhip_analytic_mask *out);
 

@@ -256,7 +256,8 @@ class Tensor {
     /// out when it built the mask itself; it replaces the dense mask tensor.
     Tensor flash_attention(const Tensor &k, const Tensor &v, float scale,
                            std::optional<std::pair<const Tensor<2> *, MaskKind>> mask = std::nullopt,
-                           const fhip_analytic_mask *analytic = nullptr, const int32_t *kv_lens = nullptr) const {
+                           const fhip_analytic_mask *analytic = nullptr, const int32_t *kv_lens = nullptr,
+                           const void *mask_intervals = nullptr) const {
         static_assert(R == 4, "flash_attention takes rank-4 tensors");
         if (!device().same(k.device()) || !device().same(v.device()))
             throw Panic("Cannot mix tensors of different devices");  // fusor lib.rs:265
@@ -273,6 +274,7 @@ class Tensor {
                 throw Panic("Mask must be on the same device as other tensors");  // fusor flash_attention.rs:64
             a.mask = mask->first->c2();
             a.mask_kind = (fhip_mask_kind)mask->second;
+            a.mask_intervals = mask_intervals;  // AttentionMask::intervals() of this very mask, or nullptr
         }
         if (analytic) a.analytic = *analytic;
         a.kv_lens = kv_lens;
@@ -295,6 +297,7 @@ class Tensor {
 class AttentionMask {
     Tensor<2> mask_;
     std::optional<fhip_analytic_mask> analytic_;
+    std::shared_ptr<Buffer> intervals_;  // the mask's interval table, computed on first use (the mask never changes)
 
    public:
     AttentionMask() = default;
@@ -310,6 +313,18 @@ class AttentionMask {
     }
     const Tensor<2> &mask() const { return mask_; }
     const std::optional<fhip_analytic_mask> &analytic() const { return analytic_; }
+    /// The table fhip_mask_intervals computes for this mask, to be passed to flash_attention with it: the calls then
+    /// skip their scan of the tensor (one mask serves every layer of a forward pass).
+    const void *intervals() {
+        if (!intervals_) {
+            size_t bytes = 0;
+            check(fhip_mask_intervals_bytes(mask_.shape()[0], &bytes));
+            intervals_ = std::make_shared<Buffer>(mask_.device(), bytes);
+            const fhip_tensor2 view = mask_.c2();
+            check(fhip_mask_intervals(mask_.device().stream(), &view, (fhip_dtype)mask_.dtype(), intervals_->ptr(), bytes));
+        }
+        return intervals_->ptr();
+    }
 };
 
 /// fusor::cache::MaskCache (mask_cache.rs:9-116): base masks cached by (seq_len, window)

@@ -121,6 +121,7 @@ pub struct fhip_attn_args {
     pub force_kernel: i32,
     pub main_kernel_done: *mut fhip_event,
     pub main_kernel_start: *mut fhip_event,
+    pub mask_intervals: *const c_void,
 }
 
 /// How a call would run on the split-KV decode kernels (`fhip_flash_attention_decode_plan`).
@@ -267,6 +268,14 @@ unsafe extern "C" {
         window: u64,
         out_device: *mut c_void,
     ) -> c_int;
+    pub fn fhip_mask_intervals_bytes(rows: u32, bytes: *mut usize) -> c_int;
+    pub fn fhip_mask_intervals(
+        s: *mut fhip_stream,
+        mask: *const fhip_tensor2,
+        dtype: fhip_dtype,
+        table: *mut c_void,
+        table_bytes: usize,
+    ) -> c_int;
     pub fn fhip_mask_get_analytic(
         seq_len: u32,
         seqlen_offset: u64,
@@ -359,7 +368,7 @@ const _: () = {
     assert!(core::mem::size_of::<fhip_tensor4>() == 64);
     assert!(core::mem::size_of::<fhip_tensor2>() == 40);
     assert!(core::mem::size_of::<fhip_analytic_mask>() == 24);
-    assert!(core::mem::size_of::<fhip_attn_args>() == 384);
+    assert!(core::mem::size_of::<fhip_attn_args>() == 392);
     assert!(core::mem::size_of::<fhip_device_info>() == 240);
     assert!(core::mem::size_of::<fhip_decode_plan_info>() == 20);
     assert!(core::mem::size_of::<fhip_rope_tables>() == 40);

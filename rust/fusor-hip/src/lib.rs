@@ -164,6 +164,21 @@ impl Drop for Buffer {
     }
 }
 
+impl<D: HipDataType> HipTensor<2, D> {
+    /// For a mask tensor whose contents will not change (a block-diagonal or padding mask built once and passed to
+    /// every layer of a forward pass): computes its interval table once, so that the attention calls it is passed
+    /// to skip their scan of the tensor.
+    pub fn with_mask_intervals(mut self) -> Result<Self> {
+        let mut bytes = 0usize;
+        check(unsafe { fhip_mask_intervals_bytes(self.shape[0] as u32, &mut bytes) })?;
+        let table = self.device.alloc(bytes)?;
+        let view = self.as_ffi();
+        check(unsafe { fhip_mask_intervals(self.device.stream(), &view, D::FHIP_DTYPE, table.ptr(), bytes) })?;
+        self.intervals = Some(table);
+        Ok(self)
+    }
+}
+
 /// Describes how to interpret a 2D attention mask (reference: fusor flash_attention.rs:11-19).
 #[derive(Debug, Clone, Copy, PartialEq, Eq)]
 pub enum MaskKind {
@@ -192,6 +207,8 @@ pub struct HipTensor<const R: usize, D> {
     strides: [i64; R],
     /// Set by `MaskCache::get_mask`: the formula this (mask) tensor was built from.
     analytic: Option<fhip_analytic_mask>,
+    /// Set by `with_mask_intervals`: the interval table of this (mask) tensor (`fhip_mask_intervals`).
+    intervals: Option<Arc<Buffer>>,
     _elem: PhantomData<D>,
 }
 
@@ -218,6 +235,7 @@ impl<const R: usize, D: HipDataType> HipTensor<R, D> {
             shape,
             strides: contiguous_strides(shape),
             analytic: None,
+            intervals: None,
             _elem: PhantomData,
         })
     }
@@ -287,6 +305,7 @@ impl<D: HipDataType> HipTensor<4, D> {
             shape: t.shape.map(|x| x as usize),
             strides: t.stride,
             analytic: None,
+            intervals: None,
             _elem: PhantomData,
         }
     }
@@ -319,6 +338,10 @@ impl<D: HipDataType> HipTensor<4, D> {
                 _ => {
                     a.mask = m.as_ffi();
                     a.mask_kind = kind.ffi();
+                    // the table computed once for this mask: the call does not scan the tensor again
+                    if let Some(table) = &m.intervals {
+                        a.mask_intervals = table.ptr();
+                    }
                 }
             }
         }

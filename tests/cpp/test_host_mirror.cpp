@@ -57,6 +57,18 @@ static void test_flash_attention_cpu_with_mask(const Device &d) {  // :241-276
     EXPECT(std::fabs(out[1] - 2.0f) < 0.01f, "row 0 should equal V[0]: %f", out[1]);
 }
 
+// the same call with the mask's interval table computed once (AttentionMask::intervals) and passed with the tensor
+static void test_flash_attention_with_mask_and_its_interval_table(const Device &d) {
+    auto q = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), k = t4(d, {1, 0, 0, 1}, 1, 1, 2, 2), v = t4(d, {1, 2, 3, 4}, 1, 1, 2, 2);
+    auto am = AttentionMask::causal(d, 2);
+    const void *table = am.intervals();
+    EXPECT(table != nullptr && table == am.intervals(), "the table is computed once");
+    auto plain = host(q.flash_attention(k, v, 1.0f / std::sqrt(2.0f), std::make_pair(&am.mask(), MaskKind::QKMask)));
+    auto out = host(q.flash_attention(k, v, 1.0f / std::sqrt(2.0f), std::make_pair(&am.mask(), MaskKind::QKMask), nullptr, nullptr, table));
+    for (int i = 0; i < 4; i++) EXPECT(out[i] == plain[i], "element %d: %f with the table, %f without", i, out[i], plain[i]);
+    EXPECT(std::fabs(out[0] - 1.0f) < 0.01f && std::fabs(out[1] - 2.0f) < 0.01f, "row 0 should equal V[0]: %f %f", out[0], out[1]);
+}
+
 static void test_flash_attention_gqa_cpu(const Device &d) {  // :278-313
     std::vector<float> q(16), k(8), v(8);
     for (int i = 0; i < 16; i++) q[i] = i * 0.1f;
@@ -272,6 +284,7 @@ int main() {
         Device d(0);
         test_flash_attention_cpu(d);
         test_flash_attention_cpu_with_mask(d);
+        test_flash_attention_with_mask_and_its_interval_table(d);
         test_flash_attention_gqa_cpu(d);
         test_flash_attention_cpu_with_batch_key_mask(d);
         test_attention_mask_causal(d);

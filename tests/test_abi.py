@@ -36,7 +36,7 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(fa.CTensor4) == 8 + 8 + 16 + 32
     assert ctypes.sizeof(fa.CTensor2) == 8 + 8 + 8 + 16
     assert ctypes.sizeof(fa.CAnalyticMask) == 24
-    assert ctypes.sizeof(fa.CAttnArgs) == 4 * 64 + 16 + 40 + 24 + 8 + 8 + 8 + 8 + 8 + 8
+    assert ctypes.sizeof(fa.CAttnArgs) == 4 * 64 + 16 + 40 + 24 + 8 + 8 + 8 + 8 + 8 + 8 + 8
 
 
 def t4(shape, strides=None, ptr=FAKE, offset=0):

@@ -30,8 +30,13 @@ def test_workloads_and_their_algorithmic_counts():
 
 def _fake_result(bench, name, with_cpu=True):
     """A record shaped like bench.run_config's, with long numbers and the longest texts the real ones carry."""
-    c = bench.configs()[name]
-    decode = c["kind"] == "decode"
+    if name in bench.LAYER_STEPS:
+        ls = bench.LAYER_STEPS[name]
+        c = dict(kind=ls["kind"], B=ls["B"], H=ls["H"], Hkv=ls["Hkv"], Sq=ls["n"], Skv=ls["start"] + ls["n"], D=ls["D"],
+                 dtype=ls["dtype"], causal=True)
+    else:
+        c = bench.configs()[name]
+    decode = c["kind"] in ("decode", "layer_decode", "layer_prompt")
     roof = dict(bound="hbm" if decode else "mfma", achieved=5912.123456789, peak=8000.0, unit="GB/s" if decode else "TFLOP/s",
                 frac=0.7390154320987, traffic=270342052.36343193,
                 traffic_note="FETCH_SIZE 2.692e+08 B + WRITE_SIZE 1.114e+06 B per launch", kernel="decode_splitkv",

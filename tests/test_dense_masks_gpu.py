@@ -324,3 +324,73 @@ def test_strided_mask_views_on_the_two_form_kernel(device):
     tmt = fa.Tensor.from_numpy(device, np.ascontiguousarray(mask.T), fa.F32).transpose(0, 1)  # column-major mask
     out = tq.flash_attention(tk, tv, D ** -0.5, (tmt, fa.MaskKind.QKMask)).to_numpy()
     assert_parity(out, ref, TOL_F32, "transposed mask")
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F32, 64), (fa.F32, 128), (fa.F16, 128), (fa.F16, 160), (fa.BF16, 96)])
+@pytest.mark.parametrize("kind", ["get_mask", "window_after_cache", "bias", "batch_key", "empty_rows"])
+def test_interval_table_computed_once_and_passed_with_the_mask(device, dtype, D, kind):
+    """fhip_mask_intervals computes a mask tensor's interval form once; a call that carries the table skips its own scan
+    and needs no workspace for the mask.  Every call with the table gives bit for bit what the call without it gives
+    (interval masks on the tiled kernel, other masks added element by element), on repeated calls and in the no-alloc
+    entry point, and stays inside the gate against the CPU checker."""
+    B, H, Hkv, Sq = 2, 4, 2, 150
+    mkind, okind = fa.MaskKind.QKMask, "qk"
+    if kind == "get_mask":
+        mask = oracle.get_mask(Sq, 0, None)
+    elif kind == "window_after_cache":
+        mask = oracle.get_mask(Sq, 400, 200)
+    elif kind == "bias":
+        mask = np.random.default_rng(9).normal(0, 1, (Sq, 260)).astype(np.float32)
+        mask[:, 100:130] = NEG_INF
+    elif kind == "batch_key":
+        mask = np.zeros((B, 300), np.float32)
+        mask[0, 250:] = NEG_INF
+        mask[1, :40] = NEG_INF
+        mkind, okind = fa.MaskKind.BatchKeyMask, "batch_key"
+    else:
+        mask = oracle.get_mask(Sq, 100, None)
+        mask[7] = NEG_INF      # rows that see nothing give NaN with or without the table
+        mask[149] = NEG_INF
+    Skv = mask.shape[1]
+    q, k, v = _normal_qkv(91, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv, tm = _tensors(device, dtype, q, k, v, mask)
+    scale = D ** -0.5
+    plain = tq.flash_attention(tk, tv, scale, (tm, mkind)).to_numpy()
+    table = fa.MaskIntervals(tm)
+    # the call needs no workspace for the mask any more (what is left, if anything, is for a key split)
+    need, need_plain = ctypes.c_size_t(), ctypes.c_size_t()
+    args = tq._attn_args(tk, tv, scale, (tm, mkind, table), None, None, None, fa.KERNEL_AUTO, None)
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+    args = tq._attn_args(tk, tv, scale, (tm, mkind), None, None, None, fa.KERNEL_AUTO, None)
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need_plain)))
+    assert need.value + 16 + 8 * mask.shape[0] <= need_plain.value + 256
+    # and is served by the type's own tiled kernel even when it brings no workspace at all
+    assert tq.selected_kernel(tk, tv, scale, mask=(tm, mkind, table)) == (fa.KERNEL_PREFILL_F32 if dtype == fa.F32 else fa.KERNEL_PREFILL_MFMA)
+    for rep in range(3):
+        out = tq.flash_attention(tk, tv, scale, (tm, mkind, table)).to_numpy()
+        assert np.array_equal(out.view(np.uint8), plain.view(np.uint8)), f"{kind} rep {rep}: differs from the call without the table"
+    out_t = fa.Tensor.from_numpy(device, np.full(q.shape, 7.0, np.float32), dtype)
+    tq.flash_attention_noalloc(tk, tv, scale, out_t, (tm, mkind, table))
+    assert np.array_equal(out_t.to_numpy().view(np.uint8), plain.view(np.uint8)), f"{kind}: no-alloc entry point differs"
+    ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), scale, rounded(mask, dtype), okind)
+    if kind == "empty_rows":
+        assert np.isnan(out[:, :, [7, 149]]).all() and np.isnan(ref[:, :, [7, 149]]).all()
+        keep = np.setdiff1d(np.arange(Sq), [7, 149])
+        out, ref = out[:, :, keep], ref[:, :, keep]
+    assert_parity(out, ref, _tol(dtype), f"{kind} with the interval table")
+
+
+def test_interval_table_arguments_are_checked(device):
+    tm = fa.Tensor.from_numpy(device, oracle.get_mask(20, 0, None), fa.F32)
+    need = ctypes.c_size_t()
+    fa.check(fa.lib().fhip_mask_intervals_bytes(20, ctypes.byref(need)))
+    assert need.value >= 16 + 20 * 8 and need.value % 16 == 0
+    small = fa.Buffer(device, 64)
+    cm = tm._c2()
+    rc = fa.lib().fhip_mask_intervals(device.stream, ctypes.byref(cm), fa.F32, ctypes.c_void_p(small.ptr), 64)
+    assert rc == fa.ERR_WORKSPACE and str(need.value) in fa.lib().fhip_last_error().decode()
+    # a table without a mask tensor is refused
+    q = fa.Tensor.from_numpy(device, np.zeros((1, 2, 20, 64), np.float32), fa.F32)
+    args = q._attn_args(q, q, 0.1, None, None, None, None, fa.KERNEL_AUTO, None)
+    args.mask_intervals = small.ptr
+    assert fa.lib().fhip_flash_attention_validate(ctypes.byref(args)) == fa.ERR_INVALID_ARG
