@@ -42,8 +42,8 @@ KERNEL_SOURCES = {"decode_splitkv": "attn_decode.hip", "prefill_mfma": "attn_pre
                   "prefill_f32": "attn_prefill_f32.hip", "generic": "attn_generic.hip"}
 
 
-def source_hash(kernel):
-    path = os.path.join(ROOT, "floneum_amd", "csrc", KERNEL_SOURCES[kernel])
+def source_hash(kernel, source=None):
+    path = os.path.join(ROOT, "floneum_amd", "csrc", source or KERNEL_SOURCES[kernel])
     return hashlib.sha256(open(path, "rb").read()).hexdigest()
 
 
@@ -55,7 +55,7 @@ def measured_traffic(name, kernel):
         rec = None
     if not rec:
         return None, "no counter record for this configuration"
-    if rec.get("kernel") != kernel or rec.get("source_sha256") != source_hash(kernel):
+    if rec.get("kernel") != kernel or rec.get("source_sha256") != source_hash(kernel, rec.get("source")):
         return None, "the kernel source has changed since the counters were read"
     return float(rec["fetch_bytes"]) + float(rec["write_bytes"]), \
         f"FETCH_SIZE {rec['fetch_bytes']:.4g} B + WRITE_SIZE {rec['write_bytes']:.4g} B per launch"
@@ -99,6 +99,10 @@ def configs():
                     mask_tensor=True, mask_table=True),
         "C1S": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=512, Skv=512, D=64, dtype="f32", std=1.0, causal=True,
                     mask_tensor=True),
+        # C2 with its lengths given as a per-sequence array (all 4096): the same split, merged by a second kernel, which is
+        # how every split-KV decode call ran before the merge moved into the main kernel for equal-length batches
+        "C2K": dict(kind="decode", B=16, H=32, Hkv=8, Sq=1, Skv=4096, D=128, dtype="f16", std=0.5, causal=False,
+                    ragged=(4096, 4096)),
         # C2's batch with the f32 cache kalosm-llama really keeps (attention_layer.rs:400-403): the f32 matrix-core
         # variant of the decode kernel; and a 16-bit cache with Gemma-3's key length 256 (the 16-bit matrix-core variant
         # with one workgroup per CU)
@@ -457,10 +461,12 @@ def run_layer_step(name, steps, warmup, with_cpu=True):
         cache.append(dev, fa.Tensor.from_numpy(dev, k0, fa.F32), fa.Tensor.from_numpy(dev, v0, fa.F32))
     q_out = fa.Tensor.empty(dev, (B, H, n, D), fa.F32)
     out_buf = fa.Tensor.empty(dev, (B, n, H, D), fa.F32)  # what attention_wo multiplies, as [b, seq, heads * hd]
+    mask_table = None
     if decode:  # get_mask(1, pos, None): a [1, pos + 1] row of zeros; one row long enough for every step, narrowed per step
         mask_t = fa.Tensor.from_numpy(dev, np.zeros((1, ctx), np.float32), fa.F32)
-    else:       # get_mask(n, 0, None), which MaskCache keeps per (seq_len, window)
-        mask_t = fa.MaskCache(fa.F32).get_mask_on_device(n, 0, None, dev).mask()
+    else:       # get_mask(n, 0, None), which MaskCache keeps per (seq_len, window), with the interval table it keeps beside it
+        am = fa.MaskCache(fa.F32).get_mask_on_device(n, 0, None, dev)
+        mask_t, mask_table = am.mask(), am.intervals()
     # argument blocks, filled once; per step only the position, the cache views and the mask width change
     tables = rope._tables(c["start"], False)
     cq, co, ck, cv = tq._c4(), q_out._c4(), tk._c4(), tv._c4()
@@ -469,8 +475,8 @@ def run_layer_step(name, steps, warmup, with_cpu=True):
     pqn, pkn = (ctypes.byref(cqn), ctypes.byref(ckn)) if c["norm"] else (None, None)
     last_len = c["start"] + n * (warmup + 2 * steps + 2) if decode else n
     dummy = fa.Tensor(q_out.buffer, fa.F32, (B, Hkv, last_len, D), (0, 0, 0, 1))  # stands in for the cache views below
-    args = q_out._attn_args(dummy, dummy, D ** -0.5, (mask_t.narrow(1, 0, last_len) if decode else mask_t, fa.MaskKind.QKMask),
-                            None, None, None, fa.KERNEL_AUTO, out_buf.transpose(1, 2))
+    mask_arg = (mask_t.narrow(1, 0, last_len), fa.MaskKind.QKMask) if decode else (mask_t, fa.MaskKind.QKMask, mask_table)
+    args = q_out._attn_args(dummy, dummy, D ** -0.5, mask_arg, None, None, None, fa.KERNEL_AUTO, out_buf.transpose(1, 2))
     # one workspace for every step: the split-KV plan, and with it the size, changes with the cache length
     need, most = ctypes.c_size_t(), 16
     for length in (range(c["start"] + n, last_len + 1, n) if decode else [n]):
@@ -557,7 +563,8 @@ def run_layer_step(name, steps, warmup, with_cpu=True):
                config=dict(workload=name, kind=c["kind"], batch=B, q_heads=H, kv_heads=Hkv, q_len=n,
                            kv_len=int(round(keys_mean)), head_dim=D, causal=True, q_norm_k_norm=c["norm"],
                            calls_per_step="fhip_kv_cache_qkv_rope_append + fhip_flash_attention (mask tensor, output as "
-                                          "[b, seq, heads * hd])" + ("" if decode else ", after fhip_kv_cache_reset"),
+                                          "[b, seq, heads * hd])" + ("" if decode else " with the mask's interval table, after "
+                                                                     "fhip_kv_cache_reset"),
                            algorithmic_flops=int(flops), algorithmic_bytes=int(byts)),
                dtype=c["dtype"], frac_of_roofline=value / PEAK_HBM_GBS, spot_check_max_abs_err=err,
                rope_and_cache_rows_bit_exact=bit_exact)
@@ -675,37 +682,64 @@ def calibration_read(mib=256, slices=5, launches=60):
                 gbps=nbytes / us / 1e3, frac_of_peak=nbytes / us / 1e3 / PEAK_HBM_GBS)
 
 
+def calibration_xcd_map(workgroups=1024, show=32):
+    """Which XCD the workgroups of a one-dimensional launch run on (fhip_calibration_xcd_map), for a few launches in a
+    row with small launches of other sizes in between (a 1-, 3- and 13-workgroup launch of the same kernel), and whether
+    workgroups with the same number modulo 8 always share an XCD: what the decode kernels' merge inside the kernel
+    relies on."""
+    import floneum_amd as fa
+    dev = fa.Device.default()
+    L = fa.lib()
+    buf = fa.Buffer(dev, workgroups)
+    host = np.empty(workgroups, np.uint8)
+    rows = []
+    for before in (0, 1, 3, 13, 0, 5):
+        if before:
+            fa.check(L.fhip_calibration_xcd_map(dev.stream, before, ctypes.c_void_p(buf.ptr), workgroups))
+        fa.check(L.fhip_calibration_xcd_map(dev.stream, workgroups, ctypes.c_void_p(buf.ptr), workgroups))
+        fa.check(L.fhip_memcpy_d2h(dev.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(buf.ptr), workgroups))
+        rows.append(dict(workgroups_of_the_launch_before=before, xcd_of_first_workgroups="".join(str(int(x)) for x in host[:show]),
+                         xcds=int(len(set(host.tolist()))),
+                         same_number_modulo_8_same_xcd=bool(all(host[i] == host[i & 7] for i in range(workgroups)))))
+    return rows
+
+
 def record_traffic(name, fetch_csv, write_csv):
     """profiles/traffic.json entry of one configuration from the two counter CSVs (one counter per profiler run).
     The copy kernel of --calibration-copy moves 256 MiB each way; its counts give the bytes per count."""
     import csv
 
     def per_kernel(path, counter):
+        """kernel name -> (mean count over its dispatches, largest count)"""
         sums = {}
         for r in csv.DictReader(open(path)):
             if r["Counter_Name"] == counter:
                 sums.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
-        return {k: float(np.mean(v)) for k, v in sums.items()}
+        return {k: (float(np.mean(v)), float(np.max(v))) for k, v in sums.items()}
 
     copied = 256 * (1 << 20)
     out = {}
     kernel = None
     for key, path, counter in (("fetch_bytes", fetch_csv, "FETCH_SIZE"), ("write_bytes", write_csv, "WRITE_SIZE")):
         counts = per_kernel(path, counter)
-        copy = [v for k, v in counts.items() if "copy_rows_kernel" in k]
+        # the calibration copies are the largest copies of the run (a workload that appends to a KV cache copies too)
+        copy = [v[1] for k, v in counts.items() if "copy_rows_kernel" in k]
         assert copy, f"{path}: no copy_rows_kernel dispatches (run bench.py with --calibration-copy)"
-        per_count = copied / copy[0]
+        per_count = copied / max(copy)
         main = {k: v for k, v in counts.items() if any(t in k for t in ("decode_mfma", "decode_vec", "prefill_mfma_kernel",
-                                                                       "prefill_f32_kernel", "prefill_f32_wide", "attn_generic"))}
+                                                                       "prefill_mfma_wide_kernel", "prefill_f32_kernel",
+                                                                       "prefill_f32_wide", "attn_generic"))}
         assert len(main) == 1, f"{path}: expected one main kernel, found {sorted(main)}"
-        kname, count = next(iter(main.items()))
+        kname, (count, _) = next(iter(main.items()))
         out[key] = count * per_count
         out[key.replace("bytes", "bytes_per_count")] = per_count
         kernel = "decode_splitkv" if "decode" in kname else "prefill_mfma" if "prefill_mfma" in kname else \
             "prefill_f32" if "prefill_f32" in kname else "generic"
         out["kernel_symbol"] = kname
     out["kernel"] = kernel
-    out["source_sha256"] = source_hash(kernel)
+    # the file the kernel lives in (the wide-head 16-bit prefill kernel has one of its own)
+    out["source"] = "attn_prefill_mfma_wide.hip" if "prefill_mfma_wide" in out["kernel_symbol"] else KERNEL_SOURCES[kernel]
+    out["source_sha256"] = source_hash(kernel, out["source"])
     try:
         rec = json.load(open(TRAFFIC_RECORD))
     except (OSError, ValueError):
@@ -736,6 +770,8 @@ def main():
                          "WRITE_SIZE with")
     ap.add_argument("--calibration-read", action="store_true",
                     help="no benchmark: run the read-only streaming kernel over 256 MiB slices and print GB/s")
+    ap.add_argument("--calibration-xcd", action="store_true",
+                    help="no benchmark: print which XCD the workgroups of a few launches in a row run on")
     ap.add_argument("--calibration-mfma", nargs="?", type=float, const=0.0, default=None, metavar="SECONDS",
                     help="no benchmark: run the register-only matrix-core loop (f16 random operands at 100 / 84 / 67 %% "
                          "duty, zero operands, bf16) and print TFLOP/s and the shader clock held; with SECONDS, keep "
@@ -751,6 +787,10 @@ def main():
         return
     if a.calibration_read:
         print(json.dumps({"read_calibration": calibration_read(), "nominal_peak_gbps": PEAK_HBM_GBS}))
+        return
+    if a.calibration_xcd:
+        for row in calibration_xcd_map():
+            print(json.dumps(row))
         return
     if a.calibration_mfma is not None:
         print(json.dumps({"mfma_calibration": calibration_mfma(a.calibration_mfma), "nominal_peak_tflops": PEAK_MFMA_F16_TFLOPS}))

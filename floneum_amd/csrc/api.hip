@@ -1025,6 +1025,15 @@ int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_opera
     return launch_calibration_mfma(dtype, cus, duty_percent, rounds, random_operands ? 1 : 0, scratch, s->s);
 }
 
+int fhip_calibration_xcd_map(fhip_stream *s, uint32_t workgroups, void *out, size_t out_bytes) {
+    if (!s || !out || workgroups == 0 || workgroups > (1u << 20) || out_bytes < workgroups) {
+        set_error("calibration: NULL stream or out, or not 1..2^20 workgroups with a byte of `out` each");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return fhip::launch_xcd_probe((uint8_t *)out, (int)workgroups, s->s);
+}
+
 int fhip_calibration_read(fhip_stream *s, const void *src, size_t bytes, void *scratch, size_t scratch_bytes) {
     if (!s || !src || !scratch) {
         set_error("calibration: NULL stream, source or scratch");

@@ -289,6 +289,13 @@ int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
 int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
                           void *scratch, size_t scratch_bytes);
 
+/* Calibration for benchmarks (no counterpart in the reference): where the workgroups of a launch run.  A
+ * one-dimensional launch of `workgroups` workgroups (64 lanes each) stores, per workgroup, the id of the XCD it ran
+ * on (the XCC_ID hardware register) into the device bytes `out` (one per workgroup).  The split-KV decode kernels
+ * that merge their splits inside the kernel rely on workgroups with the same number modulo 8 sharing an XCD; this
+ * shows the dealing they rely on (the library checks it itself when a device handle is created).  Asynchronous on `s`. */
+int fhip_calibration_xcd_map(fhip_stream *s, uint32_t workgroups, void *out, size_t out_bytes);
+
 /* Calibration for benchmarks (no counterpart in the reference): a kernel that does nothing but read `bytes` of
  * device memory at `src` (16-byte aligned) once, with 16-byte non-temporal loads, eight in flight per lane: the
  * rate a streaming kernel of this shape can reach at most.  `scratch`: device memory of at least

@@ -232,6 +232,7 @@ unsafe extern "C" {
         scratch_bytes: usize,
     ) -> c_int;
 
+    pub fn fhip_calibration_xcd_map(s: *mut fhip_stream, workgroups: u32, out: *mut c_void, out_bytes: usize) -> c_int;
     pub fn fhip_calibration_read(
         s: *mut fhip_stream,
         src: *const c_void,
