@@ -15,9 +15,16 @@ import pytest
 import floneum_amd as fa
 import oracle
 from conftest import TOL_16, TOL_F32, assert_parity
-from test_attention_gpu import _analytic_mask, _normal_qkv, rounded
+from test_attention_gpu import _analytic_mask, rounded
 
 pytestmark = pytest.mark.gpu
+
+
+def _normal_qkv(seed, B, H, Hkv, Sq, Skv, D, scale=1.0):
+    """Seeded normals (numpy's generator: these caches are tens of millions of elements)."""
+    rng = np.random.default_rng(seed)
+    return tuple(rng.standard_normal(shp, dtype=np.float32) * np.float32(scale)
+                 for shp in ((B, H, Sq, D), (B, Hkv, Skv, D), (B, Hkv, Skv, D)))
 
 
 def _tol(dtype):
@@ -111,3 +118,83 @@ def test_fused_merge_replayed_from_a_graph(device):
         device.synchronize()
         assert np.array_equal(out.to_numpy().view(np.uint8), eager.view(np.uint8)), f"replay {rep}"
         _ = uq.flash_attention(uk, uv, D ** -0.5).to_numpy()  # another call's marks in the same workspace
+
+
+def test_fused_merge_on_two_streams_at_once(device):
+    """Two host threads, two streams of one device handle, each with a workspace of its own, queue decode steps whose
+    splits are merged inside the kernel, back to back and at the same time: the workgroups of both launches share the
+    chip.  Every result equals the one computed alone, bit for bit, and later decode calls still succeed (a workgroup
+    that found its unit spread over several XCDs would have failed them)."""
+    import threading
+    second = device.with_new_stream()
+    shapes = {0: (16, 32, 8, 4096, 128), 1: (24, 8, 4, 3000, 64)}
+    alone, tensors = {}, {}
+    for i, dev in ((0, device), (1, second)):
+        B, H, Hkv, Skv, D = shapes[i]
+        q, k, v = _normal_qkv(560 + i, B, H, Hkv, 1, Skv, D, 0.5)
+        tq, tk, tv = (fa.Tensor.from_numpy(dev, a, fa.F16) for a in (q, k, v))
+        assert tq.decode_plan(tk, tv, D ** -0.5)["kernels"] == 1
+        out = tq.flash_attention(tk, tv, D ** -0.5).to_numpy()
+        ref = oracle.flash_attention(rounded(q, fa.F16), rounded(k, fa.F16), rounded(v, fa.F16), D ** -0.5)
+        assert_parity(out, ref, TOL_16, f"stream {i}, alone")
+        alone[i], tensors[i] = out, (tq, tk, tv, D)
+    errors = []
+    start = threading.Barrier(2)
+
+    def work(i, dev):
+        try:
+            tq, tk, tv, D = tensors[i]
+            outs = [fa.Tensor.empty(dev, tq.shape, fa.F16) for _ in range(40)]
+            start.wait()
+            for o in outs:                                   # queued without waiting: the two streams' kernels overlap
+                tq.flash_attention(tk, tv, D ** -0.5, out=o)
+            for n, o in enumerate(outs):
+                if not np.array_equal(o.to_numpy().view(np.uint8), alone[i].view(np.uint8)):
+                    raise AssertionError(f"stream {i}, call {n}: differs from the call made alone")
+        except BaseException as e:  # noqa: BLE001 - handed to the main thread
+            errors.append((i, e))
+            start.abort()
+
+    threads = [threading.Thread(target=work, args=(0, device)), threading.Thread(target=work, args=(1, second))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+        assert not t.is_alive()
+    assert not errors, f"stream {errors[0][0]}: {errors[0][1]!r}"
+    for i, dev in ((0, device), (1, second)):                # the form is still on, and still right
+        tq, tk, tv, D = tensors[i]
+        assert tq.decode_plan(tk, tv, D ** -0.5)["kernels"] == 1
+        assert np.array_equal(tq.flash_attention(tk, tv, D ** -0.5).to_numpy().view(np.uint8), alone[i].view(np.uint8))
+
+
+def test_fused_merge_seeded_sweep(device):
+    """Shapes drawn from a fixed seed among those the merge inside the kernel serves (2 to 8 splits): unit counts that
+    are and are not multiples of 8, GQA groups 1 to 8, one to four new rows, head dims of both matrix-core variants,
+    all three element types, with and without a sliding window."""
+    rng = np.random.default_rng(0xFD5E)
+    fused = 0
+    for it in range(30):
+        dtype = [fa.F16, fa.BF16, fa.F32][it % 3]
+        D = int(rng.choice([32, 64, 96, 128, 192, 256]))
+        Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+        G = int(rng.choice([1, 2, 4, 8]))
+        rows = int(rng.choice([1, 1, 2, 4]))
+        B = int(rng.integers(64 // Hkv + 1, 160 // Hkv + 2))
+        Skv = int(rng.integers(600, 3500))
+        window = int(rng.integers(200, Skv)) if it % 4 == 3 else 0
+        q, k, v = (rng.standard_normal(shp, dtype=np.float32) * np.float32(0.5)
+                   for shp in ((B, Hkv * G, rows, D), (B, Hkv, Skv, D), (B, Hkv, Skv, D)))
+        tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+        analytic = (True, Skv - rows, window) if (rows > 1 or window) else None
+        kw = {} if analytic is None else {"analytic": analytic}
+        plan = tq.decode_plan(tk, tv, D ** -0.5, **kw)
+        if not (plan["is_decode"] and plan["kernels"] == 1 and plan["nsplit"] > 1):
+            continue
+        fused += 1
+        out = tq.flash_attention(tk, tv, D ** -0.5, **kw).to_numpy()
+        mask = None if analytic is None else _analytic_mask(rows, Skv, *analytic)
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5, mask,
+                                     None if mask is None else "qk")
+        assert_parity(out, ref, _tol(dtype), f"it{it} B{B} H{Hkv * G}/{Hkv} rows{rows} Skv{Skv} D{D} window{window} {plan}")
+    assert fused >= 12, fused
