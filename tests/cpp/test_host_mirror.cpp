@@ -268,6 +268,38 @@ static void test_multi_token_step_on_a_cache(const Device &d) {
 }
 
 // the benchmark's calibration entry points, called through the C header
+// A batched decode step whose splits are merged inside the kernel (one launch): 16 sequences x 8 KV heads = 128 units,
+// 4096 keys each.  All keys equal: every key weighs the same, and with V[b][g][j][e] = j % 7 + e the output is the mean
+// over j of that, whichever query it is for.
+static void test_batched_decode_step_merged_inside_the_kernel(const Device &d) {
+    const uint32_t B = 16, H = 32, Hkv = 8, S = 4096, D = 128;
+    std::vector<float> k((size_t)B * Hkv * S * D, 0.125f), v((size_t)B * Hkv * S * D);
+    for (size_t r = 0; r < (size_t)B * Hkv; r++)
+        for (uint32_t j = 0; j < S; j++)
+            for (uint32_t e = 0; e < D; e++) v[(r * S + j) * D + e] = (float)(j % 7) + (float)e;
+    std::vector<float> q((size_t)B * H * D);
+    for (size_t i = 0; i < q.size(); i++) q[i] = (float)((i * 37) % 11) * 0.1f - 0.5f;
+    auto tq = t4(d, q, B, H, 1, D), tk = t4(d, k, B, Hkv, S, D), tv = t4(d, v, B, Hkv, S, D);
+    fhip_attn_args a{};
+    a.q = tq.c4(), a.k = tk.c4(), a.v = tv.c4(), a.out = tq.c4();
+    a.dtype = a.out_dtype = FHIP_F32;
+    a.scale = 0.1f;
+    fhip_decode_plan_info plan{};
+    check(fhip_flash_attention_decode_plan(d.stream(), &a, &plan));
+    EXPECT(plan.is_decode == 1 && plan.nsplit >= 2 && plan.nsplit <= 8 && plan.kernels == 1, "plan: decode %d, %d splits, %d kernels",
+           plan.is_decode, plan.nsplit, plan.kernels);
+    double mean7 = 0;
+    for (uint32_t j = 0; j < S; j++) mean7 += j % 7;
+    mean7 /= S;
+    for (int rep = 0; rep < 3; rep++) {  // the workspace's arrival counters are reused from call to call
+        auto out = host(tq.flash_attention(tk, tv, 0.1f));
+        float worst = 0;
+        for (size_t r = 0; r < (size_t)B * H; r++)
+            for (uint32_t e = 0; e < D; e++) worst = std::fmax(worst, std::fabs(out[r * D + e] - (float)(mean7 + e)));
+        EXPECT(worst < 1e-3f, "call %d: output should be the mean of V over the keys, off by %g", rep, worst);
+    }
+}
+
 static void test_calibrations(const Device &d) {
     const size_t cus = (size_t)d.info().compute_units;
     Buffer scratch(d, cus * 1040), data(d, 1 << 20);
@@ -294,6 +326,7 @@ int main() {
         test_rms_norm(d);
         test_capture(d);
         test_multi_token_step_on_a_cache(d);
+        test_batched_decode_step_merged_inside_the_kernel(d);
         test_calibrations(d);
     } catch (const std::exception &e) {
         printf("exception: %s\n", e.what());
