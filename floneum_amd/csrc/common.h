@@ -173,6 +173,7 @@ struct RopeRows {
     int32_t norm_dtype;
     float eps;
     int32_t vec;  // rows and pointers allow the 16-byte forms (set by fill_row_job)
+    int32_t few;  // the wide normalised form with its rows per wavefront block divided by 1 or 4 (set by fill_row_job)
 };
 struct RowJobs {
     RopeRows job[3];

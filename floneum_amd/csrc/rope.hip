@@ -136,7 +136,11 @@ struct NormWaveLds {
     uint32_t pos[64];        // their positions (rows of the cos / sin tables, before pos0)
     float rms[64];
 };
-template <int D>
+// FEW: the block's rows divided by FEW (1 or 4: down to 8 / 4 / 2 rows at head_dim 64 / 128 / 256), for inputs whose
+// blocks of the full size would leave most SIMDs with one wavefront or none: a block's stages (fetch, fold, normalise,
+// store) run one after the other, so a prompt of a few hundred rows is bound by one block's latencies, not by the
+// arithmetic.
+template <int D, int FEW>
 __device__ __forceinline__ void norm_rope_rows_vec_body(const RopeRows &a, NormWaveLds *w) {
     constexpr int HALF = D / 2, CPR = D / 4, P = D + 1;
     static_assert(CPR <= 64 && 64 % CPR == 0 && D % 64 == 0, "head_dim 64, 128 or 256");
@@ -145,7 +149,7 @@ __device__ __forceinline__ void norm_rope_rows_vec_body(const RopeRows &a, NormW
     // steps = PSTEPS pair steps, all requested before the first is parked.
     constexpr int RS = 64 / CPR;
     constexpr int PRS = HALF <= 64 ? 64 / HALF : 1, PP = HALF <= 64 ? 1 : HALF / 64;
-    constexpr int RPW = D == 64 ? 32 : D == 128 ? 16 : 8;  // rows per block
+    constexpr int RPW = (D == 64 ? 32 : D == 128 ? 16 : 8) / FEW;  // rows per block
     constexpr int LSTEPS = RPW / RS, PSTEPS = RPW * PP / PRS;
     static_assert(RPW * P <= NORM_TILE_FLOATS, "tile");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
@@ -264,9 +268,15 @@ __device__ __forceinline__ void norm_rope_rows_vec_body(const RopeRows &a, NormW
     }
 }
 __device__ __forceinline__ void norm_rope_rows_vec_any(const RopeRows &a, NormWaveLds *w) {
-    if (a.shape[3] == 128) norm_rope_rows_vec_body<128>(a, w);
-    else if (a.shape[3] == 256) norm_rope_rows_vec_body<256>(a, w);
-    else norm_rope_rows_vec_body<64>(a, w);
+    if (a.few == 4) {
+        if (a.shape[3] == 128) norm_rope_rows_vec_body<128, 4>(a, w);
+        else if (a.shape[3] == 256) norm_rope_rows_vec_body<256, 4>(a, w);
+        else norm_rope_rows_vec_body<64, 4>(a, w);
+        return;
+    }
+    if (a.shape[3] == 128) norm_rope_rows_vec_body<128, 1>(a, w);
+    else if (a.shape[3] == 256) norm_rope_rows_vec_body<256, 1>(a, w);
+    else norm_rope_rows_vec_body<64, 1>(a, w);
 }
 
 // The general form of the normalised variant (any strides): a workgroup takes groups of rows; one lane per row folds the squares in the
@@ -420,16 +430,25 @@ void fill_row_job(RopeRows *out, const void *src, const int64_t ss[4], fhip_dtyp
     a.vec = D % 8 == 0 && D >= 8 && wide(src, ss, src_dtype) && wide(dst, ds, dst_dtype) &&
             (mode == 2 || (((uintptr_t)cos % 16) == 0 && ((uintptr_t)sin % 16) == 0));
     if (a.norm_w && !(D == 64 || D == 128 || D == 256)) a.vec = 0;  // the head dims the wide normalised form is built for
+    // fewer than two full-size blocks per SIMD of a 256-CU chip: a quarter of the rows per block, four times the blocks
+    const int64_t rows = (int64_t)shape[0] * shape[1] * shape[2];
+    const int64_t full = D == 64 ? 32 : D == 128 ? 16 : 8;
+    // a quarter of the rows per block below 2048 full blocks (an eighth measured slower: 33.8 against 31.9 us on a
+    // 512-token prompt step whose full blocks took 35.9 us)
+    a.few = a.norm_w && a.vec && rows < 2048 * full ? 4 : 1;
 }
 
 // rows per wavefront block of the wide normalised form (RPW in norm_rope_rows_vec_body)
-static int norm_rows_per_wave(int D) { return D == 64 ? 32 : D == 128 ? 16 : 8; }
+static int norm_rows_per_wave(const RopeRows &a) {
+    const int D = (int)a.shape[3];
+    return (D == 64 ? 32 : D == 128 ? 16 : 8) / (a.few > 1 ? a.few : 1);
+}
 
 static int64_t job_blocks(const RopeRows &a) {
     const int64_t rows = (int64_t)a.shape[0] * a.shape[1] * a.shape[2];
     if (rows == 0 || a.shape[3] == 0) return 0;
     if (a.norm_w) {
-        const int rpb = a.vec ? 4 * norm_rows_per_wave((int)a.shape[3]) : (a.shape[3] / 2 >= 256 ? 1 : 256 / (a.shape[3] / 2));
+        const int rpb = a.vec ? 4 * norm_rows_per_wave(a) : (a.shape[3] / 2 >= 256 ? 1 : 256 / (a.shape[3] / 2));
         return (rows + rpb - 1) / rpb;
     }
     const int64_t total = a.vec ? rows * (a.mode == 2 ? a.shape[3] / 4 : a.shape[3] / 8)
