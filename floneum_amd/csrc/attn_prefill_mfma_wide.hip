@@ -437,6 +437,8 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // Up to head_dim 192 a wavefront can hold 32 rows (two column blocks: every K and V operand read from LDS then feeds
     // two matrix instructions): 256-row workgroups where those still give every CU one (f16, 4096 x 4096 causal:
     // head_dim 160 497 -> 559 TFLOP/s, 192 450 -> 511; at 224 and 256 the registers do not suffice)
+    if (bm == PW_BM && prefill_mfma_rows32_takes(p))
+        return launch_prefill_mfma_rows32(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     const long wgs256 = (long)p.B * p.H * ((p.Sq + 255) / 256);
     const bool big = wgs256 >= p.cus;
     if (!p.pf_pack && !small && p.pf_nsplit <= 1 && p.D <= 192 && big) bm = 256;

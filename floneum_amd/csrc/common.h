@@ -125,6 +125,9 @@ int launch_prefill_mfma(const AttnParams &p, fhip_dtype dtype, hipStream_t strea
 // the same for head dims 160 / 192 / 224 / 256 (four wavefronts per workgroup, 128 query rows, 32-key tiles)
 int launch_prefill_mfma_wide(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 void prefill_mfma_wide_plan(int B, int H, int G, int Sq, int Skv, bool causal_square, int compute_units, int *nsplit, int *chunk);
+// head dims above 192 on 128-row workgroups of four wavefronts with 32 rows each (one per SIMD, software-pipelined)
+bool prefill_mfma_rows32_takes(const AttnParams &p);
+int launch_prefill_mfma_rows32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 // f32 arithmetic on the f32 matrix cores; `dtype` is the tensors' storage type (16-bit rows are widened on load)
 int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 
