@@ -727,7 +727,8 @@ def record_traffic(name, fetch_csv, write_csv):
         assert copy, f"{path}: no copy_rows_kernel dispatches (run bench.py with --calibration-copy)"
         per_count = copied / max(copy)
         main = {k: v for k, v in counts.items() if any(t in k for t in ("decode_mfma", "decode_vec", "prefill_mfma_kernel",
-                                                                       "prefill_mfma_wide_kernel", "prefill_f32_kernel",
+                                                                       "prefill_mfma_wide_kernel", "prefill_mfma_wide_rows32_kernel",
+                                                                       "prefill_f32_kernel",
                                                                        "prefill_f32_wide", "attn_generic"))}
         assert len(main) == 1, f"{path}: expected one main kernel, found {sorted(main)}"
         kname, (count, _) = next(iter(main.items()))
@@ -737,8 +738,9 @@ def record_traffic(name, fetch_csv, write_csv):
             "prefill_f32" if "prefill_f32" in kname else "generic"
         out["kernel_symbol"] = kname
     out["kernel"] = kernel
-    # the file the kernel lives in (the wide-head 16-bit prefill kernel has one of its own)
-    out["source"] = "attn_prefill_mfma_wide.hip" if "prefill_mfma_wide" in out["kernel_symbol"] else KERNEL_SOURCES[kernel]
+    # the file the kernel lives in (the wide-head 16-bit prefill kernels have files of their own)
+    out["source"] = "attn_prefill_mfma_rows32.hip" if "prefill_mfma_wide_rows32" in out["kernel_symbol"] else \
+        "attn_prefill_mfma_wide.hip" if "prefill_mfma_wide" in out["kernel_symbol"] else KERNEL_SOURCES[kernel]
     out["source_sha256"] = source_hash(kernel, out["source"])
     try:
         rec = json.load(open(TRAFFIC_RECORD))
