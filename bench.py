@@ -611,6 +611,37 @@ def calibration_copy(mib=256, reps=3):
         del cache
 
 
+ISSUE_MIXES = ["matrix instructions only", "a dependent chain of matrix instructions", "+ 4 v_fma", "+ 8 v_fma", "+ 4 v_exp",
+               "+ 4 scalar adds", "+ 1 ds_read_b128 (the operand 8 steps later)", "+ 3 ds_read_b128",
+               "+ 2 ds_read_b64_tr_b16 (used 8 steps later)", "+ 1 ds_read_b128 + 2 ds_read_b64_tr_b16",
+               "+ 1 ds_read_b128 + 2 ds_read_b64_tr_b16 + fma, exp2, add", "+ 2 ds_read_b128 + fma, exp2, add",
+               "+ 2 ds_read_b128 + 1/2 ds_read_b64_tr_b16 + 1/4 ds_write_b128"]
+
+
+def calibration_issue(rounds=20000):
+    """What one wavefront per SIMD can issue beside its matrix instructions (fhip_calibration_issue): shader-clock
+    cycles per step of one v_mfma_f32_32x32x16_f16 (32 cycles of the matrix pipe) and the named companions."""
+    import floneum_amd as fa
+    dev = fa.Device.default()
+    L = fa.lib()
+    cus = dev.compute_units
+    nbytes = cus * (256 * 4 + 16)
+    scratch = fa.Buffer(dev, nbytes)
+    host = np.empty(nbytes, np.uint8)
+    rows = []
+    for mix, what in enumerate(ISSUE_MIXES):
+        for r in (rounds // 10, rounds):  # the first brings the clock to where this load holds it
+            fa.check(L.fhip_calibration_issue(dev.stream, mix, r, ctypes.c_void_p(scratch.ptr), nbytes))
+        dev.synchronize()
+        fa.check(L.fhip_memcpy_d2h(dev.stream, host.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(scratch.ptr), nbytes))
+        ticks = host[cus * 1024:].view(np.uint64).reshape(cus, 2).astype(np.float64)
+        steps = 16.0 * rounds
+        rows.append(dict(mix=mix, companions=what, cycles_per_step=_r(float(np.median(ticks[:, 0])) / steps, 4),
+                         ns_per_step=_r(float(np.median(ticks[:, 1])) * 10.0 / steps, 4),
+                         sclk_ghz=_r(float(np.median(ticks[:, 0] / ticks[:, 1])) * 0.1, 4)))
+    return rows
+
+
 def calibration_mfma(seconds=0.0):
     """What the matrix cores deliver with nothing else in the way (fhip_calibration_mfma: a register-only loop of
     the prefill kernel's matrix instruction, one wavefront per SIMD), with the clock the chip held meanwhile.  The
@@ -774,6 +805,8 @@ def main():
                     help="no benchmark: run the read-only streaming kernel over 256 MiB slices and print GB/s")
     ap.add_argument("--calibration-xcd", action="store_true",
                     help="no benchmark: print which XCD the workgroups of a few launches in a row run on")
+    ap.add_argument("--calibration-issue", action="store_true",
+                    help="cycles per step of one matrix instruction and companions, one wavefront per SIMD (fhip_calibration_issue)")
     ap.add_argument("--calibration-mfma", nargs="?", type=float, const=0.0, default=None, metavar="SECONDS",
                     help="no benchmark: run the register-only matrix-core loop (f16 random operands at 100 / 84 / 67 %% "
                          "duty, zero operands, bf16) and print TFLOP/s and the shader clock held; with SECONDS, keep "
@@ -793,6 +826,10 @@ def main():
     if a.calibration_xcd:
         for row in calibration_xcd_map():
             print(json.dumps(row))
+        return
+    if a.calibration_issue:
+        for row in calibration_issue():
+            print(json.dumps(row), flush=True)
         return
     if a.calibration_mfma is not None:
         print(json.dumps({"mfma_calibration": calibration_mfma(a.calibration_mfma), "nominal_peak_tflops": PEAK_MFMA_F16_TFLOPS}))

@@ -123,6 +123,7 @@ SYMBOLS = {
     "fhip_flash_attention": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
     "fhip_flash_attention_noalloc": (ctypes.c_int, [_P, ctypes.POINTER(CAttnArgs)]),
     "fhip_calibration_mfma": (ctypes.c_int, [_P, ctypes.c_int, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _P, ctypes.c_size_t]),
+    "fhip_calibration_issue": (ctypes.c_int, [_P, ctypes.c_int32, ctypes.c_int32, _P, ctypes.c_size_t]),
     "fhip_calibration_xcd_map": (ctypes.c_int, [_P, ctypes.c_uint32, _P, ctypes.c_size_t]),
     "fhip_calibration_read": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P, ctypes.c_size_t]),
     "fhip_mask_causal": (ctypes.c_int, [ctypes.c_int, ctypes.c_uint32, _P]),

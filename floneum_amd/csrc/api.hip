@@ -1025,6 +1025,25 @@ int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_opera
     return launch_calibration_mfma(dtype, cus, duty_percent, rounds, random_operands ? 1 : 0, scratch, s->s);
 }
 
+int fhip_calibration_issue(fhip_stream *s, int32_t mix, int32_t rounds, void *scratch, size_t scratch_bytes) {
+    if (!s || !scratch) {
+        set_error("calibration: NULL stream or scratch");
+        return FHIP_ERR_INVALID_ARG;
+    }
+    if (mix < 0 || mix >= FHIP_CALIBRATION_ISSUE_MIXES || rounds < 1 || rounds > FHIP_CALIBRATION_MFMA_MAX_ROUNDS) {
+        set_error("calibration: mix %d must be in 0..%d and rounds %d in 1..%d", mix, FHIP_CALIBRATION_ISSUE_MIXES - 1, rounds,
+                  FHIP_CALIBRATION_MFMA_MAX_ROUNDS);
+        return FHIP_ERR_INVALID_ARG;
+    }
+    const int cus = s->dev->prop.multiProcessorCount;
+    if (scratch_bytes < calibration_mfma_bytes(cus) || ((uintptr_t)scratch & 15) != 0) {
+        set_error("calibration: scratch of %zu bytes, 16-byte aligned, needed (got %zu)", calibration_mfma_bytes(cus), scratch_bytes);
+        return FHIP_ERR_WORKSPACE;
+    }
+    FHIP_HIP_CHECK(hipSetDevice(s->dev->ordinal));
+    return launch_calibration_issue(mix, cus, rounds, scratch, s->s);
+}
+
 int fhip_calibration_xcd_map(fhip_stream *s, uint32_t workgroups, void *out, size_t out_bytes) {
     if (!s || !out || workgroups == 0 || workgroups > (1u << 20) || out_bytes < workgroups) {
         set_error("calibration: NULL stream or out, or not 1..2^20 workgroups with a byte of `out` each");

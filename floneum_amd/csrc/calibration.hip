@@ -126,6 +126,120 @@ int launch_calibration_read(const void *src, size_t bytes, int compute_units, vo
     return FHIP_OK;
 }
 
+// issue_probe_kernel: what ONE wavefront per SIMD can issue beside its matrix instructions.  A wavefront issues in order,
+// so in a kernel that runs a single wavefront per SIMD (attn_prefill_mfma_rows32.hip: Q and O^T of 32 rows at head_dim
+// 256 leave no registers for a second one) everything that is not a matrix instruction either fits into the 32 cycles
+// the matrix pipe is busy with the last one or is paid for in full.  The loop is steps of one v_mfma_f32_32x32x16_f16
+// on independent accumulators plus the companions `MIX` names, fenced so that the compiler keeps the steps apart; values
+// read from LDS are used eight steps later, as operands or by a vector instruction.
+template <int MIX>
+__global__ __launch_bounds__(256, 1) void issue_probe_kernel(float *sink, uint64_t *ticks, int rounds) {
+    __shared__ __attribute__((aligned(16))) char smem[49152];
+    auto lds = (__attribute__((address_space(3))) char *)smem;
+    for (int i = threadIdx.x; i < 49152 / 4; i += 256) ((__attribute__((address_space(3))) float *)lds)[i] = 1.0f;
+    __syncthreads();
+    const uint64_t c0 = clock64(), w0 = wall_clock64();
+    const int lane = threadIdx.x & 63;
+    float16_t acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+    half8_t a, b;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[e] = (half_t)(0.25f + 0.125f * e), b[e] = (half_t)0.5f;
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = 1.0f + i;
+    int addr = lane * 16;
+    asm volatile("" : "+v"(addr));  // one address register, immediate offsets
+    uint4_t la[8], lb[8], lc[8];
+    short4_t tr[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        la[i] = lb[i] = lc[i] = uint4_t{0, 0, 0, 0};
+        tr[i][0] = tr[i][1] = short4_t{0, 0, 0, 0};
+    }
+    int sacc = rounds;
+    constexpr bool OPERAND_FROM_LDS = MIX == 6 || MIX == 7 || MIX == 9 || MIX == 10 || MIX == 11 || MIX == 12;
+    for (int it = 0; it < rounds; it++) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const int i = k & 7;
+            if (MIX == 1) acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[0], 0, 0, 0);  // a dependent chain
+            else if (OPERAND_FROM_LDS) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, la[i]), b, acc[i], 0, 0, 0);
+            else acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+            if (MIX == 2 || MIX == 3) {
+#pragma unroll
+                for (int j = 0; j < (MIX == 2 ? 4 : 8); j++) x[j] = __builtin_fmaf(x[j], 1.0001f, 0.5f);
+            }
+            if (MIX == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) x[j] = __builtin_amdgcn_exp2f(x[j]);
+            }
+            if (MIX == 5) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) asm volatile("s_add_u32 %0, %0, 3" : "+s"(sacc) : : "scc");
+            }
+            if (OPERAND_FROM_LDS) la[i] = *(__attribute__((address_space(3))) uint4_t *)(lds + addr + i * 1024);
+            if (MIX == 7) {
+                lb[i] = *(__attribute__((address_space(3))) uint4_t *)(lds + 8192 + addr + i * 1024);
+                lc[i] = *(__attribute__((address_space(3))) uint4_t *)(lds + 16384 + addr + i * 1024);
+            }
+            if (MIX == 8 || MIX == 9 || MIX == 10) {
+                // (what the transposing reads of eight steps ago brought is consumed first)
+                x[i] += __builtin_bit_cast(float, (int)tr[i][0][0] | ((int)tr[i][1][0] << 16));
+                tr[i][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t *)(lds + 24576 + lane * 8 + i * 512));
+                tr[i][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t *)(lds + 32768 + lane * 8 + i * 512));
+            }
+            if (MIX == 10 || MIX == 11) {
+                x[(k + 1) & 7] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[(k + 1) & 7], 1.0001f, -0.5f));
+                x[(k + 2) & 7] += x[(k + 3) & 7];
+            }
+            if (MIX == 11 || MIX == 12) lb[i] = *(__attribute__((address_space(3))) uint4_t *)(lds + 8192 + addr + i * 1024);
+            if (MIX == 12) {
+                // a tile transposed once per workgroup instead of once per wavefront: this wavefront's share per step
+                // (half a transposing read, a quarter of a 16-byte write of what such reads brought eight steps ago)
+                if ((k & 1) == 0) tr[i][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t *)(lds + 24576 + lane * 8 + i * 512));
+                if ((k & 3) == 3) {
+                    const uint2_t u0 = __builtin_bit_cast(uint2_t, tr[(i + 1) & 7][0]), u1 = __builtin_bit_cast(uint2_t, tr[(i + 3) & 7][0]);
+                    *(__attribute__((address_space(3))) uint4_t *)(lds + 32768 + addr + (k >> 2) * 1024) = uint4_t{u0[0], u0[1], u1[0], u1[1]};
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float res = (float)sacc;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        res += x[i] + (float)la[i][0] + (float)lb[i][1] + (float)lc[i][2] + (float)tr[i][0][1] + (float)tr[i][1][2];
+#pragma unroll
+        for (int r = 0; r < 16; r++) res += acc[i][r];
+    }
+    const uint64_t c1 = clock64(), w1 = wall_clock64();
+    sink[blockIdx.x * 256 + threadIdx.x] = res;
+    if (threadIdx.x == 0) {
+        ticks[2 * blockIdx.x] = c1 - c0;
+        ticks[2 * blockIdx.x + 1] = w1 - w0;
+    }
+}
+
+int launch_calibration_issue(int mix, int compute_units, int rounds, void *scratch, hipStream_t stream) {
+    float *sink = (float *)scratch;
+    uint64_t *ticks = (uint64_t *)((char *)scratch + (size_t)compute_units * 256 * sizeof(float));
+    const dim3 grid((unsigned)compute_units);
+#define FHIP_ISSUE(M) \
+    case M: hipLaunchKernelGGL((issue_probe_kernel<M>), grid, dim3(256), 0, stream, sink, ticks, rounds); break
+    switch (mix) {
+        FHIP_ISSUE(0); FHIP_ISSUE(1); FHIP_ISSUE(2); FHIP_ISSUE(3); FHIP_ISSUE(4); FHIP_ISSUE(5);
+        FHIP_ISSUE(6); FHIP_ISSUE(7); FHIP_ISSUE(8); FHIP_ISSUE(9); FHIP_ISSUE(10); FHIP_ISSUE(11); FHIP_ISSUE(12);
+        default: set_error("calibration: mix %d is not one of 0..12", mix); return FHIP_ERR_INVALID_ARG;
+    }
+#undef FHIP_ISSUE
+    FHIP_HIP_CHECK(hipGetLastError());
+    return FHIP_OK;
+}
+
 size_t calibration_mfma_bytes(int compute_units) { return (size_t)compute_units * (256 * sizeof(float) + 2 * sizeof(uint64_t)); }
 
 int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,

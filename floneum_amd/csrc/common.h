@@ -141,6 +141,8 @@ size_t decode_workspace_bytes(int B, int H, int Hkv, int D, int nsplit);
 size_t calibration_mfma_bytes(int compute_units);
 int launch_calibration_mfma(fhip_dtype dtype, int compute_units, int duty_percent, int rounds, int random_operands, void *scratch,
                             hipStream_t stream);
+// steps of one matrix instruction and the companions `mix` names, one wavefront per SIMD; scratch as for the loop above
+int launch_calibration_issue(int mix, int compute_units, int rounds, void *scratch, hipStream_t stream);
 
 int launch_calibration_read(const void *src, size_t bytes, int compute_units, void *sink, hipStream_t stream);
 

@@ -289,6 +289,23 @@ int fhip_flash_attention_noalloc(fhip_stream *s, const fhip_attn_args *args);
 int fhip_calibration_mfma(fhip_stream *s, fhip_dtype dtype, int32_t random_operands, int32_t duty_percent, int32_t rounds,
                           void *scratch, size_t scratch_bytes);
 
+/* Calibration for benchmarks (no counterpart in the reference): what ONE wavefront per SIMD can issue beside its
+ * matrix instructions.  A wavefront issues in order; a kernel that runs a single wavefront per SIMD (the prefill
+ * kernel of head dims above 192, whose Q and O^T of 32 rows leave no registers for a second one) pays in full for
+ * whatever does not fit into the 32 cycles the matrix pipe is busy with one v_mfma_f32_32x32x16.  One workgroup of
+ * four wavefronts per compute unit runs `rounds` rounds of 16 steps, a step being one such instruction (f16,
+ * independent accumulators) and the companions `mix` names:
+ *   0 nothing; 1 nothing, and every matrix instruction depends on the one before; 2 four v_fma; 3 eight v_fma;
+ *   4 four v_exp; 5 four scalar adds; 6 one ds_read_b128 that is the matrix operand eight steps later;
+ *   7 as 6 and two more ds_read_b128; 8 two ds_read_b64_tr_b16 whose values a vector instruction takes eight steps
+ *   later; 9 as 6 and 8 together; 10 as 9 and fma, exp2, add (the mix of the prefill kernel's softmax steps);
+ *   11 two ds_read_b128 and fma, exp2, add; 12 two ds_read_b128, every other step a transposing read and every fourth
+ *   a 16-byte LDS write (11 and 12: the steps of a kernel whose workgroup transposes a tile once for all its wavefronts).
+ * `scratch` and what it receives are as for fhip_calibration_mfma: per compute unit the shader-clock cycles and the
+ * 100 MHz wall-clock ticks of its workgroup; cycles / (16 * rounds) = cycles per step.  Asynchronous on `s`. */
+#define FHIP_CALIBRATION_ISSUE_MIXES 13
+int fhip_calibration_issue(fhip_stream *s, int32_t mix, int32_t rounds, void *scratch, size_t scratch_bytes);
+
 /* Calibration for benchmarks (no counterpart in the reference): where the workgroups of a launch run.  A
  * one-dimensional launch of `workgroups` workgroups (64 lanes each) stores, per workgroup, the id of the XCD it ran
  * on (the XCC_ID hardware register) into the device bytes `out` (one per workgroup).  The split-KV decode kernels

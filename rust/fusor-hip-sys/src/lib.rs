@@ -68,6 +68,8 @@ pub const FHIP_KERNEL_DECODE_SPLITKV: fhip_kernel_id = 4;
 pub const FHIP_NOALLOC_WORKSPACE_BYTES: usize = 32 << 20;
 /// Most `rounds` `fhip_calibration_mfma` accepts (about a second of matrix work).
 pub const FHIP_CALIBRATION_MFMA_MAX_ROUNDS: i32 = 2000000;
+/// Number of companion mixes `fhip_calibration_issue` knows (0 .. this - 1).
+pub const FHIP_CALIBRATION_ISSUE_MIXES: i32 = 13;
 
 // ---- structs -----------------------------------------------------------------------------------
 /// Rank-4 strided view `[batch, heads, seq, head_dim]`; offset and strides in elements
@@ -232,6 +234,7 @@ unsafe extern "C" {
         scratch_bytes: usize,
     ) -> c_int;
 
+    pub fn fhip_calibration_issue(s: *mut fhip_stream, mix: i32, rounds: i32, scratch: *mut c_void, scratch_bytes: usize) -> c_int;
     pub fn fhip_calibration_xcd_map(s: *mut fhip_stream, workgroups: u32, out: *mut c_void, out_bytes: usize) -> c_int;
     pub fn fhip_calibration_read(
         s: *mut fhip_stream,

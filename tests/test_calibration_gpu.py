@@ -54,3 +54,30 @@ def test_read_calibration_runs_and_rejects_bad_arguments(device):
                                    device.compute_units * 32) == fa.ERR_WORKSPACE
     assert L.fhip_calibration_read(device.stream, ctypes.c_void_p(buf.ptr), n, ctypes.c_void_p(sink.ptr), 16) == fa.ERR_WORKSPACE
     assert L.fhip_calibration_read(device.stream, None, n, ctypes.c_void_p(sink.ptr), 1 << 20) == fa.ERR_INVALID_ARG
+
+
+def test_issue_calibration_runs_every_mix_and_rejects_bad_arguments(device):
+    """fhip_calibration_issue: steps of one matrix instruction and companions, one wavefront per SIMD.  A step cannot
+    take fewer cycles than the matrix pipe is busy with its instruction (32), and companions do not make it shorter."""
+    L = fa.lib()
+    cus = device.compute_units
+    nbytes = cus * (256 * 4 + 16)
+    scratch = fa.Buffer(device, nbytes)
+    p = ctypes.c_void_p(scratch.ptr)
+    host = np.zeros(nbytes, np.uint8)
+    rounds = 300
+    cycles = []
+    for mix in range(13):
+        fa.check(L.fhip_memset(device.stream, p, 0, nbytes))
+        fa.check(L.fhip_calibration_issue(device.stream, mix, rounds, p, nbytes))
+        fa.check(L.fhip_memcpy_d2h(device.stream, host.ctypes.data_as(ctypes.c_void_p), p, nbytes))
+        ticks = host[cus * 1024:].view(np.uint64).reshape(cus, 2).astype(np.float64)
+        assert (ticks > 0).all(), f"mix {mix}: every workgroup reports cycles and wall ticks"
+        assert (ticks[:, 0] >= 0.85 * rounds * 16 * 32).all(), f"mix {mix}: fewer cycles than the matrix instructions take"
+        cycles.append(float(np.median(ticks[:, 0])) / (rounds * 16))
+    assert cycles[3] > cycles[2] - 2 and cycles[10] > cycles[0], cycles
+    assert L.fhip_calibration_issue(device.stream, 13, 10, p, nbytes) == fa.ERR_INVALID_ARG
+    assert L.fhip_calibration_issue(device.stream, -1, 10, p, nbytes) == fa.ERR_INVALID_ARG
+    assert L.fhip_calibration_issue(device.stream, 0, 0, p, nbytes) == fa.ERR_INVALID_ARG
+    assert L.fhip_calibration_issue(device.stream, 0, 10, p, nbytes - 16) == fa.ERR_WORKSPACE
+    assert L.fhip_calibration_issue(device.stream, 0, 10, None, nbytes) == fa.ERR_INVALID_ARG
