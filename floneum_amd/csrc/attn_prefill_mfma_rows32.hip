@@ -1,5 +1,5 @@
-// Prefill attention for f16 / bf16 at head dims above 192 (Gemma-3's key length is 256) on the gfx950 matrix cores,
-// for prompts long enough to give every CU a workgroup of 128 query rows.
+// Prefill attention for f16 / bf16 at head dims above 192 (Gemma-3's key length is 256) on the gfx950 matrix cores:
+// every call at these head dims whose keys are not split over workgroups and whose heads are not packed.
 //
 // At this head dim Q and O^T of 32 query rows are 192 registers of a wavefront, so two wavefronts per SIMD can only
 // hold 16 rows each (prefill_mfma_wide_kernel), and every K and V operand a wavefront reads from LDS then feeds a

@@ -429,6 +429,11 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // CUs and even out the long and short row blocks of a causal mask, each reading K and V from LDS for half as
     // many matrix instructions (f16, head_dim 256, 16 heads: 512 tokens 48 -> 33 us, 1024: 72 -> 52, 2048: 125 -> 108,
     // 3072: 179 -> 170).
+    // Above head_dim 192 every call whose keys are not split and whose heads are not packed runs on the kernel of four
+    // 32-row wavefronts (attn_prefill_mfma_rows32.hip), whatever the grid: f16, head_dim 256, causal, 8 heads: 512 tokens
+    // 27.9 -> 24.5 us, 1024: 44.0 -> 36.1, 2048: 77.8 -> 60.3, 4096: 172 -> 116; 16 heads, 4096: 207 -> 152.
+    if (prefill_mfma_rows32_takes(p))
+        return launch_prefill_mfma_rows32(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     const long wgs128 = (long)p.B * p.H * ((p.Sq + PW_BM - 1) / PW_BM);
     // (With the keys split, up to 64 rows are one row block either way: the 64-row form computes half as much per tile
     // and runs two workgroups per CU: f16, head_dim 256, B8 x 16 heads, 64 rows on 8192 keys 271 -> 181 us.)
@@ -437,8 +442,6 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // Up to head_dim 192 a wavefront can hold 32 rows (two column blocks: every K and V operand read from LDS then feeds
     // two matrix instructions): 256-row workgroups where those still give every CU one (f16, 4096 x 4096 causal:
     // head_dim 160 497 -> 559 TFLOP/s, 192 450 -> 511; at 224 and 256 the registers do not suffice)
-    if (bm == PW_BM && prefill_mfma_rows32_takes(p))
-        return launch_prefill_mfma_rows32(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     const long wgs256 = (long)p.B * p.H * ((p.Sq + 255) / 256);
     const bool big = wgs256 >= p.cus;
     if (!p.pf_pack && !small && p.pf_nsplit <= 1 && p.D <= 192 && big) bm = 256;

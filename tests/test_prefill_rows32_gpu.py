@@ -1,9 +1,9 @@
-"""GPU parity tests of the prefill kernel that head dims above 192 take on a grid that fills the chip: 128-row
-workgroups of four wavefronts with 32 rows each, one per SIMD, software-pipelined over 32-key tiles
-(floneum_amd/csrc/attn_prefill_mfma_rows32.hip).
+"""GPU parity tests of the prefill kernel of head dims above 192: 128-row workgroups of four wavefronts with 32 rows
+each, one per SIMD, software-pipelined over 32-key tiles (floneum_amd/csrc/attn_prefill_mfma_rows32.hip).
 
-The library chooses it when 128-row blocks give every CU two workgroups, the keys are not split over workgroups and the
-heads are not packed; every case here has 512 such blocks on a 256-CU chip (the test asserts it).  Reference semantics:
+The library chooses it whenever the keys are not split over workgroups and the heads are not packed.  Every case here
+has at least 512 workgroups on a 256-CU chip (the tests assert it): two rounds, every LDS stage and register reused by a
+second workgroup; the small-grid cases of tests/test_attention_gpu.py at these head dims run on it too.  Reference semantics:
 fusor-ml/fusor/src/composite/flash_attention.rs:141-199; the cases follow the prefill cases of
 tests/test_attention_gpu.py at the shapes this kernel is chosen for.
 """
