@@ -1,5 +1,6 @@
 // Prefill attention for f16 / bf16 at head dims above 192 (Gemma-3's key length is 256) on the gfx950 matrix cores:
-// every call at these head dims whose keys are not split over workgroups and whose heads are not packed.
+// every call at these head dims but those of up to 64 query rows whose keys are split over workgroups or whose heads
+// are packed (a few new rows on a long cache, attn_prefill_mfma_wide.hip).
 //
 // At this head dim Q and O^T of 32 query rows are 192 registers of a wavefront, so two wavefronts per SIMD can only
 // hold 16 rows each (prefill_mfma_wide_kernel), and every K and V operand a wavefront reads from LDS then feeds a
@@ -118,7 +119,9 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     // workgroup -> (query block, batch, head): long (late) query blocks first; consecutive workgroups land on
     // consecutive XCDs, so with H a multiple of 8 the heads are dealt so that an XCD works on neighbouring heads
     const int bh_count = p.B * p.H;
-    const int id = blockIdx.x;
+    const int nks = max(p.pf_nsplit, 1);
+    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
+    const int id = blockIdx.x / nks;
     const int qb = nqb - 1 - id / bh_count;
     const int rem = id % bh_count;
     const int b = rem / p.H;
@@ -131,7 +134,13 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
 
     const int q0 = qb * R32_BM, qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
-    const RowBounds rb = row_bounds(p, b, q0, R32_BM, qw0, lane);
+    RowBounds rb = row_bounds(p, b, q0, R32_BM, qw0, lane);
+    if (nks > 1) {  // a few query blocks on a long cache: this workgroup takes one share of the keys
+        const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
+        rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
+        rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
+        rb.klo = max(rb.klo, c_lo), rb.khi = min(rb.khi, c_hi);
+    }
     const int klo = rb.klo, khi = rb.khi;
     const int lo_wg = __builtin_amdgcn_readfirstlane(rb.lo_wg), hi_wg = __builtin_amdgcn_readfirstlane(rb.hi_wg);
     const int full_lo_w = __builtin_amdgcn_readfirstlane(rb.full_lo_w), full_hi_w = __builtin_amdgcn_readfirstlane(rb.full_hi_w);
@@ -428,6 +437,24 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     lds_barrier();
     // ---- epilogue: out[query][dim] = O^T[dim][query] / l (no visible key: NaN like the reference's 0 / 0) -----------
     const float l_tot = r32_half_swap_sum(l);
+    if (nks > 1) {
+        // this share's state: O unnormalised as f32, then (m in base-2 exponent units, l); the merge kernel normalises
+        if (query < p.Sq) {
+            float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * p.pf_pitch;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int dim = 32 * db + 8 * rq + 4 * h2;
+                    if (dim < hd) *(float4_t *)(ws + dim) = float4_t{o[db][4 * rq], o[db][4 * rq + 1], o[db][4 * rq + 2], o[db][4 * rq + 3]};
+                }
+            if (h2 == 0) {
+                ws[hd] = m * rr;
+                ws[hd + 1] = l_tot;
+            }
+        }
+        return;
+    }
     const float inv = 1.0f / l_tot;
     const bool dead = l_tot == 0.0f;
     if (out_vec) {
@@ -492,7 +519,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
 template <typename T>
 int launch_rows32_t(const AttnParams &p, hipStream_t stream) {
     const int nqb = (p.Sq + R32_BM - 1) / R32_BM;
-    const long blocks = (long)nqb * p.B * p.H;
+    const long blocks = (long)nqb * p.B * p.H * (p.pf_nsplit > 1 ? p.pf_nsplit : 1);
     if (blocks > 0x7fffffffL) {
         set_error("prefill: too many workgroups (%ld)", blocks);
         return FHIP_ERR_UNSUPPORTED;
@@ -504,6 +531,7 @@ int launch_rows32_t(const AttnParams &p, hipStream_t stream) {
         if ((p.os[i] * oeb) % 16 != 0) out_vec = 0;
     FHIP_LAUNCH_MAIN((prefill_mfma_wide_rows32_kernel<T>), dim3((unsigned)blocks), dim3(256), stream, p, p, nqb, out_vec);
     FHIP_HIP_CHECK(hipGetLastError());
+    if (p.pf_nsplit > 1) return launch_prefill_merge(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     return FHIP_OK;
 }
 
@@ -511,11 +539,14 @@ int launch_rows32_t(const AttnParams &p, hipStream_t stream) {
 
 // The calls this form takes: head dims above 192 (padded with zeros up to 256: f16, 4096 x 4096 causal, 16 heads, head_dim
 // 200 / 224 / 232 195 / 208 / 218 -> 155 / 160 / 161 us against the 16-row form; up to 192 a wavefront of that form holds
-// 32 rows itself), keys not split over workgroups, no packed heads, and a scale whose power-of-two part Q can carry
-// without leaving the 16-bit type's normal range.
+// 32 rows itself), no packed heads, keys split over workgroups only from 65 query rows on (f16, head_dim 256, 16 / 4
+// heads, 128 rows on B8 x 8192 keys 263 -> 186 us, on B1 x 32768 keys 120 -> 102), and a scale whose power-of-two part Q
+// can carry without leaving the 16-bit type's normal range.
 bool prefill_mfma_rows32_takes(const AttnParams &p) {
     const float scale2 = p.scale * R32_LOG2E;
-    return p.D > 192 && p.D <= R32_D && p.D % 8 == 0 && p.pf_nsplit <= 1 && !p.pf_pack && scale2 >= 0.00390625f && scale2 < 2.0f;
+    // (keys split over workgroups: from 65 query rows on; up to 64 the 16-row kernel's 64-row and packed forms serve)
+    return p.D > 192 && p.D <= R32_D && p.D % 8 == 0 && (p.pf_nsplit <= 1 || p.Sq > 64) && !p.pf_pack && scale2 >= 0.00390625f &&
+           scale2 < 2.0f;
 }
 
 int launch_prefill_mfma_rows32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {

@@ -429,7 +429,7 @@ int launch_wide_t(const AttnParams &p_in, hipStream_t stream) {
     // CUs and even out the long and short row blocks of a causal mask, each reading K and V from LDS for half as
     // many matrix instructions (f16, head_dim 256, 16 heads: 512 tokens 48 -> 33 us, 1024: 72 -> 52, 2048: 125 -> 108,
     // 3072: 179 -> 170).
-    // Above head_dim 192 every call whose keys are not split and whose heads are not packed runs on the kernel of four
+    // Above head_dim 192 every call but the split and packed ones of up to 64 query rows runs on the kernel of four
     // 32-row wavefronts (attn_prefill_mfma_rows32.hip), whatever the grid: f16, head_dim 256, causal, 8 heads: 512 tokens
     // 27.9 -> 24.5 us, 1024: 44.0 -> 36.1, 2048: 77.8 -> 60.3, 4096: 172 -> 116; 16 heads, 4096: 207 -> 152.
     if (prefill_mfma_rows32_takes(p))

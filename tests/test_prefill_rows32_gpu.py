@@ -7,6 +7,8 @@ second workgroup; the small-grid cases of tests/test_attention_gpu.py at these h
 fusor-ml/fusor/src/composite/flash_attention.rs:141-199; the cases follow the prefill cases of
 tests/test_attention_gpu.py at the shapes this kernel is chosen for.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -208,3 +210,22 @@ def test_rows_without_a_visible_key_and_queries_beyond_the_last_block(device):
                                      rounded(v[b:b + 1, :, :n], fa.F16), D ** -0.5, mask[:, :n], "qk")
         # rows behind the sequence's keys see all of them (causality hides nothing more): still finite
         assert_parity(out[b:b + 1], ref, TOL_16, f"sequence {b} of {n} keys")
+
+
+@pytest.mark.parametrize("dtype,D", [(fa.F16, 256), (fa.BF16, 256), (fa.F16, 232)])
+@pytest.mark.parametrize("Sq,Skv,window", [(128, 8192, 0), (100, 5000, 0), (160, 6000, 1500), (65, 4096, 0)])
+def test_keys_split_over_workgroups(device, dtype, D, Sq, Skv, window):
+    """A new chat turn: 65 and more query rows on a long cache leave most CUs without a 128-row block, so the keys are
+    split over workgroups too (the planner's shares of 1024 keys and more); every workgroup parks (O, m, l) of its share
+    and a merge kernel folds them.  (Up to 64 rows the 16-row kernel's 64-row and packed forms serve.)"""
+    B, H, Hkv = 1, 8, 4
+    q, k, v = qkv(41 + Sq, B, H, Hkv, Sq, Skv, D)
+    tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+    desc = (True, Skv - Sq, window)
+    need = ctypes.c_size_t()
+    args = tq._attn_args(tk, tv, D ** -0.5, None, desc, None, None, fa.KERNEL_AUTO, None)
+    fa.check(fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(args), device.compute_units, ctypes.byref(need)))
+    assert need.value > 0, "the call is planned with split keys"
+    out = tq.flash_attention(tk, tv, D ** -0.5, analytic=desc).to_numpy()
+    ref = reference(q, k, v, D, dtype, analytic_mask(Sq, Skv, *desc))
+    assert_parity(out, ref, TOL_BF16 if dtype == fa.BF16 else TOL_16, f"D{D} {Sq} rows on {Skv} keys, window {window}")
