@@ -101,7 +101,9 @@ __device__ __forceinline__ float r32_half_swap_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <typename T>
+// SPLIT: the keys are split over workgroups (an instantiation of its own: the kernel sits at the edge of the register
+// file, and the code of the split form costs the unsplit one spills inside its loop).
+template <typename T, bool SPLIT>
 __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnParams p, int nqb, int out_vec) {
     typedef typename R32Mma<T>::vec8 vec8;
     constexpr int D = R32_D, ROWB = R32_ROWB, KG = R32_KG, VG = R32_VG;
@@ -119,9 +121,9 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     // workgroup -> (query block, batch, head): long (late) query blocks first; consecutive workgroups land on
     // consecutive XCDs, so with H a multiple of 8 the heads are dealt so that an XCD works on neighbouring heads
     const int bh_count = p.B * p.H;
-    const int nks = max(p.pf_nsplit, 1);
-    const int ksplit = blockIdx.x % nks;  // which share of the keys (0 when the keys are not split over workgroups)
-    const int id = blockIdx.x / nks;
+    const int nks = SPLIT ? max(p.pf_nsplit, 1) : 1;
+    const int ksplit = SPLIT ? blockIdx.x % nks : 0;  // which share of the keys
+    const int id = SPLIT ? blockIdx.x / nks : blockIdx.x;
     const int qb = nqb - 1 - id / bh_count;
     const int rem = id % bh_count;
     const int b = rem / p.H;
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     const int q0 = qb * R32_BM, qw0 = q0 + 32 * wave;
     const int query = qw0 + ln;
     RowBounds rb = row_bounds(p, b, q0, R32_BM, qw0, lane);
-    if (nks > 1) {  // a few query blocks on a long cache: this workgroup takes one share of the keys
+    if (SPLIT) {  // a few query blocks on a long cache: this workgroup takes one share of the keys
         const int c_lo = ksplit * p.pf_chunk, c_hi = c_lo + p.pf_chunk;
         rb.lo_wg = max(rb.lo_wg, c_lo), rb.hi_wg = min(rb.hi_wg, c_hi);
         rb.full_lo_w = max(rb.full_lo_w, c_lo), rb.full_hi_w = min(rb.full_hi_w, c_hi);
@@ -437,7 +439,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     lds_barrier();
     // ---- epilogue: out[query][dim] = O^T[dim][query] / l (no visible key: NaN like the reference's 0 / 0) -----------
     const float l_tot = r32_half_swap_sum(l);
-    if (nks > 1) {
+    if (SPLIT) {
         // this share's state: O unnormalised as f32, then (m in base-2 exponent units, l); the merge kernel normalises
         if (query < p.Sq) {
             float *ws = p.partials + ((((int64_t)b * p.H + h) * p.Sq + query) * nks + ksplit) * p.pf_pitch;
@@ -529,7 +531,8 @@ int launch_rows32_t(const AttnParams &p, hipStream_t stream) {
     int out_vec = p.os[3] == 1 && ((uintptr_t)p.out % 16 == 0);
     for (int i = 0; i < 3; i++)
         if ((p.os[i] * oeb) % 16 != 0) out_vec = 0;
-    FHIP_LAUNCH_MAIN((prefill_mfma_wide_rows32_kernel<T>), dim3((unsigned)blocks), dim3(256), stream, p, p, nqb, out_vec);
+    if (p.pf_nsplit > 1) FHIP_LAUNCH_MAIN((prefill_mfma_wide_rows32_kernel<T, true>), dim3((unsigned)blocks), dim3(256), stream, p, p, nqb, out_vec);
+    else FHIP_LAUNCH_MAIN((prefill_mfma_wide_rows32_kernel<T, false>), dim3((unsigned)blocks), dim3(256), stream, p, p, nqb, out_vec);
     FHIP_HIP_CHECK(hipGetLastError());
     if (p.pf_nsplit > 1) return launch_prefill_merge(p, std::is_same<T, half_t>::value ? FHIP_F16 : FHIP_BF16, stream);
     return FHIP_OK;
