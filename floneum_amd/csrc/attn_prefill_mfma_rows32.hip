@@ -9,11 +9,11 @@
 // v_mfma_f32_32x32x16 with the arithmetic of the 256-row kernel (attn_prefill_mfma.hip): half the LDS bytes per matrix
 // instruction.  With one wavefront per SIMD nothing overlaps unless the instruction stream itself interleaves it, so
 // the loop is software-pipelined over the 32-key tiles.  Iteration t:
-//   block B:  O^T += V(t-1)^T . P(t-1)^T on the matrix pipe; beside it the LDS hands over the rest of V(t-1)'s operands
-//             and the first of K(t+1)'s, the scores S^T(t) move to where the vector ALU reads them, and the tile loads
-//             of the iteration are issued
+//   block B:  O^T += V(t-1)^T . P(t-1)^T on the matrix pipe; beside it the LDS hands over the rest of V(t-1)'s operands,
+//             the first of K(t+1)'s and the first of V(t)'s, the scores S^T(t) move to where the vector ALU reads them,
+//             and the tile loads of the iteration are issued
 //   block A:  S^T(t+1) = K(t+1) . Q^T on the matrix pipe; beside it the vector ALU turns S^T(t) into probabilities and
-//             the LDS hands over the rest of K(t+1)'s operands and the first of V(t)'s
+//             the LDS hands over the rest of K(t+1)'s operands
 // Each block is sixteen steps of one matrix instruction and what runs beside it, fenced so that the compiler keeps
 // them apart (a lone wavefront issues in order: a matrix instruction leaves room for about four other instructions
 // before the next one is due, and whatever is not placed beside one is paid for in full).  K and V tiles live in rings
@@ -304,14 +304,16 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
     // Both blocks are written as sixteen steps that nothing crosses: a matrix instruction first, then the LDS reads,
     // tile loads and vector work that run beside it (left to itself the scheduler issues the matrix instructions back
     // to back and the rest behind them, where nothing hides it).
-    // Block B of tile u: O^T += V(u)^T . P(u)^T.  Beside it: the second contraction slice of V(u) and the first operands
-    // of K(u + 2) leave the LDS; the scores of tile u + 1 leave the accumulation half of the register file, one per
-    // step; this iteration's tile loads are issued, one every other step: K(u + 4) into the stage K(u) left one
-    // iteration ago, V(u + 3) into the stage V(u - 1) left then.
+    // Block B of tile u: O^T += V(u)^T . P(u)^T.  Beside it: the second contraction slice of V(u) leaves the LDS in the
+    // first eight steps, the first operands of K(u + 2) and the first slice of V(u + 1) (for the next iteration's block
+    // B: in block A, beside the exponentials, the transposing reads cost more) in the last eight; the scores of tile
+    // u + 1 leave the accumulation half of the register file, one per step; this iteration's tile loads are issued, one
+    // every other step: K(u + 4) into the stage K(u) left one iteration ago, V(u + 3) into the stage V(u - 1) left then.
     auto block_b = [&](int u) __attribute__((always_inline)) {
         __builtin_amdgcn_sched_barrier(0);
         const int vbase = v_addr(u);
         const int kbase = k_addr(u + 2);
+        const int vnext = v_addr(u + 1);
         const int soff_k = __builtin_amdgcn_readfirstlane(min(j_begin + (u + 4) * R32_KEYS, p.Skv) * krow_bytes);
         const int soff_v = __builtin_amdgcn_readfirstlane(min(j_begin + (u + 3) * R32_KEYS, p.Skv) * vrow_bytes);
         const int lds_k = __builtin_amdgcn_readfirstlane(lds0 + k_stage(u + 4) + wave * KG);
@@ -327,6 +329,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
                 o[db] = R32Mma<T>::mfma(kk == 0 ? __builtin_bit_cast(vec8, va[0][db]) : acc_half(va[1][db]), bop, o[db]);
                 if (kk == 0) read_v(vbase, 1, db);
                 else read_k(kbase, db);
+                if (kk == 1) read_v(vnext, 0, db);
                 if ((db & 1) == 0) {
                     if (kk == 0) issue_piece_k(db >> 1, lds_k, soff_k);
                     else issue_piece_v(db >> 1, lds_v, soff_v);
@@ -342,10 +345,9 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
         }
     };
     // Block A of tile t: S^T(t + 1) on the matrix pipe (first operands in ka); beside it the probabilities of tile t
-    // (scores in sx), the rest of K(t + 1)'s operands and the first contraction slice of V(t).  Returns the lane's sum.
+    // (scores in sx) and the rest of K(t + 1)'s operands.  Returns the lane's sum.
     auto block_a = [&](int t) __attribute__((always_inline)) {
         __builtin_amdgcn_sched_barrier(0);
-        const int vbase = v_addr(t);
         const int kbase = k_addr(t + 1);
         float ts = 0.0f;
         float pe[16];
@@ -353,7 +355,6 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_wide_rows32_kernel(AttnPa
         for (int kb = 0; kb < D / 16; kb++) {
             sn = R32Mma<T>::mfma(acc_half(ka[kb % PFK]), qreg[kb], kb == 0 ? zero16 : sn);
             if (kb + PFK < D / 16) read_k(kbase, kb + PFK);
-            if (kb < D / 32) read_v(vbase, 0, kb);
             pe[kb] = __builtin_amdgcn_exp2f(__builtin_fmaf(sx[kb], rr, nmr));
             if (kb & 1) {
                 // (formed here, in its step, not behind the branch that follows the block)
