@@ -75,6 +75,12 @@ def configs():
         # whole 16896-key cache is passed and the analytic window leaves every query exactly 4096 keys
         "C4B": dict(kind="prefill", B=4, H=32, Hkv=8, Sq=512, Skv=16896, D=128, dtype="f16", std=1.0, causal=True,
                     q_pos_offset=16384, window=4096),
+        # C3 and C4 on the form of the tiled kernel the library never chooses (force_kernel 5: four wavefronts of 64 query
+        # rows per workgroup, one per SIMD; half the LDS operand reads per matrix instruction, everything issued in order)
+        "C3R": dict(kind="prefill", B=1, H=32, Hkv=8, Sq=8192, Skv=8192, D=128, dtype="f16", std=1.0, causal=True,
+                    force_kernel=5),
+        "C4R": dict(kind="prefill", B=4, H=32, Hkv=8, Sq=512, Skv=4096, D=128, dtype="f16", std=1.0, causal=True,
+                    q_pos_offset=3584, window=4096, force_kernel=5),
         "C5": dict(kind="decode", B=32, H=32, Hkv=32, Sq=1, Skv=32768, D=96, dtype="f16", std=1.0, causal=False,
                    ragged=(128, 32768)),
         # not a headline configuration: a new chat turn, 128 query rows on 8192 cached keys (the shape at which the
@@ -211,7 +217,7 @@ def prepare(fa, dev, c, sets, lens_t):
         analytic = None
         if c["causal"] and mask is None:
             analytic = (True, c.get("q_pos_offset", c["Skv"] - c["Sq"]), c.get("window", 0))
-        args = q._attn_args(k, v, c["D"] ** -0.5, mask, analytic, lens_t, None, fa.KERNEL_AUTO, None)
+        args = q._attn_args(k, v, c["D"] ** -0.5, mask, analytic, lens_t, None, c.get("force_kernel", fa.KERNEL_AUTO), None)
         need = ctypes.c_size_t()
         fa.check(L.fhip_flash_attention_workspace_bytes(ctypes.byref(args), dev.compute_units, ctypes.byref(need)))
         if need.value:
@@ -759,6 +765,7 @@ def record_traffic(name, fetch_csv, write_csv):
         per_count = copied / max(copy)
         main = {k: v for k, v in counts.items() if any(t in k for t in ("decode_mfma", "decode_vec", "prefill_mfma_kernel",
                                                                        "prefill_mfma_wide_kernel", "prefill_mfma_wide_rows32_kernel",
+                                                                       "prefill_mfma_rows64_kernel",
                                                                        "prefill_f32_kernel",
                                                                        "prefill_f32_wide", "attn_generic"))}
         assert len(main) == 1, f"{path}: expected one main kernel, found {sorted(main)}"
@@ -771,6 +778,7 @@ def record_traffic(name, fetch_csv, write_csv):
     out["kernel"] = kernel
     # the file the kernel lives in (the wide-head 16-bit prefill kernels have files of their own)
     out["source"] = "attn_prefill_mfma_rows32.hip" if "prefill_mfma_wide_rows32" in out["kernel_symbol"] else \
+        "attn_prefill_mfma_rows64.hip" if "prefill_mfma_rows64" in out["kernel_symbol"] else \
         "attn_prefill_mfma_wide.hip" if "prefill_mfma_wide" in out["kernel_symbol"] else KERNEL_SOURCES[kernel]
     out["source_sha256"] = source_hash(kernel, out["source"])
     try:

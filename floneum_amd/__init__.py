@@ -29,7 +29,8 @@ F32, F16, BF16 = 0, 1, 2
 _DTYPE_BYTES = {F32: 4, F16: 2, BF16: 2}
 
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_PREFILL_MFMA, KERNEL_PREFILL_F32, KERNEL_DECODE_SPLITKV = 0, 1, 2, 3, 4
-KERNEL_NAMES = {1: "generic", 2: "prefill_mfma", 3: "prefill_f32", 4: "decode_splitkv"}
+KERNEL_PREFILL_MFMA_ROWS64 = 5  # only as force_kernel: the tiled 16-bit kernel's 64-rows-per-wavefront form at head_dim 128
+KERNEL_NAMES = {1: "generic", 2: "prefill_mfma", 3: "prefill_f32", 4: "decode_splitkv", 5: "prefill_mfma_rows64"}
 
 OK, ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = 0, 1, 2, 3, 4
 NOALLOC_WORKSPACE_BYTES = 32 << 20  # FHIP_NOALLOC_WORKSPACE_BYTES

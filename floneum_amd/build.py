@@ -6,7 +6,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["api.hip", "attn_generic.hip", "attn_decode.hip", "attn_prefill_mfma.hip", "attn_prefill_mfma_wide.hip", "attn_prefill_mfma_rows32.hip",
+SOURCES = ["api.hip", "attn_generic.hip", "attn_decode.hip", "attn_prefill_mfma.hip", "attn_prefill_mfma_wide.hip", "attn_prefill_mfma_rows32.hip", "attn_prefill_mfma_rows64.hip",
            "attn_prefill_f32.hip",
            "kv_cache.hip", "mask_intervals.hip", "rope.hip", "calibration.hip"]
 LIB = os.path.join(HERE, "libfusor_hip.so")

@@ -328,6 +328,11 @@ static void f32_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *c
 }
 static size_t f32_partials_offset(const fhip_attn_args *a) { return (mask_scratch_bytes(a) + 255) & ~(size_t)255; }
 static void mfma_split_plan(const fhip_attn_args *a, int cus, int *nsplit, int *chunk) {
+    if (a->force_kernel == FHIP_KERNEL_PREFILL_MFMA_ROWS64) {  // that form never splits the keys
+        *nsplit = 1;
+        *chunk = (int)a->k.shape[2];
+        return;
+    }
     const bool causal_square = a->analytic.enabled && a->analytic.causal && 2ull * a->q.shape[2] > a->k.shape[2];
     const int Hkv = (int)a->k.shape[1];
     if (!(a->q.shape[3] == 64 || a->q.shape[3] == 96 || a->q.shape[3] == 128))  // the wide-head form: 128-row query blocks
@@ -364,6 +369,9 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
         switch (f) {
             case FHIP_KERNEL_GENERIC: ok = true; break;
             case FHIP_KERNEL_PREFILL_MFMA: ok = prefill_mfma_eligible(a) && mask_ok; break;
+            case FHIP_KERNEL_PREFILL_MFMA_ROWS64:
+                ok = prefill_mfma_eligible(a) && mask_ok && prefill_mfma_rows64_takes((int)a->q.shape[3], a->scale);
+                break;
             case FHIP_KERNEL_PREFILL_F32: ok = prefill_f32_eligible(a) && (mask_ok || f32_adds_masks(a)); break;
             case FHIP_KERNEL_DECODE_SPLITKV: ok = decode_eligible(a); break;
             default: set_error("unknown force_kernel %d", f); return FHIP_ERR_INVALID_ARG;
@@ -373,7 +381,8 @@ static int select_kernel(const fhip_attn_args *a, int32_t *id, bool assume_works
                       "the workspace its interval form needs)", f);
             return FHIP_ERR_UNSUPPORTED;
         }
-        *id = f;
+        // (the forced form of the tiled 16-bit kernel is that kernel to everything that follows; AttnParams carries the form)
+        *id = f == FHIP_KERNEL_PREFILL_MFMA_ROWS64 ? (int)FHIP_KERNEL_PREFILL_MFMA : f;
         return FHIP_OK;
     }
     if (decode_eligible(a))
@@ -753,7 +762,10 @@ int fhip_flash_attention_select(const fhip_attn_args *args, int32_t *kernel_id) 
     }
     int rc = validate(args);
     if (rc) return rc;
-    return select_kernel(args, kernel_id);
+    rc = select_kernel(args, kernel_id);
+    if (rc == FHIP_OK && args->force_kernel == FHIP_KERNEL_PREFILL_MFMA_ROWS64 && *kernel_id == FHIP_KERNEL_PREFILL_MFMA)
+        *kernel_id = FHIP_KERNEL_PREFILL_MFMA_ROWS64;
+    return rc;
 }
 
 int fhip_flash_attention_workspace_bytes(const fhip_attn_args *args, int32_t compute_units, size_t *bytes) {
@@ -823,6 +835,10 @@ static void plan_decode_call(fhip_device *dev, const fhip_attn_args *args, AttnP
 
 // the 16-bit tiled prefill kernels: 64 / 96 / 128, and the wide-head form above
 static int launch_mfma_by_head_dim(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
+    // the form of four wavefronts with 64 rows each (attn_prefill_mfma_rows64.hip), when the caller forces it: measured
+    // 3-6 % slower than the 256-row form of eight wavefronts on the benchmark prompts (fewer LDS reads and a higher clock,
+    // but a lone wavefront per SIMD issues everything in order), so it is never chosen
+    if (p.pf_rows64) return launch_prefill_mfma_rows64(p, dtype, stream);
     return (p.D == 64 || p.D == 96 || p.D == 128) ? launch_prefill_mfma(p, dtype, stream) : launch_prefill_mfma_wide(p, dtype, stream);
 }
 
@@ -901,6 +917,7 @@ int fhip_flash_attention(fhip_stream *s, const fhip_attn_args *args) {
         }
     }
     if (id == FHIP_KERNEL_PREFILL_MFMA) {
+        p.pf_rows64 = args->force_kernel == FHIP_KERNEL_PREFILL_MFMA_ROWS64;
         int ns, chunk;
         mfma_split_plan(args, s->dev->prop.multiProcessorCount, &ns, &chunk);
         const size_t off = f32_partials_offset(args);

@@ -65,6 +65,7 @@ struct AttnParams {
     int32_t pf_nsplit, pf_chunk;
     int32_t pf_pitch;  // floats per (row, share) in `partials`: D + 2, or D + 4 where rows are written in 16-byte pieces
     int32_t pf_pack;   // tiled kernels, set by their launchers: query heads per workgroup of the packed form, or 0
+    int32_t pf_rows64; // 16-bit tiled prefill at head_dim 128: the caller forced the 64-rows-per-wavefront form
 };
 
 // the key split of a tiled f32 prefill call (1 = none) and the scratch it needs
@@ -128,6 +129,9 @@ void prefill_mfma_wide_plan(int B, int H, int G, int Sq, int Skv, bool causal_sq
 // head dims above 192 on 128-row workgroups of four wavefronts with 32 rows each (one per SIMD, software-pipelined)
 bool prefill_mfma_rows32_takes(const AttnParams &p);
 int launch_prefill_mfma_rows32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
+// head_dim 128 on 256-row workgroups of four wavefronts with 64 rows each (FHIP_KERNEL_PREFILL_MFMA_ROWS64: forced only)
+bool prefill_mfma_rows64_takes(int D, float scale);
+int launch_prefill_mfma_rows64(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 // f32 arithmetic on the f32 matrix cores; `dtype` is the tensors' storage type (16-bit rows are widened on load)
 int launch_prefill_f32(const AttnParams &p, fhip_dtype dtype, hipStream_t stream);
 

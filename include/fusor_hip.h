@@ -151,13 +151,19 @@ typedef enum {
     FHIP_KERNEL_PREFILL_F32 = 3, /* f32 arithmetic on the f32 MFMA, LDS-tiled: f32 tensors, and 16-bit tensors
                                     (widened on load) the kernel above does not take; head_dim multiple of
                                     4 up to 256; masks by interval or, up to head_dim 128, added as they are */
-    FHIP_KERNEL_DECODE_SPLITKV = 4 /* 1..4 query rows per sequence, head_dim multiple of 8 up to 256: split-KV
+    FHIP_KERNEL_DECODE_SPLITKV = 4,/* 1..4 query rows per sequence, head_dim multiple of 8 up to 256: split-KV
                                       streaming + LSE combine.  Matrix cores at every head_dim that is a multiple
                                       of 32 up to 256 (the 16-bit or the f32 instruction, by the tensors' type;
                                       f32 at 224 / 256 from five columns per KV head on), vector units otherwise.  At the matrix-core head dims
                                       more rows ride along while rows x GQA group <= 32 (16 above head_dim 128;
                                       f32 tensors: 64 up to head_dim 192, 32 above): an 8-token draft on a 4-way
                                       GQA model                                                               */
+    FHIP_KERNEL_PREFILL_MFMA_ROWS64 = 5 /* only as force_kernel, never chosen: FHIP_KERNEL_PREFILL_MFMA's calls at
+                                      head_dim 128 on its other form, four wavefronts of 64 query rows per workgroup
+                                      (one per SIMD, half the LDS operand reads per matrix instruction, keys never split
+                                      over workgroups).  Same results; 3-6 % slower than the 256-row form of eight
+                                      wavefronts on this chip, whose matrix kernels are bound by power.  Kept selectable
+                                      for measurement (bench.py --config C3R)                                  */
 } fhip_kernel_id;
 
 

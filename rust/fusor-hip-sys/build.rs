@@ -17,6 +17,7 @@ const SOURCES: &[&str] = &[
     "attn_prefill_mfma.hip",
     "attn_prefill_mfma_wide.hip",
     "attn_prefill_mfma_rows32.hip",
+    "attn_prefill_mfma_rows64.hip",
     "attn_prefill_f32.hip",
     "kv_cache.hip",
     "mask_intervals.hip",

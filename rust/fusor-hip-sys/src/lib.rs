@@ -63,6 +63,7 @@ pub const FHIP_KERNEL_GENERIC: fhip_kernel_id = 1;
 pub const FHIP_KERNEL_PREFILL_MFMA: fhip_kernel_id = 2;
 pub const FHIP_KERNEL_PREFILL_F32: fhip_kernel_id = 3;
 pub const FHIP_KERNEL_DECODE_SPLITKV: fhip_kernel_id = 4;
+pub const FHIP_KERNEL_PREFILL_MFMA_ROWS64: fhip_kernel_id = 5;
 
 /// Size of the per-GPU array `fhip_flash_attention_noalloc` uses as its workspace.
 pub const FHIP_NOALLOC_WORKSPACE_BYTES: usize = 32 << 20;
