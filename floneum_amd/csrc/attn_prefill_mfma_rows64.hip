@@ -6,16 +6,20 @@
 // blocks, Q (64 registers) and O^T (128) of both in registers, and every operand it reads feeds TWO matrix
 // instructions: half the LDS instructions and bytes per matrix instruction.  With one wavefront per SIMD nothing
 // overlaps unless the instruction stream itself interleaves it, so the loop is software-pipelined over 32-key
-// sub-tiles exactly as in attn_prefill_mfma_rows32.hip.  Iteration t:
+// sub-tiles as in attn_prefill_mfma_rows32.hip.  For sub-tile t:
 //   block B:  O^T += V(t-1)^T . P(t-1)^T on the matrix pipe; beside it the LDS hands over the rest of V(t-1)'s operands,
-//             the first of K(t+1)'s and the first of V(t)'s, the scores S^T(t) move to where the vector ALU reads them,
-//             and the tile loads of the iteration are issued
-//   block A:  S^T(t+1) = K(t+1) . Q^T on the matrix pipe; beside it the vector ALU turns S^T(t) into probabilities and
-//             the LDS hands over the rest of K(t+1)'s operands
+//             the first of K(t+1)'s and the first of V(t)'s, the vector ALU turns the first row block's scores S^T(t)
+//             into probabilities, and tile loads are issued
+//   block A:  S^T(t+1) = K(t+1) . Q^T on the matrix pipe; beside it the vector ALU turns the second row block's scores
+//             S^T(t) into probabilities and the LDS hands over the rest of K(t+1)'s operands
+// The scores accumulate in vector registers, where the softmax reads them, and scores and probabilities are kept twice,
+// by the sub-tile's parity (the matrix pipe writes S^T(t+1) while the vector ALU reads S^T(t), and reads P(t-1) while
+// the vector ALU writes P(t)): the loop body is two sub-tiles.
 // Each block is sixteen steps of one matrix instruction and what runs beside it, fenced so that the compiler keeps
 // them apart.  K and V live in rings of four 64-key LDS tiles each (two sub-tiles per tile, the LDS image of the
-// 256-row kernel), loaded straight into LDS half a tile per iteration, at least two iterations ahead of the first
-// reader; one workgroup barrier per iteration publishes what has landed.
+// 256-row kernel), loaded straight into LDS: an iteration is two sub-tiles and issues one K tile in its first half and
+// one V tile in its second, each a whole iteration and a barrier ahead of its first reader; the one workgroup barrier
+// per iteration publishes what has landed.
 //
 // Softmax as in the 256-row kernel: Q carries the power-of-two part of scale * log2(e), the rest (rr in [1, 2))
 // multiplies the scores in f32; a probability is exp2(fma(s, rr, -m * rr)) against the reference m the row already
@@ -483,15 +487,16 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_rows64_kernel(AttnParams 
         }
         // Iteration T, sub-tiles 2 T and 2 T + 1: P . V of sub-tile 2 T - 1 beside the first half of sub-tile 2 T's
         // softmax, S^T of 2 T + 1 beside the second half; then the same one sub-tile on.  At its top all of this
-        // wavefront's tile loads but the eight of the last iteration have landed and the barrier publishes them: K and V
-        // tiles T + 1 among them, issued two iterations ago.  (No wait for the wavefront's LDS reads at the barrier:
-        // nothing is loaded into a stage they can still be reading before the next barrier.)
+        // wavefront's tile loads but the last four have landed and the barrier publishes them.  The last four are V tile
+        // T + 1's, first read in the next iteration; K tile T + 1, issued in the first half of the last iteration, is
+        // read in the second half of this one and must be among those waited for.  (No wait for the wavefront's LDS
+        // reads at the barrier: nothing is loaded into a stage they can still be reading before the next barrier.)
         const int npairs = (ntiles + 1) >> 1;
         for (int tt = 0; tt < npairs; tt++) {
             const int t = 2 * tt;
             float ts[RB] = {0.0f, 0.0f};
             __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
             block_b(t - 1, c1{}, std::false_type{}, std::true_type{}, ts[0]);
             block_a(t, c0{}, ts[1]);
             settle(t, c0{}, ts);
