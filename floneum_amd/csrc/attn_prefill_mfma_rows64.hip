@@ -72,7 +72,7 @@ struct R64Mma<half_t> {
     // there, and 32 moves per sub-tile follow.  (Nothing reads a score sooner than a block after its last matrix
     // instruction, and the matrix instructions of a chain are two apart: no wait states are owed.)
     static __device__ __forceinline__ void mfma_first_v(float16_t &d, uint4_t a, vec8 b) {
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(d) : "a"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "a"(a), "v"(b));
     }
     static __device__ __forceinline__ void mfma_v(float16_t &d, uint4_t a, vec8 b) {
         asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "a"(a), "v"(b));
@@ -94,7 +94,7 @@ struct R64Mma<bf16_t> {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ void mfma_first_v(float16_t &d, uint4_t a, vec8 b) {
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "a"(a), "v"(b));
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "a"(a), "v"(b));
     }
     static __device__ __forceinline__ void mfma_v(float16_t &d, uint4_t a, vec8 b) {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "a"(a), "v"(b));
