@@ -246,3 +246,62 @@ def test_forced_on_a_call_it_cannot_run(device):
     tq, tk, tv = (fa.Tensor.from_numpy(device, a, fa.F16) for a in (q, k, v))
     with pytest.raises(fa.FhipError):
         tq.flash_attention(tk, tv, 4.0, **FORCE)
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_mixed_feature_sweep(device, seed):
+    """A seeded sweep with the form forced: both 16-bit types, GQA groups, batches, prompt / chunk-on-cache / few-rows
+    shapes and every way of masking the call accepts (a mask that is not made of intervals, or carries finite biases,
+    leaves the call to the kernel queued behind this one).  Rows without a visible key must be NaN on both sides."""
+    rng = np.random.default_rng(seed)
+    gate = {fa.F16: (2e-3, 1e-3), fa.BF16: (2e-2, 8e-3)}
+    for it in range(40):
+        dtype = [fa.F16, fa.BF16][rng.integers(2)]
+        Hkv = int(rng.integers(1, 4))
+        H = Hkv * int(rng.choice([1, 2, 4]))
+        B = int(rng.integers(1, 4))
+        shape = rng.choice(["square", "chunk", "few_rows"])
+        if shape == "square":
+            Sq = Skv = int(rng.integers(1, 700))
+        elif shape == "chunk":
+            Sq, Skv = int(rng.integers(1, 300)), int(rng.integers(300, 1500))
+        else:
+            Sq, Skv = int(rng.integers(1, 70)), int(rng.integers(1000, 3000))
+        q, k, v = qkv(int(rng.integers(1 << 30)), B, H, Hkv, Sq, Skv, D)
+        mk = rng.choice(["none", "analytic", "get_mask", "bias", "batch_key", "kv_lens"])
+        mask = kind = analytic = mt = lens_t = None
+        if mk == "analytic":
+            w = int(rng.integers(1, Skv + 5)) if rng.random() < 0.5 else 0
+            analytic = (True, Skv - Sq, w)
+            mask, kind = analytic_mask(Sq, Skv, True, Skv - Sq, w), "qk"
+        elif mk == "get_mask":
+            w = int(rng.integers(1, 2 * Skv)) if rng.random() < 0.5 else None
+            full = oracle.get_mask(Sq, Skv - Sq, w)
+            if full.shape == (Sq, Skv):
+                mask, kind = full, "qk"
+                mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+        elif mk == "bias":
+            mask, kind = rng.normal(0, 1, (Sq, Skv)).astype(np.float32), "qk"
+            mask[:, rng.integers(1, Skv):] = NEG_INF
+            mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.QKMask)
+        elif mk == "batch_key":
+            mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+            for b in range(B):
+                mask[b, int(rng.integers(1, Skv + 1)):] = NEG_INF if rng.random() < 0.7 else -10000.0
+            mt = (fa.Tensor.from_numpy(device, mask, dtype), fa.MaskKind.BatchKeyMask)
+        elif mk == "kv_lens":
+            lens = rng.integers(1, Skv + 1, B).astype(np.int32)
+            lens_t = fa.IntTensor(device, lens)
+            mask, kind = np.zeros((B, Skv), np.float32), "batch_key"
+            for b in range(B):
+                mask[b, lens[b]:] = NEG_INF
+        what = f"case {it}: dtype {dtype} B {B} H {H} Hkv {Hkv} Sq {Sq} Skv {Skv} {mk} {analytic}"
+        tq, tk, tv = (fa.Tensor.from_numpy(device, a, dtype) for a in (q, k, v))
+        out = tq.flash_attention(tk, tv, D ** -0.5, mt, analytic=analytic, kv_lens=lens_t, out_dtype=fa.F32, **FORCE).to_numpy()
+        ref = oracle.flash_attention(rounded(q, dtype), rounded(k, dtype), rounded(v, dtype), D ** -0.5,
+                                     None if mask is None else rounded(mask, dtype), kind)
+        dead_ref = np.isnan(ref).any(-1)
+        assert np.array_equal(np.isnan(out).any(-1), dead_ref), f"{what}: rows without a visible key differ"
+        live = ~dead_ref
+        if live.any():
+            assert_parity(out[live], ref[live], dict(max_abs=gate[dtype][0], rel_l2=gate[dtype][1]), what)
