@@ -253,9 +253,6 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_rows64_kernel(AttnParams 
     float m[RB], l[RB], nmr[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) m[rb] = -INFINITY, l[rb] = 0.0f, nmr[rb] = INFINITY;
-    float16_t zero16;
-#pragma unroll
-    for (int r = 0; r < 16; r++) zero16[r] = 0.0f;
 
     // LDS operands in flight: the K operand slices of an S^T (the first half read during the block before), V's two
     // contraction slices, read one block apart.  Every operand feeds the matrix instructions of both row blocks.
