@@ -192,6 +192,18 @@ def test_kernel_selection():
     a = make_args(Sq=7, Skv=9, D=33)
     a.force_kernel = fa.KERNEL_PREFILL_MFMA
     assert selected(a)[0] == fa.ERR_UNSUPPORTED
+    # the id that is never chosen: the tiled 16-bit kernel's 64-rows-per-wavefront form, head_dim 128 only, keys never
+    # split over workgroups (no partials in the workspace it asks for)
+    a = make_args(Sq=128, Skv=8192, D=128)
+    need = ctypes.c_size_t()
+    assert fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK and need.value > 0
+    a.force_kernel = fa.KERNEL_PREFILL_MFMA_ROWS64
+    assert selected(a) == (fa.OK, fa.KERNEL_PREFILL_MFMA_ROWS64)
+    assert fa.lib().fhip_flash_attention_workspace_bytes(ctypes.byref(a), 256, ctypes.byref(need)) == fa.OK and need.value == 0
+    for kw in (dict(D=64), dict(D=256), dict(D=128, dtype=fa.F32)):
+        a = make_args(Sq=64, Skv=64, **kw)
+        a.force_kernel = fa.KERNEL_PREFILL_MFMA_ROWS64
+        assert selected(a)[0] == fa.ERR_UNSUPPORTED, kw
 
 
 def test_workspace_bytes():
