@@ -836,7 +836,7 @@ static void plan_decode_call(fhip_device *dev, const fhip_attn_args *args, AttnP
 // the 16-bit tiled prefill kernels: 64 / 96 / 128, and the wide-head form above
 static int launch_mfma_by_head_dim(const AttnParams &p, fhip_dtype dtype, hipStream_t stream) {
     // the form of four wavefronts with 64 rows each (attn_prefill_mfma_rows64.hip), when the caller forces it: measured
-    // 3-6 % slower than the 256-row form of eight wavefronts on the benchmark prompts (fewer LDS reads and a higher clock,
+    // 1-3 % slower than the 256-row form of eight wavefronts on the benchmark prompts (fewer LDS reads and a higher clock,
     // but a lone wavefront per SIMD issues everything in order), so it is never chosen
     if (p.pf_rows64) return launch_prefill_mfma_rows64(p, dtype, stream);
     return (p.D == 64 || p.D == 96 || p.D == 128) ? launch_prefill_mfma(p, dtype, stream) : launch_prefill_mfma_wide(p, dtype, stream);

@@ -24,7 +24,10 @@
 // Softmax as in the 256-row kernel: Q carries the power-of-two part of scale * log2(e), the rest (rr in [1, 2))
 // multiplies the scores in f32; a probability is exp2(fma(s, rr, -m * rr)) against the reference m the row already
 // has, and m moves only when a lane's probabilities of a tile sum to more than 2^15.
-// Masking is by interval (attn_bounds.h): analytic descriptors, key counts, the interval form of a mask tensor.
+// Masking is by interval (attn_bounds.h): analytic descriptors, key counts, the interval form of a mask tensor; the
+// scores of a sub-tile that is not visible to all of the wavefront's rows get their -inf before the softmax reads them.
+// Two branches per sub-tile stay on the path of every sub-tile (must a reference move; does the next sub-tile need its
+// mask): merged into one, or with the next block's addresses formed ahead of them, the kernel measured slower.
 //
 // Reference semantics: fusor-ml/fusor/src/composite/flash_attention.rs:141-199 with the f32 accumulation of 16-bit
 // inputs of fusor-ml/core/src/composite/flash_attention.rs:186-203,323-327.
@@ -390,63 +393,67 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_rows64_kernel(AttnParams 
         }
         softmax_rest(pk[PAR][1], ts1);
     };
-    // After a sub-tile's probabilities have been formed.  Two cases form them again from the scores: a lane's sum is not
-    // at most 2^15 (which also catches the +inf and NaN a row without a reference produces), i.e. some row of the
-    // wavefront needs its reference moved; or the sub-tile is not visible to all of the wavefront's rows (the matrix
-    // instructions' scores stay as they are: the scores outside a row's interval become -inf here; element r is key
-    // j0 + 8 (r / 4) + 4 h2 + r % 4).  Every row's reference moves to at least the tile's maximum, and what the row has
-    // accumulated is rescaled if some row's reference did move.
-    auto settle = [&](int t, auto par_c, float (&ts)[RB]) __attribute__((always_inline)) {
+    // The scores of sub-tile t outside the rows' intervals become -inf before the softmax reads them (element r is key
+    // j0 + 8 (r / 4) + 4 h2 + r % 4); a sub-tile none of the wavefront's rows sees (the workgroup's other wavefronts do)
+    // is all -inf.  Runs right behind the matrix instructions that wrote the scores: those are issued from inline
+    // assembly, so the wait states a vector instruction owes them are written out here.
+    auto mask_scores = [&](int t, auto par_c) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par_c)::value;
         const int j0 = j_begin + t * R64_KEYS;
-        const bool partial = !(j0 >= full_lo_w && j0 + R64_KEYS <= full_hi_w);
-        if (__builtin_expect(j0 >= hi_w || j0 + R64_KEYS <= lo_w, 0)) {
-            // no row of the wavefront sees a key of this sub-tile (the workgroup's other wavefronts do): probabilities of
-            // zero, nothing else changes
+        if (__builtin_expect(!(j0 >= full_lo_w && j0 + R64_KEYS <= full_hi_w), 0)) {
+            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+            if (j0 >= hi_w || j0 + R64_KEYS <= lo_w) {
 #pragma unroll
-            for (int rb = 0; rb < RB; rb++) {
+                for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-                for (int i = 0; i < 8; i++) pk[PAR][rb][i] = 0;
-                ts[rb] = 0.0f;
+                    for (int r = 0; r < 16; r++) sc[PAR][rb][r] = -INFINITY;
+            } else {
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
+                        sc[PAR][rb][r] = (key >= klo[rb] && key < khi[rb]) ? sc[PAR][rb][r] : -INFINITY;
+                    }
             }
-        } else if (__builtin_expect(partial || __builtin_amdgcn_ballot_w64(!(ts[0] <= 32768.0f) || !(ts[1] <= 32768.0f)) != 0, 0)) {
+        }
+    };
+    // After a sub-tile's probabilities have been formed: a lane's sum not at most 2^15 (which also catches the +inf and
+    // NaN a row without a reference produces) means some row of the wavefront needs its reference moved.  Every row's
+    // reference moves to at least the tile's maximum, what the row has accumulated is rescaled if some row's reference
+    // did move, and the tile's probabilities are formed again.
+    auto settle = [&](auto par_c, float (&ts)[RB]) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ts[0] <= 32768.0f) || !(ts[1] <= 32768.0f)) != 0, 0)) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++) {
                 float s[16];
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = j0 + 8 * (r >> 2) + 4 * h2 + (r & 3);
-                    s[r] = (key >= klo[rb] && key < khi[rb]) ? sc[PAR][rb][r] : -INFINITY;
+                for (int r = 0; r < 16; r++) s[r] = sc[PAR][rb][r];
+                float mx = s[0];
+#pragma unroll
+                for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[r]);
+                mx = r64_half_swap_max(mx);
+                const float m_new = fmaxf(m[rb], mx);
+                const float corr = (m[rb] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m[rb] - m_new) * rr);
+                if (__builtin_amdgcn_ballot_w64(m[rb] != -INFINITY && m_new != m[rb]) != 0) {
+                    // (element by element where it lives, in the accumulation half of the register file: written as
+                    // arithmetic the compiler copies all of O^T out ahead of the branch, on the path of every sub-tile)
+#pragma unroll
+                    for (int db = 0; db < DB; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            float tmp;
+                            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                                         : "+a"(o[rb][db][r]), "=&v"(tmp)
+                                         : "v"(corr));
+                        }
+                    asm volatile("s_nop 7" ::: "memory");  // before a matrix instruction takes them as its C operand
                 }
-                // against the reference the row has; it moves only if these cannot be used
-                float t2 = probabilities(s, pk[PAR][rb], nmr[rb]);
-                if (__builtin_amdgcn_ballot_w64(!(t2 <= 32768.0f)) != 0) {
-                    float mx = s[0];
-#pragma unroll
-                    for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[r]);
-                    mx = r64_half_swap_max(mx);
-                    const float m_new = fmaxf(m[rb], mx);
-                    const float corr = (m[rb] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m[rb] - m_new) * rr);
-                    if (__builtin_amdgcn_ballot_w64(m[rb] != -INFINITY && m_new != m[rb]) != 0) {
-                        // (element by element where it lives, in the accumulation half of the register file: written as
-                        // arithmetic the compiler copies all of O^T out ahead of the branch, on the path of every sub-tile)
-#pragma unroll
-                        for (int db = 0; db < DB; db++)
-#pragma unroll
-                            for (int r = 0; r < 16; r++) {
-                                float tmp;
-                                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
-                                             : "+a"(o[rb][db][r]), "=&v"(tmp)
-                                             : "v"(corr));
-                            }
-                        asm volatile("s_nop 7" ::: "memory");  // before a matrix instruction takes them as its C operand
-                    }
-                    m[rb] = m_new;
-                    l[rb] *= corr;
-                    nmr[rb] = (m[rb] == -INFINITY) ? INFINITY : -m[rb] * rr;
-                    t2 = probabilities(s, pk[PAR][rb], (m[rb] == -INFINITY) ? 0.0f : nmr[rb]);
-                }
-                ts[rb] = t2;
+                m[rb] = m_new;
+                l[rb] *= corr;
+                nmr[rb] = (m[rb] == -INFINITY) ? INFINITY : -m[rb] * rr;
+                ts[rb] = probabilities(s, pk[PAR][rb], (m[rb] == -INFINITY) ? 0.0f : nmr[rb]);
             }
         }
 #pragma unroll
@@ -482,6 +489,7 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_rows64_kernel(AttnParams 
                     if (kb == 0) R64Mma<T>::mfma_first_v(sc[0][rb], ka[kb], qreg[rb][kb]);
                     else R64Mma<T>::mfma_v(sc[0][rb], ka[kb], qreg[rb][kb]);
         }
+        mask_scores(0, c0{});
         // Iteration T, sub-tiles 2 T and 2 T + 1: P . V of sub-tile 2 T - 1 beside the first half of sub-tile 2 T's
         // softmax, S^T of 2 T + 1 beside the second half; then the same one sub-tile on.  At its top all of this
         // wavefront's tile loads but the last four have landed and the barrier publishes them.  The last four are V tile
@@ -496,11 +504,13 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_rows64_kernel(AttnParams 
             asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
             block_b(t - 1, c1{}, std::false_type{}, std::true_type{}, ts[0]);
             block_a(t, c0{}, ts[1]);
-            settle(t, c0{}, ts);
+            settle(c0{}, ts);
+            mask_scores(t + 1, c1{});
             ts[0] = ts[1] = 0.0f;
             block_b(t, c0{}, std::true_type{}, std::true_type{}, ts[0]);
             block_a(t + 1, c1{}, ts[1]);
-            settle(t + 1, c1{}, ts);
+            settle(c1{}, ts);
+            mask_scores(t + 2, c0{});
         }
         __builtin_amdgcn_sched_barrier(0);
         float unused = 0.0f;

@@ -161,7 +161,7 @@ typedef enum {
     FHIP_KERNEL_PREFILL_MFMA_ROWS64 = 5 /* only as force_kernel, never chosen: FHIP_KERNEL_PREFILL_MFMA's calls at
                                       head_dim 128 on its other form, four wavefronts of 64 query rows per workgroup
                                       (one per SIMD, half the LDS operand reads per matrix instruction, keys never split
-                                      over workgroups).  Same results; 3-6 % slower than the 256-row form of eight
+                                      over workgroups).  Same results; 1-3 % slower than the 256-row form of eight
                                       wavefronts on this chip, whose matrix kernels are bound by power.  Kept selectable
                                       for measurement (bench.py --config C3R)                                  */
 } fhip_kernel_id;
